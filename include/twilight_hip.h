@@ -1,0 +1,235 @@
+/*
+ * twilight_hip.h — C ABI of libtwilight_hip.so: the Select-then-Prune decode hot path of
+ * Twilight (Quest page selector -> INT4-K score GEMV -> softmax + top-p prune -> sparse paged
+ * decode attention) as hand-written HIP kernels for gfx950 (MI355X).
+ *
+ * Conventions shared by every entry point
+ *   - All pointers are DEVICE pointers unless the name ends in _host. The library never
+ *     allocates, frees or synchronises: outputs and workspaces are caller-owned, kernels are
+ *     enqueued on `stream` (a hipStream_t passed as void*; NULL = the default stream).
+ *   - Return value: TWL_OK (0) or a negative TWL_E* code; twl_strerror() names it. Arguments are
+ *     validated on the host before anything touches the GPU, so TWL_EINVAL/TWL_ENULL/... are
+ *     returned even on a machine without a GPU.
+ *   - rows = batch * num_q_heads, row r = b * num_q_heads + h. KV head of q head h is
+ *     h / (num_q_heads / num_kv_heads). head_dim is 128, page size is 16 tokens (TWL_PAGE).
+ *   - Page tables are FlashInfer-style CSR: request b owns logical pages
+ *     kv_page_indices[kv_page_indptr[b] .. kv_page_indptr[b+1]) (values = physical page ids);
+ *     its last logical page holds kv_last_page_len[b] (1..16) valid tokens.
+ *   - A "page list" is per row: sel_pages[r * sel_stride + i], i < sel_count[r], holds LOGICAL
+ *     page numbers of request b in ascending order. Candidate c of a row is token (c % 16) of
+ *     its (c / 16)-th listed page. sel_pages == NULL means "all pages of the request".
+ *   - A "survivor list" is per row: idx[r * idx_stride + j], j < count[r], holds LOGICAL token
+ *     positions (page * 16 + slot) in ascending order.
+ *
+ * Storage formats defined by this library (nothing in the reference pins them)
+ *   - INT4 K shadow: one 1280-byte record per (physical page, kv head), records ordered
+ *     [page][kv_head]. Bytes [0,1024): token t (0..15) occupies bytes [64t, 64t+64); element d
+ *     (0..127) of that token is the low (d even) or high (d odd) nibble of byte d/2. Bytes
+ *     [1024,1280): 64 pairs of IEEE fp16 (scale, zero), pair index t*4 + g for quantisation group
+ *     g = d/32. Dequantised value = float(nibble) * float(scale) + float(zero), one fp32 rounding.
+ *   - Quest page metadata: one 512-byte record per (physical page, kv head), ordered
+ *     [page][kv_head]: 32 chunks of 16 bytes; chunk c holds fp16 min[4c..4c+3] then fp16
+ *     max[4c..4c+3] over the valid tokens of the page.
+ *   - Paged K / V caches: fp16 or bf16, addressed with explicit element strides
+ *     (page, token, kv head); head_dim is contiguous.
+ */
+#ifndef TWILIGHT_HIP_H_
+#define TWILIGHT_HIP_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TWL_PAGE 16          /* tokens per KV page */
+#define TWL_HEAD_DIM 128     /* head dimension */
+#define TWL_QGROUP 32        /* INT4 quantisation group along head_dim */
+#define TWL_INT4_RECORD_BYTES 1280
+#define TWL_META_RECORD_BYTES 512
+#define TWL_MAX_CANDIDATES 32768 /* longest row twl_top_p_* / twl_softmax_top_p_f32 accept */
+
+enum twl_status {
+  TWL_OK = 0,
+  TWL_ENULL = -1,    /* a required pointer is NULL */
+  TWL_EINVAL = -2,   /* a size / stride / mode argument is out of range */
+  TWL_EDTYPE = -3,   /* unsupported element type code */
+  TWL_EALIGN = -4,   /* a pointer or stride breaks the alignment the kernel needs */
+  TWL_ELAUNCH = -5,  /* the HIP runtime rejected the launch (hipGetLastError != hipSuccess) */
+  TWL_ENODEVICE = -6 /* no usable HIP device */
+};
+
+enum twl_dtype { TWL_F16 = 0, TWL_BF16 = 1, TWL_F32 = 2 };
+
+/* how the top-p bisection initialises its upper bound */
+enum twl_top_p_high {
+  TWL_HIGH_FIRST = 0, /* probs[row][0], as csrc/include/sampling.cuh:156-159 does */
+  TWL_HIGH_MAX = 1    /* the row maximum (paper Algorithm 1) */
+};
+
+const char* twl_strerror(int status);
+/* ABI version of this header; bumps when a signature changes. */
+int twl_abi_version(void);
+/* Number of HIP devices visible, or a negative twl_status. */
+int twl_device_count(void);
+
+/* ---------------------------------------------------------------------------------------------
+ * Top-p pruner on normalised probabilities.
+ * Replaces: top_p_fp32_return_mask / top_p_fp16_return_mask, csrc/src/sampling.cu:22-63, and the
+ * kernel they launch, TopPReturnMaskKernel, csrc/include/sampling.cuh:119-231 (launcher :233-250).
+ * probs is [rows, d] contiguous (the reference's [B,H,1,N] tensor with rows = B*H, d = N).
+ * p_arr (nullable) holds one p per row and overrides p, as top_p_arr does (sampling.cuh:125).
+ * Outputs, each nullable (at least one must be given):
+ *   mask  uint8 [rows, d]: 1 where probs > low at the end of the bisection (sampling.cuh:219-230)
+ *   idx   int32 [rows, idx_stride] + count int32 [rows]: the positions where mask is 1, ascending.
+ * low_out (nullable) float [rows]: the final lower pivot; iters_out (nullable) int32 [rows]: the
+ * number of bisection iterations executed.
+ * d must be in [1, TWL_MAX_CANDIDATES]; idx_stride >= d when idx is given.
+ * ------------------------------------------------------------------------------------------- */
+int twl_top_p_f32(const float* probs, uint8_t* mask, int32_t* idx, int32_t* count,
+                  const float* p_arr, float p, uint32_t rows, uint32_t d, uint32_t idx_stride,
+                  int high_mode, float* low_out, int32_t* iters_out, void* stream);
+/* Same for fp16 (dtype = TWL_F16) or bf16 (TWL_BF16) probabilities; the bisection runs in that
+ * type's value set (pivots are rounded to it each iteration) like the reference's DType template
+ * (sampling.cuh:156-217 with DType = half / nv_bfloat16). */
+int twl_top_p_f16(const void* probs, int dtype, uint8_t* mask, int32_t* idx, int32_t* count,
+                  const float* p_arr, float p, uint32_t rows, uint32_t d, uint32_t idx_stride,
+                  int high_mode, float* low_out, int32_t* iters_out, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Fused softmax + top-p + stream compaction over raw (un-normalised) scores.
+ * Replaces: top_p_unnormalized, twilight/pyimpl/top_p.py:10-15 (softmax in fp32 then the mask
+ * kernel) and the mask combine twilight/pyimpl/attention.py:280-281 in index-list form.
+ * scores is [rows, score_stride] fp32; row r has lens[r] candidates (lens == NULL: every row has
+ * d). -inf scores are legal and get probability 0. Survivors are emitted as
+ *   idx[r*idx_stride + j] = token_of(position) ascending, count[r],
+ * where token_of(c) = sel_pages[r*sel_stride + c/16]*16 + c%16 when sel_pages != NULL, else c.
+ * probs_out (nullable) float [rows, score_stride] receives the softmax for inspection.
+ * ------------------------------------------------------------------------------------------- */
+int twl_softmax_top_p_f32(const float* scores, uint32_t score_stride, const int32_t* lens,
+                          uint32_t rows, uint32_t d, const float* p_arr, float p, int high_mode,
+                          const int32_t* sel_pages, uint32_t sel_stride, int32_t* idx,
+                          uint32_t idx_stride, int32_t* count, float* probs_out, float* low_out,
+                          void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * INT4-K score GEMV over candidate pages: out[r, c] = sm_scale * sum_d q[r,d] * dequant(K[c,d]).
+ * Replaces: the estimator matmul twilight/pyimpl/attention.py:252-255 and the absent
+ * ftka.cuda_ops.gemv.batched_sparse_gemv_int4_k whose call site is
+ * benchmark/efficiency/bench_gemv.py:445-454.
+ * q [batch, num_q_heads, 128] in q_dtype (TWL_F16 or TWL_BF16); k_int4 = the INT4 shadow records.
+ * out fp32 [rows, out_stride]; candidates past the request's length get -inf. sel_count (nullable
+ * with sel_pages) gives pages per row; out_count (nullable) int32 [rows] receives the number of
+ * candidate slots written (pages * 16).
+ * ------------------------------------------------------------------------------------------- */
+int twl_gemv_int4(const void* q, int q_dtype, float* out, uint32_t out_stride, int32_t* out_count,
+                  const void* k_int4, const int32_t* sel_pages, const int32_t* sel_count,
+                  uint32_t sel_stride, const int32_t* kv_page_indices,
+                  const int32_t* kv_page_indptr, const int32_t* kv_last_page_len, uint32_t batch,
+                  uint32_t num_q_heads, uint32_t num_kv_heads, uint32_t max_pages_per_row,
+                  float sm_scale, void* stream);
+
+/* Same GEMV in the tensor layout of benchmark/efficiency/bench_gemv.py:390-454: k_u8
+ * [max_pages, page_size, num_heads, 64] uint8 (low nibble = even element), scales / zeros fp16
+ * [max_pages, page_size, num_heads] (one group per token), q fp16 [batch, num_heads, 128], o fp16
+ * [batch, num_heads, o_stride] written in place for n < request length; one page list per request
+ * shared by all heads. */
+int twl_gemv_int4_nhd(const void* q, void* o, uint32_t o_stride, const uint8_t* k_u8,
+                      const void* scales, const void* zeros, const int32_t* kv_page_indices,
+                      const int32_t* kv_page_indptr, const int32_t* kv_last_page_len,
+                      uint32_t batch, uint32_t num_heads, uint32_t page_size,
+                      uint32_t max_pages_per_req, float sm_scale, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Sparse paged decode attention over survivor lists.
+ * Replaces: the masked softmax.V of twilight/pyimpl/attention.py:188-190,299-306 restricted to
+ * the surviving tokens. logits = sm_scale * q.K (fp32), softmax in fp32, probabilities rounded to
+ * the q dtype before the V product (attention.py:302-304), fp32 accumulation, output in the q
+ * dtype [batch, num_q_heads, 128]. Rows with count 0 produce zeros. lse_out (nullable) float
+ * [rows] receives log(sum exp(logit)) of the row.
+ * k_cache / v_cache: element type kv_dtype (TWL_F16 / TWL_BF16, must equal q's type); element
+ * (page, token, kv_head, d) lives at page*page_stride + token*token_stride + kv_head*head_stride + d.
+ * ------------------------------------------------------------------------------------------- */
+int twl_sparse_attn(const void* q, void* out, int dtype, const void* k_cache, const void* v_cache,
+                    uint64_t page_stride, uint64_t token_stride, uint64_t head_stride,
+                    const int32_t* idx, uint32_t idx_stride, const int32_t* count,
+                    const int32_t* kv_page_indices, const int32_t* kv_page_indptr, uint32_t batch,
+                    uint32_t num_q_heads, uint32_t num_kv_heads, float sm_scale, float* lse_out,
+                    void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Quest page selector: page score + top-k pages per row.
+ * Replaces: quest_selector, twilight/pyimpl/quest.py:17-122, in its page-metadata form:
+ * score(page) = sum_d max(q_d * max_d, q_d * min_d) (== (q*sign) . amax(K*sign), quest.py:37-84),
+ * k = min(pages of the request, max(1, budget/16) + (budget%16 != 0)) (quest.py:93-98), top-k by
+ * score with ties resolved toward the lower page number. Output: sel_pages [rows, sel_stride]
+ * ascending logical page numbers, sel_count [rows]. page_scores (nullable) float
+ * [rows, score_stride] receives the raw page scores.
+ * ------------------------------------------------------------------------------------------- */
+int twl_quest_select(const void* q, int q_dtype, const void* meta, const int32_t* kv_page_indices,
+                     const int32_t* kv_page_indptr, uint32_t batch, uint32_t num_q_heads,
+                     uint32_t num_kv_heads, uint32_t token_budget, uint32_t max_pages_per_req,
+                     int32_t* sel_pages, uint32_t sel_stride, int32_t* sel_count,
+                     float* page_scores, uint32_t score_stride, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * KV-append side: build the INT4 shadow and the Quest metadata of whole pages from the paged K.
+ * Replaces: min_max_per_token_quant_kv, twilight/pyimpl/quantize.py:4-13 (applied per group of 32
+ * with fp16 scale / zero storage) and the per-chunk amax of twilight/pyimpl/quest.py:68-74.
+ * Processes physical pages page_ids[0..num_pages) (page_ids == NULL: pages 0..num_pages-1);
+ * valid_len (nullable) int32 [num_pages] gives the valid tokens of each page (default 16): the
+ * metadata covers only valid tokens, nibbles of invalid tokens are written as 0 with scale 0.
+ * k_int4 and/or meta may be NULL to skip that output.
+ * ------------------------------------------------------------------------------------------- */
+int twl_kv_shadow_build(const void* k_cache, int kv_dtype, uint64_t page_stride,
+                        uint64_t token_stride, uint64_t head_stride, const int32_t* page_ids,
+                        const int32_t* valid_len, uint32_t num_pages, uint32_t num_kv_heads,
+                        void* k_int4, void* meta, void* stream);
+
+/* Unpack INT4 shadow records to fp32: out [num_pages, num_kv_heads, 16, 128] (record order).
+ * Exists so that tests can compare dequantised values bit for bit. */
+int twl_dequant_int4(const void* k_int4, uint32_t num_records, float* out, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * The whole decode layer on one stream: quest select -> INT4 GEMV -> softmax + top-p -> sparse
+ * attention (twilight/pyimpl/attention.py:188-306 for q_len == 1). Every intermediate is a
+ * caller-provided buffer (see the field comments); no host synchronisation happens inside.
+ * ------------------------------------------------------------------------------------------- */
+typedef struct twl_layer_args {
+  /* inputs */
+  const void* q;            /* [batch, num_q_heads, 128], dtype */
+  int dtype;                /* TWL_F16 or TWL_BF16: type of q, K, V and out */
+  const void* k_cache;      /* paged K */
+  const void* v_cache;      /* paged V */
+  uint64_t page_stride, token_stride, head_stride; /* element strides of both caches */
+  const void* k_int4;       /* INT4 shadow records */
+  const void* meta;         /* Quest metadata records */
+  const int32_t* kv_page_indices;
+  const int32_t* kv_page_indptr;
+  const int32_t* kv_last_page_len;
+  uint32_t batch, num_q_heads, num_kv_heads;
+  uint32_t max_pages_per_req; /* >= the longest request's page count */
+  uint32_t token_budget;      /* Quest budget in tokens (selector: token_budget) */
+  float top_p;                /* pruner threshold */
+  int high_mode;              /* twl_top_p_high */
+  float sm_scale;             /* 1/sqrt(128) in the reference */
+  /* workspaces / intermediate outputs, all caller-owned */
+  int32_t* sel_pages;  uint32_t sel_stride;  /* [rows, sel_stride], sel_stride >= selected pages */
+  int32_t* sel_count;                        /* [rows] */
+  float* page_scores;  uint32_t page_score_stride; /* [rows, >= max_pages_per_req]; NULL: the
+                                                      head of `scores` is used as staging and
+                                                      score_stride must be >= max_pages_per_req */
+  float* scores;       uint32_t score_stride;/* [rows, score_stride], >= 16 * selected pages */
+  int32_t* cand_count;                       /* [rows] */
+  int32_t* idx;        uint32_t idx_stride;  /* [rows, idx_stride], >= 16 * selected pages */
+  int32_t* count;                            /* [rows] */
+  /* output */
+  void* out;                /* [batch, num_q_heads, 128], dtype */
+} twl_layer_args;
+
+int twl_decode_layer(const twl_layer_args* args, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TWILIGHT_HIP_H_ */

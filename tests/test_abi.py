@@ -1,0 +1,128 @@
+"""CPU-only checks of the C-ABI boundary: the library loads, exports every symbol the header
+declares, and validates arguments on the host (no GPU is touched by any call here)."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from twilight_amd import _lib
+import twilight_amd.kernel as K
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_header_symbols_are_exported(hip_lib):
+    hdr = open(os.path.join(ROOT, "include", "twilight_hip.h")).read()
+    declared = set(re.findall(r"\b(twl_[a-z0-9_]+)\s*\(", hdr))
+    declared -= {"twl_top_p_"}  # no partial names
+    assert declared == set(_lib.EXPORTS)
+    for name in declared:
+        assert hasattr(hip_lib, name), name
+    assert hip_lib.twl_abi_version() == 1
+
+
+def test_header_compiles_as_c():
+    import subprocess, tempfile
+    with tempfile.TemporaryDirectory() as d:
+        src = os.path.join(d, "t.c")
+        open(src, "w").write('#include "twilight_hip.h"\nint main(void){return sizeof(twl_layer_args)>0?0:1;}\n')
+        subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-I", os.path.join(ROOT, "include"),
+                        "-c", src, "-o", os.path.join(d, "t.o")], check=True)
+
+
+def test_layer_struct_matches_header(hip_lib):
+    import subprocess, tempfile
+    with tempfile.TemporaryDirectory() as d:
+        src = os.path.join(d, "t.c")
+        open(src, "w").write('#include <stdio.h>\n#include <stddef.h>\n#include "twilight_hip.h"\n'
+                             'int main(void){printf("%zu %zu %zu %zu", sizeof(twl_layer_args),'
+                             'offsetof(twl_layer_args, sm_scale), offsetof(twl_layer_args, scores),'
+                             'offsetof(twl_layer_args, out));return 0;}\n')
+        exe = os.path.join(d, "t")
+        subprocess.run(["gcc", "-I", os.path.join(ROOT, "include"), src, "-o", exe], check=True)
+        sizes = [int(x) for x in subprocess.run([exe], capture_output=True, text=True).stdout.split()]
+    A = _lib.LayerArgs
+    assert sizes == [ctypes.sizeof(A), A.sm_scale.offset, A.scores.offset, A.out.offset]
+
+
+def test_strerror(hip_lib):
+    assert _lib.strerror(0) == "ok"
+    for rc in range(-6, 0):
+        assert _lib.strerror(rc) and "unknown" not in _lib.strerror(rc)
+    assert "unknown" in _lib.strerror(-99)
+
+
+def test_c_level_validation_without_gpu(hip_lib):
+    L = hip_lib
+    fake = 0x1000  # never dereferenced: validation fails first
+    assert L.twl_top_p_f32(0, fake, 0, 0, 0, 0.9, 1, 8, 8, 0, 0, 0, 0) == -1          # probs NULL
+    assert L.twl_top_p_f32(fake, 0, 0, 0, 0, 0.9, 1, 8, 8, 0, 0, 0, 0) == -1          # no output
+    assert L.twl_top_p_f32(fake, 0, fake, 0, 0, 0.9, 1, 8, 8, 0, 0, 0, 0) == -1       # idx without count
+    assert L.twl_top_p_f32(fake, fake, 0, 0, 0, 0.9, 1, 0, 8, 0, 0, 0, 0) == -2       # d == 0
+    assert L.twl_top_p_f32(fake, fake, 0, 0, 0, 0.9, 1, 40000, 8, 0, 0, 0, 0) == -2   # d too large
+    assert L.twl_top_p_f32(fake, fake, 0, 0, 0, 0.0, 1, 8, 8, 0, 0, 0, 0) == -2       # p out of (0,1]
+    assert L.twl_top_p_f32(fake, fake, 0, 0, 0, 1.5, 1, 8, 8, 0, 0, 0, 0) == -2
+    assert L.twl_top_p_f32(fake, fake, 0, 0, 0, 0.9, 1, 8, 8, 7, 0, 0, 0) == -2       # bad high_mode
+    assert L.twl_top_p_f32(fake, 0, fake, fake, 0, 0.9, 1, 8, 4, 0, 0, 0, 0) == -2    # idx_stride < d
+    assert L.twl_top_p_f32(fake + 2, fake, 0, 0, 0, 0.9, 1, 8, 8, 0, 0, 0, 0) == -4   # misaligned
+    assert L.twl_top_p_f16(fake, 2, fake, 0, 0, 0, 0.9, 1, 8, 8, 0, 0, 0, 0) == -3    # dtype
+    assert L.twl_gemv_int4(fake, 0, 0, 16, 0, fake, 0, 0, 0, fake, fake, fake, 1, 1, 1, 1, 1.0, 0) == -1
+    assert L.twl_gemv_int4(fake, 2, fake, 16, 0, fake, 0, 0, 0, fake, fake, fake, 1, 1, 1, 1, 1.0, 0) == -3
+    assert L.twl_gemv_int4(fake, 0, fake, 16, 0, fake, 0, 0, 0, fake, fake, fake, 1, 3, 2, 1, 1.0, 0) == -2
+    assert L.twl_gemv_int4(fake, 0, fake, 8, 0, fake, 0, 0, 0, fake, fake, fake, 1, 1, 1, 1, 1.0, 0) == -2
+    assert L.twl_gemv_int4(fake + 4, 0, fake, 16, 0, fake, 0, 0, 0, fake, fake, fake, 1, 1, 1, 1, 1.0, 0) == -4
+    assert L.twl_sparse_attn(fake, fake, 0, fake, fake, 4096, 256, 128, 0, 8, fake, fake, fake,
+                             1, 1, 1, 1.0, 0, 0) == -1
+    assert L.twl_sparse_attn(fake, fake, 0, fake, fake, 4096, 256, 130, fake, 8, fake, fake, fake,
+                             1, 1, 1, 1.0, 0, 0) == -4
+    assert L.twl_sparse_attn(fake, fake, 0, fake, fake, 4096, 256, 128, fake, 0, fake, fake, fake,
+                             1, 1, 1, 1.0, 0, 0) == -2
+    assert L.twl_quest_select(fake, 0, fake, fake, fake, 1, 1, 1, 0, 4, fake, 4, fake, fake, 4, 0) == -2
+    assert L.twl_quest_select(fake, 0, fake, fake, fake, 1, 1, 1, 64, 4, fake, 2, fake, fake, 4, 0) == -2
+    assert L.twl_kv_shadow_build(fake, 0, 4096, 256, 128, 0, 0, 1, 1, 0, 0, 0) == -1
+    assert L.twl_dequant_int4(fake, 0, fake, 0) == -2
+    assert L.twl_decode_layer(None, 0) == -1
+
+
+def test_python_ops_reject_cpu_and_malformed_tensors(hip_lib):
+    # same conditions as CHECK_INPUT / CHECK_DIM (csrc/src/sampling.cu:25-27): RuntimeError
+    p = torch.rand(2, 3, 1, 64)
+    with pytest.raises(RuntimeError, match="CUDA"):
+        K.top_p_fp32_return_mask(p, 0.9)
+    with pytest.raises(RuntimeError, match="CUDA"):
+        K.top_p_fp16_return_mask(p.half(), 0.9)
+    with pytest.raises(RuntimeError):
+        K.top_p_fp32_return_mask("nope", 0.9)
+    with pytest.raises(RuntimeError, match="CUDA"):
+        K.sparse_gemv_int4(torch.zeros(1, 1, 128).half(), torch.zeros(1, 1, 1280, dtype=torch.uint8),
+                           torch.zeros(1, dtype=torch.int32), torch.zeros(2, dtype=torch.int32),
+                           torch.ones(1, dtype=torch.int32), max_pages=1)
+    with pytest.raises(RuntimeError, match="CUDA"):
+        K.softmax_top_p(torch.zeros(1, 1, 16), 0.9)
+    with pytest.raises(RuntimeError, match="CUDA"):
+        K.quest_select(torch.zeros(1, 1, 128).half(), torch.zeros(1, 1, 512, dtype=torch.uint8),
+                       torch.zeros(1, dtype=torch.int32), torch.zeros(2, dtype=torch.int32), 16, 1)
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "nope.so"))
+    with pytest.raises(RuntimeError, match="no CPU or PyTorch fallback"):
+        _lib.lib()
+
+
+def test_sparse_config_parsing():
+    from twilight_amd.layer import parse_sparse_config
+    cfg = {"compressor": {"type": "none"},
+           "selector": {"type": "quest", "token_budget": 8192, "chunk_size": 16},
+           "weight_estimator": {"type": "min_max_quant", "quant_bit": 4},
+           "weight_pruner": {"type": "top_p", "threshold": 0.85},
+           "skip_first_two_layers": True, "use_estimated_weights_in_attn": False}
+    assert parse_sparse_config(cfg) == {"token_budget": 8192, "top_p": 0.85}
+    bad = dict(cfg, selector={"type": "ds"})
+    with pytest.raises(RuntimeError):
+        parse_sparse_config(bad)
+    with pytest.raises(RuntimeError):
+        parse_sparse_config(dict(cfg, weight_estimator={"type": "min_max_quant", "quant_bit": 2}))

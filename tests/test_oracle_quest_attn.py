@@ -1,0 +1,121 @@
+"""Pins the oracle's Quest selector (twilight/pyimpl/quest.py:17-122), estimator GEMV and masked
+attention (twilight/pyimpl/attention.py:188-306) against brute force / library routines."""
+import math
+
+import numpy as np
+import torch
+
+from oracle import native
+from oracle import pyimpl_port as P
+
+
+def test_quest_dense_vs_brute_force_with_padding():
+    g = torch.Generator().manual_seed(0)
+    B, H, N, D, C = 1, 2, 40, 128, 16        # 40 = 2.5 chunks: exercises quest.py:48-65
+    q = torch.randn((B, H, 1, D), generator=g)
+    k = torch.randn((B, H, N, D), generator=g)
+    est = P.quest_chunk_scores_dense(q, k, C)
+    assert est.shape == (B, H, 1, 3)
+    for h in range(H):
+        for c in range(3):
+            toks = range(c * C, min(N, (c + 1) * C))
+            s = 0.0
+            for d in range(D):
+                qd = float(q[0, h, 0, d])
+                s += max(qd * float(k[0, h, t, d]) for t in toks)
+            assert abs(s - float(est[0, h, 0, c])) < 1e-3
+    mask, topk = P.quest_selector_dense(q, k, C, token_budget=20)   # 20 -> 1 + 1 chunks
+    assert topk.shape[-1] == 2
+    for h in range(H):
+        best = torch.argsort(est[0, h, 0], descending=True)[:2].tolist()
+        want = torch.zeros(N, dtype=torch.bool)
+        for c in best:
+            want[c * C:min(N, (c + 1) * C)] = True
+        assert torch.equal(mask[0, h, 0], want)
+
+
+def test_quest_budget_rule():
+    # quest.py:93-98
+    assert P.quest_chunk_budget(8192, 16, 2048) == 512
+    assert P.quest_chunk_budget(8200, 16, 2048) == 513
+    assert P.quest_chunk_budget(5, 16, 2048) == 2      # max(1, 0) + 1 for the remainder
+    assert P.quest_chunk_budget(16, 16, 2048) == 1
+    assert P.quest_chunk_budget(8192, 16, 100) == 100
+
+
+def test_quest_meta_form_equals_dense_form():
+    g = torch.Generator().manual_seed(1)
+    B, Hkv, N, D = 2, 2, 72, 128                 # last page holds 8 valid tokens
+    q = torch.randn((B, Hkv, 1, D), generator=g).half().float()
+    q[0, 0, 0, 5] = 0.0                            # quest.py:37: sign(0) = -1, contributes 0
+    k = torch.randn((B, Hkv, N, D), generator=g).half().float()
+    dense = P.quest_chunk_scores_dense(q, k, 16)
+    pages, ids, indptr, last = P.dense_to_paged(k, torch.randperm(B * 5, generator=g))
+    valid = torch.full((B * 5,), 16, dtype=torch.int64)
+    for b in range(B):
+        valid[ids[indptr[b + 1] - 1].long()] = int(last[b])
+    meta = P.quest_page_meta(pages, valid)
+    rec = P.pack_meta_records(meta)
+    assert rec.shape == (B * 5, Hkv, 512)
+    # record layout: chunk c = fp16 min[4c..4c+3] then max[4c..4c+3]
+    r = rec[3, 1].view(np.float16).reshape(32, 2, 4)
+    assert np.array_equal(r[:, 0].reshape(-1), meta[3, 1, 0].numpy().astype(np.float16))
+    assert np.array_equal(r[:, 1].reshape(-1), meta[3, 1, 1].numpy().astype(np.float16))
+    for b in range(B):
+        for h in range(Hkv):
+            phys = ids[indptr[b]:indptr[b + 1]].long()
+            s = P.quest_page_scores_meta(q[b, h, 0], meta[phys, h])
+            assert torch.allclose(s.float(), dense[b, h, 0], rtol=1e-5, atol=1e-4)
+
+
+def test_estimator_scores_is_a_matmul():
+    g = torch.Generator().manual_seed(2)
+    q = torch.randn((1, 4, 1, 128), generator=g).half().float()
+    k = torch.randn((1, 4, 96, 128), generator=g).half().float()
+    _, _, _, deq = P.int4_quant_storage(k)
+    s = P.estimator_scores(q, torch.from_numpy(deq))
+    ref = np.einsum("bhqd,bhnd->bhqn", q.double().numpy(), deq.astype(np.float64)) / math.sqrt(128)
+    np.testing.assert_allclose(s.numpy(), ref, rtol=1e-5, atol=1e-5)
+    # the constant-input case of benchmark/efficiency/bench_gemv.py:390-422: q = 1, nibble 3,
+    # scale 1, zero 0 -> every raw score is 3 * 128
+    ones = torch.ones((1, 1, 1, 128))
+    deq3 = native.int4_dequant(np.full((1, 128), 3, np.uint8), np.ones((1, 4), np.float16),
+                               np.zeros((1, 4), np.float16))
+    assert float(P.estimator_scores(ones, torch.from_numpy(deq3)[None, None], sm_scale=1.0)) == 384.0
+
+
+def test_masked_attention_equals_gathered_softmax():
+    g = torch.Generator().manual_seed(3)
+    B, H, N, D = 2, 3, 200, 128
+    q = torch.randn((B, H, 1, D), generator=g).half().float()
+    k = torch.randn((B, H, N, D), generator=g).half().float()
+    v = torch.randn((B, H, N, D), generator=g).half().float()
+    mask = torch.rand((B, H, 1, N), generator=g) < 0.1
+    mask[..., 0] = True
+    for dt in (torch.float32, torch.float16):
+        out = P.masked_attention(q, k, v, mask, dt)
+        for b in range(B):
+            for h in range(H):
+                sel = mask[b, h, 0].nonzero().squeeze(-1)
+                logit = (k[b, h, sel].double() @ q[b, h, 0].double()) / math.sqrt(D)
+                pr = torch.softmax(logit, -1)
+                if dt == torch.float16:
+                    pr = pr.float().half().double()
+                ref = pr @ v[b, h, sel].double()
+                assert torch.allclose(out[b, h, 0].double(), ref, rtol=1e-4, atol=1e-5)
+    idx, count = P.mask_to_lists(mask)
+    assert count.sum() == int(mask.sum()) and idx[0, 0] == 0
+
+
+def test_decode_layer_dense_consistency():
+    from twilight_amd import synth
+    q, k, v = synth.heavy_hitter_qkv(1, 2, 512, n_heavy=8, mass=0.6, seed=0)
+    r = P.decode_layer_dense(q, k, v, top_p=0.95, token_budget=256)
+    assert r["mask0"].sum(-1).unique().tolist() == [256]
+    assert torch.all(r["mask"] <= r["mask0"])
+    kept = (r["probs"] * r["mask"]).sum(-1)
+    assert torch.all(kept >= 0.95 - 1e-6)
+    # heavy hitters carry ~0.6 of the exact softmax by construction
+    w = torch.softmax((q @ k.transpose(2, 3)) / math.sqrt(128), -1)
+    top8 = w.topk(8, dim=-1).values.sum(-1)
+    assert torch.all((top8 > 0.55) & (top8 < 0.66))

@@ -1,0 +1,99 @@
+"""ctypes binding of ``libtwilight_hip.so`` (declared in ``include/twilight_hip.h``).
+
+There is no fallback: if the library is missing, :func:`lib` raises, and every op of
+``twilight_amd.kernel`` fails with it.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import POINTER, c_char_p, c_float, c_int, c_int32, c_uint8, c_uint32, c_uint64, c_void_p
+
+from .build import LIB_PATH
+
+TWL_OK = 0
+TWL_F16, TWL_BF16, TWL_F32 = 0, 1, 2
+TWL_HIGH_FIRST, TWL_HIGH_MAX = 0, 1
+PAGE = 16
+HEAD_DIM = 128
+INT4_RECORD_BYTES = 1280
+META_RECORD_BYTES = 512
+MAX_CANDIDATES = 32768
+
+# every symbol include/twilight_hip.h declares
+EXPORTS = (
+    "twl_strerror", "twl_abi_version", "twl_device_count", "twl_top_p_f32", "twl_top_p_f16",
+    "twl_softmax_top_p_f32", "twl_gemv_int4", "twl_gemv_int4_nhd", "twl_sparse_attn",
+    "twl_quest_select", "twl_kv_shadow_build", "twl_dequant_int4", "twl_decode_layer",
+)
+
+
+class LayerArgs(ctypes.Structure):
+    """Mirror of ``struct twl_layer_args``."""
+    _fields_ = [
+        ("q", c_void_p), ("dtype", c_int), ("k_cache", c_void_p), ("v_cache", c_void_p),
+        ("page_stride", c_uint64), ("token_stride", c_uint64), ("head_stride", c_uint64),
+        ("k_int4", c_void_p), ("meta", c_void_p),
+        ("kv_page_indices", c_void_p), ("kv_page_indptr", c_void_p), ("kv_last_page_len", c_void_p),
+        ("batch", c_uint32), ("num_q_heads", c_uint32), ("num_kv_heads", c_uint32),
+        ("max_pages_per_req", c_uint32), ("token_budget", c_uint32),
+        ("top_p", c_float), ("high_mode", c_int), ("sm_scale", c_float),
+        ("sel_pages", c_void_p), ("sel_stride", c_uint32),
+        ("sel_count", c_void_p),
+        ("page_scores", c_void_p), ("page_score_stride", c_uint32),
+        ("scores", c_void_p), ("score_stride", c_uint32),
+        ("cand_count", c_void_p),
+        ("idx", c_void_p), ("idx_stride", c_uint32),
+        ("count", c_void_p),
+        ("out", c_void_p),
+    ]
+
+
+_lib = None
+
+
+def lib() -> ctypes.CDLL:
+    """Load the library once. Raises ``RuntimeError`` when it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: build it with `python -m twilight_amd.build` "
+            "(hipcc --offload-arch=gfx950); twilight_amd has no CPU or PyTorch fallback")
+    L = ctypes.CDLL(LIB_PATH)
+    vp, u32, u64, f32, i32 = c_void_p, c_uint32, c_uint64, c_float, c_int
+    L.twl_strerror.argtypes = [c_int]
+    L.twl_strerror.restype = c_char_p
+    L.twl_abi_version.argtypes = []
+    L.twl_device_count.argtypes = []
+    L.twl_top_p_f32.argtypes = [vp, vp, vp, vp, vp, f32, u32, u32, u32, i32, vp, vp, vp]
+    L.twl_top_p_f16.argtypes = [vp, i32, vp, vp, vp, vp, f32, u32, u32, u32, i32, vp, vp, vp]
+    L.twl_softmax_top_p_f32.argtypes = [vp, u32, vp, u32, u32, vp, f32, i32, vp, u32, vp, u32, vp,
+                                        vp, vp, vp]
+    L.twl_gemv_int4.argtypes = [vp, i32, vp, u32, vp, vp, vp, vp, u32, vp, vp, vp, u32, u32, u32,
+                                u32, f32, vp]
+    L.twl_gemv_int4_nhd.argtypes = [vp, vp, u32, vp, vp, vp, vp, vp, vp, u32, u32, u32, u32, f32, vp]
+    L.twl_sparse_attn.argtypes = [vp, vp, i32, vp, vp, u64, u64, u64, vp, u32, vp, vp, vp, u32, u32,
+                                  u32, f32, vp, vp]
+    L.twl_quest_select.argtypes = [vp, i32, vp, vp, vp, u32, u32, u32, u32, u32, vp, u32, vp, vp,
+                                   u32, vp]
+    L.twl_kv_shadow_build.argtypes = [vp, i32, u64, u64, u64, vp, vp, u32, u32, vp, vp, vp]
+    L.twl_dequant_int4.argtypes = [vp, u32, vp, vp]
+    L.twl_decode_layer.argtypes = [POINTER(LayerArgs), vp]
+    for name in EXPORTS:
+        if name != "twl_strerror":
+            getattr(L, name).restype = c_int
+    _lib = L
+    return L
+
+
+def strerror(rc: int) -> str:
+    return lib().twl_strerror(rc).decode()
+
+
+def check(rc: int, what: str) -> None:
+    """Raise ``RuntimeError`` for a non-zero status, as the reference's TORCH_CHECK does
+    (csrc/src/sampling.cu:39-40,61-62)."""
+    if rc != TWL_OK:
+        raise RuntimeError(f"{what} failed with error code {rc}: {strerror(rc)}")

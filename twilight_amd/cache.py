@@ -1,0 +1,128 @@
+"""Paged KV cache with the two side structures the decode path reads: the INT4 K shadow and the
+Quest page metadata. Storage only — every computation is a call into ``twilight_amd.kernel``."""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from . import _lib
+from .kernel import kv_shadow_build
+
+PAGE = _lib.PAGE
+HEAD_DIM = _lib.HEAD_DIM
+
+
+class PagedKVCache:
+    """K / V pages ``[num_pages, 16, Hkv, 128]`` (fp16 or bf16) plus ``k_int4``
+    ``[num_pages, Hkv, 1280]`` and ``meta`` ``[num_pages, Hkv, 512]`` (uint8 records), and the
+    CSR page table of the current batch (``kv_page_indices``, ``kv_page_indptr``,
+    ``kv_last_page_len``; the layout benchmark/efficiency/bench_gemv.py:425-431 builds)."""
+
+    def __init__(self, num_pages: int, num_kv_heads: int, dtype: torch.dtype, device):
+        if dtype not in (torch.float16, torch.bfloat16):
+            raise RuntimeError("PagedKVCache dtype must be float16 or bfloat16")
+        self.num_pages, self.num_kv_heads, self.dtype = num_pages, num_kv_heads, dtype
+        self.device = torch.device(device)
+        shape = (num_pages, PAGE, num_kv_heads, HEAD_DIM)
+        self.k_cache = torch.zeros(shape, dtype=dtype, device=self.device)
+        self.v_cache = torch.zeros(shape, dtype=dtype, device=self.device)
+        self.k_int4 = torch.zeros((num_pages, num_kv_heads, _lib.INT4_RECORD_BYTES),
+                                  dtype=torch.uint8, device=self.device)
+        self.meta = torch.zeros((num_pages, num_kv_heads, _lib.META_RECORD_BYTES),
+                                dtype=torch.uint8, device=self.device)
+        self.kv_page_indices: Optional[torch.Tensor] = None
+        self.kv_page_indptr: Optional[torch.Tensor] = None
+        self.kv_last_page_len: Optional[torch.Tensor] = None
+        self.max_pages_per_req = 0
+        self._seq_lens = None  # host copy, for append bookkeeping
+
+    # ---- page table ---------------------------------------------------------------------------
+    def set_page_table(self, kv_page_indices: torch.Tensor, kv_page_indptr: torch.Tensor,
+                       kv_last_page_len: torch.Tensor) -> None:
+        self.kv_page_indices = kv_page_indices.to(self.device, torch.int32).contiguous()
+        self.kv_page_indptr = kv_page_indptr.to(self.device, torch.int32).contiguous()
+        self.kv_last_page_len = kv_last_page_len.to(self.device, torch.int32).contiguous()
+        ip = kv_page_indptr.cpu().long()
+        npg = ip[1:] - ip[:-1]
+        self.max_pages_per_req = int(npg.max().item())
+        self._seq_lens = ((npg - 1) * PAGE + kv_last_page_len.cpu().long()).tolist()
+
+    @property
+    def batch(self) -> int:
+        return self.kv_page_indptr.numel() - 1
+
+    # ---- filling ------------------------------------------------------------------------------
+    def rebuild_shadow(self, page_ids: Optional[torch.Tensor] = None,
+                       valid_len: Optional[torch.Tensor] = None) -> None:
+        """(Re)build INT4 records and Quest metadata of ``page_ids`` (default: every page, all 16
+        tokens valid)."""
+        kv_shadow_build(self.k_cache, self.k_int4, self.meta, page_ids, valid_len)
+
+    @classmethod
+    def from_dense(cls, k: torch.Tensor, v: torch.Tensor, device, page_perm: Optional[torch.Tensor] = None,
+                   spare_pages: int = 0) -> "PagedKVCache":
+        """Page dense ``k`` / ``v`` [B, Hkv, N, 128] (prefill fill). ``page_perm`` (a permutation of
+        ``B*ceil(N/16)`` ids) scatters logical pages over physical slots."""
+        B, Hkv, N, D = k.shape
+        assert D == HEAD_DIM and v.shape == k.shape
+        npg = (N + PAGE - 1) // PAGE
+        total = B * npg
+        c = cls(total + spare_pages, Hkv, k.dtype, device)
+        if page_perm is None:
+            page_perm = torch.arange(total)
+        page_perm = page_perm.long()
+
+        def paged(x):
+            pad = npg * PAGE - N
+            if pad:
+                x = torch.nn.functional.pad(x, (0, 0, 0, pad))
+            return x.reshape(B, Hkv, npg, PAGE, D).permute(0, 2, 3, 1, 4).reshape(total, PAGE, Hkv, D)
+
+        perm_dev = page_perm.to(c.device)
+        c.k_cache[perm_dev] = paged(k).to(c.device)
+        c.v_cache[perm_dev] = paged(v).to(c.device)
+        last = N - (npg - 1) * PAGE
+        c.set_page_table(page_perm.to(torch.int32), (torch.arange(B + 1) * npg).to(torch.int32),
+                         torch.full((B,), last, dtype=torch.int32))
+        # valid tokens per physical page: 16 everywhere except each request's last page
+        valid = torch.full((total + spare_pages,), PAGE, dtype=torch.int32)
+        last_pages = page_perm.reshape(B, npg)[:, -1]
+        valid[last_pages] = last
+        ids = torch.arange(total + spare_pages, dtype=torch.int32)
+        c.rebuild_shadow(ids.to(c.device), valid.to(c.device))
+        return c
+
+    def append(self, k_new: torch.Tensor, v_new: torch.Tensor, free_pages: Optional[list] = None) -> None:
+        """Decode append of one token per request: ``k_new`` / ``v_new`` [B, Hkv, 128]. Writes the
+        token, extends the page table when a request's last page is full (taking ids from
+        ``free_pages``), and refreshes the shadow records of the touched pages."""
+        B = self.batch
+        ip = self.kv_page_indptr.cpu().tolist()
+        idx = self.kv_page_indices.cpu().tolist()
+        last = self.kv_last_page_len.cpu().tolist()
+        per_req = [idx[ip[b]:ip[b + 1]] for b in range(B)]
+        touched, valid, slots = [], [], []
+        for b in range(B):
+            if last[b] == PAGE:
+                if not free_pages:
+                    raise RuntimeError("PagedKVCache.append: no free page left")
+                per_req[b].append(int(free_pages.pop(0)))
+                last[b] = 0
+            page = per_req[b][-1]
+            slots.append((page, last[b]))
+            last[b] += 1
+            touched.append(page)
+            valid.append(last[b])
+        pg = torch.tensor([s[0] for s in slots], device=self.device)
+        sl = torch.tensor([s[1] for s in slots], device=self.device)
+        self.k_cache[pg, sl] = k_new.to(self.device, self.dtype)
+        self.v_cache[pg, sl] = v_new.to(self.device, self.dtype)
+        flat = [p for r in per_req for p in r]
+        ptr = [0]
+        for r in per_req:
+            ptr.append(ptr[-1] + len(r))
+        self.set_page_table(torch.tensor(flat, dtype=torch.int32), torch.tensor(ptr, dtype=torch.int32),
+                            torch.tensor(last, dtype=torch.int32))
+        self.rebuild_shadow(torch.tensor(touched, dtype=torch.int32, device=self.device),
+                            torch.tensor(valid, dtype=torch.int32, device=self.device))

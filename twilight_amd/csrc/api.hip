@@ -1,0 +1,72 @@
+// Library-level entry points: status strings, version, and the whole decode layer as one call
+// that enqueues the five kernels of the path back to back on the caller's stream.
+#include <hip/hip_runtime.h>
+
+#include "../../include/twilight_hip.h"
+
+extern "C" const char* twl_strerror(int status) {
+  switch (status) {
+    case TWL_OK: return "ok";
+    case TWL_ENULL: return "a required pointer is NULL";
+    case TWL_EINVAL: return "a size, stride or mode argument is out of range";
+    case TWL_EDTYPE: return "unsupported element type";
+    case TWL_EALIGN: return "pointer or stride alignment not supported";
+    case TWL_ELAUNCH: return "HIP kernel launch failed";
+    case TWL_ENODEVICE: return "no usable HIP device";
+    default: return "unknown twl_status";
+  }
+}
+
+extern "C" int twl_abi_version(void) { return 1; }
+
+extern "C" int twl_device_count(void) {
+  int n = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess) {
+    (void)hipGetLastError();
+    return TWL_ENODEVICE;
+  }
+  return n;
+}
+
+// twilight/pyimpl/attention.py:188-306 for q_len == 1: selector -> estimator -> pruner -> attention.
+extern "C" int twl_decode_layer(const twl_layer_args* a, void* stream) {
+  if (!a) return TWL_ENULL;
+  if (!a->sel_pages || !a->sel_count || !a->scores || !a->cand_count || !a->idx || !a->count ||
+      !a->out)
+    return TWL_ENULL;
+  if (a->batch == 0 || a->num_q_heads == 0) return TWL_EINVAL;
+  const uint32_t rows = a->batch * a->num_q_heads;
+  uint32_t k = (a->token_budget / TWL_PAGE ? a->token_budget / TWL_PAGE : 1) +
+               (a->token_budget % TWL_PAGE ? 1 : 0);
+  if (k > a->max_pages_per_req) k = a->max_pages_per_req;
+  if (a->sel_stride < k || a->score_stride < k * TWL_PAGE || a->idx_stride < k * TWL_PAGE)
+    return TWL_EINVAL;
+  float* page_scores = a->page_scores ? a->page_scores : a->scores;
+  const uint32_t ps_stride = a->page_scores ? a->page_score_stride : a->score_stride;
+  if (ps_stride < a->max_pages_per_req) return TWL_EINVAL;
+  if (k * TWL_PAGE > TWL_MAX_CANDIDATES) return TWL_EINVAL;
+  (void)rows;
+
+  // 1. Quest page scores + top-k pages
+  int rc = twl_quest_select(a->q, a->dtype, a->meta, a->kv_page_indices, a->kv_page_indptr,
+                            a->batch, a->num_q_heads, a->num_kv_heads, a->token_budget,
+                            a->max_pages_per_req, a->sel_pages, a->sel_stride, a->sel_count,
+                            page_scores, ps_stride, stream);
+  if (rc != TWL_OK) return rc;
+  // 2. INT4 estimate over the selected pages
+  rc = twl_gemv_int4(a->q, a->dtype, a->scores, a->score_stride, a->cand_count, a->k_int4,
+                     a->sel_pages, a->sel_count, a->sel_stride, a->kv_page_indices,
+                     a->kv_page_indptr, a->kv_last_page_len, a->batch, a->num_q_heads,
+                     a->num_kv_heads, k, a->sm_scale, stream);
+  if (rc != TWL_OK) return rc;
+  // 3. softmax + top-p + compaction to token positions
+  rc = twl_softmax_top_p_f32(a->scores, a->score_stride, a->cand_count, rows, k * TWL_PAGE,
+                             nullptr, a->top_p, a->high_mode, a->sel_pages, a->sel_stride, a->idx,
+                             a->idx_stride, a->count, nullptr, nullptr, stream);
+  if (rc != TWL_OK) return rc;
+  // 4. exact attention over the survivors
+  return twl_sparse_attn(a->q, a->out, a->dtype, a->k_cache, a->v_cache, a->page_stride,
+                         a->token_stride, a->head_stride, a->idx, a->idx_stride, a->count,
+                         a->kv_page_indices, a->kv_page_indptr, a->batch, a->num_q_heads,
+                         a->num_kv_heads, a->sm_scale, nullptr, stream);
+}

@@ -1,0 +1,298 @@
+// INT4-K score GEMV: out[row, c] = sm_scale * sum_d q[row, d] * (nibble * scale + zero).
+//
+// Restates the estimator matmul of twilight/pyimpl/attention.py:252-254 over the candidate pages
+// only, reading the INT4 shadow records defined in twilight_hip.h. It is a pure HBM stream
+// (80 bytes per token-head for 256 flops), so there is no MFMA: one wavefront owns a run of
+// candidate pages of one (batch, head) row and, per page, issues one 16-byte load per lane
+// (64 lanes x 16 B = the page's 1 KiB of nibbles) plus one 4-byte load per lane (its fp16 scale /
+// zero pair). Lane l holds token l/4, quantisation group l%4 — exactly the 32 nibbles that share
+// one scale — so dequantisation factors out of the inner loop:
+//     partial = scale * sum_j q_j * nibble_j + zero * sum_j q_j
+// with sum_j q_j precomputed once per row. Nibbles become exact fp16 integers with one
+// v_and_or (1024 + n) and one packed subtract, products are accumulated in fp32 by v_dot2, and a
+// two-step DPP quad reduction yields the token's score.
+#include "twl_common.h"
+
+namespace twl {
+
+struct GemvArgs {
+  const void* q;
+  float* out;
+  uint32_t out_stride;
+  int32_t* out_count;
+  const uint8_t* k_int4;
+  const int32_t* sel_pages;
+  const int32_t* sel_count;
+  uint32_t sel_stride;
+  const int32_t* kv_page_indices;
+  const int32_t* kv_page_indptr;
+  const int32_t* kv_last_page_len;
+  uint32_t num_q_heads;
+  uint32_t num_kv_heads;
+  uint32_t max_pages;  // pages per row the grid and the output row are sized for
+  float sm_scale;
+};
+
+constexpr int kGemvThreads = 256;                 // 4 wavefronts
+constexpr int kGemvPagesPerWave = 16;
+constexpr int kGemvPagesPerBlock = kGemvPagesPerWave * (kGemvThreads / kWave);
+constexpr int kGemvUnroll = 4;
+
+// 8 nibbles of one dword against 8 q values held as 4 half2 pairs (n0,n4),(n1,n5),(n2,n6),(n3,n7)
+__device__ __forceinline__ float dot8_nibbles(uint32_t w, const half2_t* qp, float acc) {
+  const half2_t bias = {(_Float16)1024.0f, (_Float16)1024.0f};
+  const uint32_t m = 0x000F000Fu, magic = 0x64006400u;  // fp16 1024 + n
+  half2_t a0 = __builtin_bit_cast(half2_t, (w & m) | magic) - bias;
+  half2_t a1 = __builtin_bit_cast(half2_t, ((w >> 4) & m) | magic) - bias;
+  half2_t a2 = __builtin_bit_cast(half2_t, ((w >> 8) & m) | magic) - bias;
+  half2_t a3 = __builtin_bit_cast(half2_t, ((w >> 12) & m) | magic) - bias;
+  acc = __builtin_amdgcn_fdot2(a0, qp[0], acc, false);
+  acc = __builtin_amdgcn_fdot2(a1, qp[1], acc, false);
+  acc = __builtin_amdgcn_fdot2(a2, qp[2], acc, false);
+  acc = __builtin_amdgcn_fdot2(a3, qp[3], acc, false);
+  return acc;
+}
+
+template <int QDT>
+__global__ __launch_bounds__(kGemvThreads) void gemv_int4_kernel(GemvArgs a) {
+  const uint32_t row = blockIdx.y;
+  const uint32_t b = row / a.num_q_heads;
+  const uint32_t h = row - b * a.num_q_heads;
+  const uint32_t kvh = h / (a.num_q_heads / a.num_kv_heads);
+  const int lane = lane_id();
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+
+  const int pg_begin = a.kv_page_indptr[b];
+  const int req_pages = a.kv_page_indptr[b + 1] - pg_begin;
+  int n_pages = a.sel_pages ? (a.sel_count ? a.sel_count[row] : (int)a.sel_stride) : req_pages;
+  n_pages = min(max(n_pages, 0), (int)a.max_pages);
+  if (req_pages <= 0) n_pages = 0;
+  if (blockIdx.x == 0 && threadIdx.x == 0 && a.out_count) a.out_count[row] = n_pages * TWL_PAGE;
+
+  const int p0 = blockIdx.x * kGemvPagesPerBlock + wave * kGemvPagesPerWave;
+  if (p0 >= n_pages) return;
+  const int np = min(kGemvPagesPerWave, n_pages - p0);
+
+  // ---- q: lane (t = l/4, g = l%4) keeps q[32g .. 32g+32) as 16 half2 pairs -------------------
+  const int g = lane & 3;
+  const int t = lane >> 2;
+  half2_t qp[16];
+  float qsum = 0.0f;
+  {
+    const uint16_t* qrow = (const uint16_t*)a.q + (size_t)row * TWL_HEAD_DIM + 32 * g;
+    float qf[32];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      u32x4 v = *(const u32x4*)(qrow + 8 * i);
+      const uint32_t ws[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        qf[8 * i + 2 * j] = bits16_to_f32<QDT>(ws[j] & 0xFFFFu);
+        qf[8 * i + 2 * j + 1] = bits16_to_f32<QDT>(ws[j] >> 16);
+      }
+    }
+#pragma unroll
+    for (int w = 0; w < 4; ++w)
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        half2_t pr = {(_Float16)qf[8 * w + s], (_Float16)qf[8 * w + s + 4]};
+        qp[4 * w + s] = pr;
+      }
+#pragma unroll
+    for (int i = 0; i < 32; ++i) qsum += (float)(_Float16)qf[i];
+  }
+
+  // ---- page ids of this wave's run: lane i owns run entry i ---------------------------------
+  int my_logical = -1, my_phys = 0;
+  if (lane < np) {
+    my_logical = a.sel_pages ? a.sel_pages[(size_t)row * a.sel_stride + p0 + lane] : p0 + lane;
+    my_logical = min(max(my_logical, 0), req_pages - 1);  // a corrupt list must not leave the table
+    my_phys = a.kv_page_indices[pg_begin + my_logical];
+  }
+  const int last_len = a.kv_last_page_len[b];
+  const size_t rec_stride = (size_t)a.num_kv_heads * TWL_INT4_RECORD_BYTES;
+  const uint8_t* base = a.k_int4 + (size_t)kvh * TWL_INT4_RECORD_BYTES;
+  float* orow = a.out + (size_t)row * a.out_stride + (size_t)p0 * TWL_PAGE;
+  const float ninf = -__builtin_inff();
+
+#pragma unroll
+  for (int i0 = 0; i0 < kGemvPagesPerWave; i0 += kGemvUnroll) {
+    if (i0 >= np) break;
+    u32x4 nib[kGemvUnroll];
+    uint32_t sz[kGemvUnroll];
+    int logical[kGemvUnroll];
+#pragma unroll
+    for (int u = 0; u < kGemvUnroll; ++u) {
+      const int i = i0 + u;
+      // entries past the run reuse entry 0: a valid address, result discarded
+      const int src_lane = (i < np) ? i : 0;
+      const int phys = __builtin_amdgcn_readlane(my_phys, src_lane);
+      logical[u] = __builtin_amdgcn_readlane(my_logical, src_lane);
+      const uint8_t* rec = base + (size_t)phys * rec_stride;
+      nib[u] = *(const u32x4*)(rec + 16 * lane);
+      sz[u] = *(const uint32_t*)(rec + 1024 + 4 * lane);
+    }
+#pragma unroll
+    for (int u = 0; u < kGemvUnroll; ++u) {
+      const int i = i0 + u;
+      float acc = 0.0f;
+      acc = dot8_nibbles(nib[u].x, qp + 0, acc);
+      acc = dot8_nibbles(nib[u].y, qp + 4, acc);
+      acc = dot8_nibbles(nib[u].z, qp + 8, acc);
+      acc = dot8_nibbles(nib[u].w, qp + 12, acc);
+      const float scale = f16_bits_to_f32(sz[u] & 0xFFFFu);
+      const float zero = f16_bits_to_f32(sz[u] >> 16);
+      float part = fmaf(zero, qsum, scale * acc);
+      part = quad_allreduce<OpSum>(part);
+      if (i < np && g == 0) {
+        const int valid = (logical[u] == req_pages - 1) ? last_len : TWL_PAGE;
+        orow[i * TWL_PAGE + t] = (t < valid) ? part * a.sm_scale : ninf;
+      }
+    }
+  }
+}
+
+// ---- the same arithmetic over the tensor layout of benchmark/efficiency/bench_gemv.py:390-454 ---
+struct GemvNhdArgs {
+  const uint16_t* q;
+  uint16_t* o;
+  uint32_t o_stride;
+  const uint8_t* k_u8;
+  const uint16_t* scales;
+  const uint16_t* zeros;
+  const int32_t* kv_page_indices;
+  const int32_t* kv_page_indptr;
+  const int32_t* kv_last_page_len;
+  uint32_t num_heads;
+  uint32_t page_size;
+  uint32_t max_tok;  // tokens per request the grid and the output row are sized for
+  float sm_scale;
+};
+
+// One wavefront scores 16 tokens per step: lane l -> token l/4 of the step, 32-element slice l%4.
+// A token's 64 nibble bytes are contiguous; scale / zero are per token.
+__global__ __launch_bounds__(kGemvThreads) void gemv_int4_nhd_kernel(GemvNhdArgs a) {
+  const uint32_t row = blockIdx.y;
+  const uint32_t b = row / a.num_heads;
+  const uint32_t h = row - b * a.num_heads;
+  const int lane = lane_id();
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int g = lane & 3;
+  const int t = lane >> 2;
+
+  const int pg_begin = a.kv_page_indptr[b];
+  const int req_pages = a.kv_page_indptr[b + 1] - pg_begin;
+  if (req_pages <= 0) return;
+  const int n_tok = min((req_pages - 1) * (int)a.page_size + a.kv_last_page_len[b], (int)a.max_tok);
+
+  half2_t qp[16];
+  float qsum = 0.0f;
+  {
+    const uint16_t* qrow = a.q + (size_t)row * TWL_HEAD_DIM + 32 * g;
+    float qf[32];
+#pragma unroll
+    for (int i = 0; i < 32; ++i) qf[i] = f16_bits_to_f32(qrow[i]);
+#pragma unroll
+    for (int w = 0; w < 4; ++w)
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        half2_t pr = {(_Float16)qf[8 * w + s], (_Float16)qf[8 * w + s + 4]};
+        qp[4 * w + s] = pr;
+      }
+#pragma unroll
+    for (int i = 0; i < 32; ++i) qsum += qf[i];
+  }
+
+  constexpr int kTokPerBlock = 16 * 4 * 4;  // 4 waves x 4 steps x 16 tokens
+  const int n0 = blockIdx.x * kTokPerBlock + wave * 64;
+#pragma unroll
+  for (int s = 0; s < 4; ++s) {
+    const int n = n0 + 16 * s + t;
+    if (n < n_tok) {
+      const int lp = n / (int)a.page_size;
+      const int slot = n - lp * (int)a.page_size;
+      const size_t tok = ((size_t)a.kv_page_indices[pg_begin + lp] * a.page_size + slot) *
+                             a.num_heads + h;
+      u32x4 nib = *(const u32x4*)(a.k_u8 + tok * 64 + 16 * g);
+      const float scale = f16_bits_to_f32(a.scales[tok]);
+      const float zero = f16_bits_to_f32(a.zeros[tok]);
+      float acc = 0.0f;
+      acc = dot8_nibbles(nib.x, qp + 0, acc);
+      acc = dot8_nibbles(nib.y, qp + 4, acc);
+      acc = dot8_nibbles(nib.z, qp + 8, acc);
+      acc = dot8_nibbles(nib.w, qp + 12, acc);
+      float part = fmaf(zero, qsum, scale * acc);
+      // tokens are aligned to quads, so all four lanes of a quad take this branch together
+      part = quad_allreduce<OpSum>(part);
+      if (g == 0)
+        a.o[(size_t)row * a.o_stride + n] = (uint16_t)f32_to_f16_bits(part * a.sm_scale);
+    }
+  }
+}
+
+}  // namespace twl
+
+extern "C" int twl_gemv_int4(const void* q, int q_dtype, float* out, uint32_t out_stride,
+                             int32_t* out_count, const void* k_int4, const int32_t* sel_pages,
+                             const int32_t* sel_count, uint32_t sel_stride,
+                             const int32_t* kv_page_indices, const int32_t* kv_page_indptr,
+                             const int32_t* kv_last_page_len, uint32_t batch,
+                             uint32_t num_q_heads, uint32_t num_kv_heads,
+                             uint32_t max_pages_per_row, float sm_scale, void* stream) {
+  if (!q || !out || !k_int4 || !kv_page_indices || !kv_page_indptr || !kv_last_page_len)
+    return TWL_ENULL;
+  if (sel_count && !sel_pages) return TWL_ENULL;
+  if (q_dtype != TWL_F16 && q_dtype != TWL_BF16) return TWL_EDTYPE;
+  if (batch == 0 || num_q_heads == 0 || num_kv_heads == 0 || num_q_heads % num_kv_heads != 0)
+    return TWL_EINVAL;
+  if (max_pages_per_row == 0 || (uint64_t)max_pages_per_row * TWL_PAGE > out_stride)
+    return TWL_EINVAL;
+  if (sel_pages && sel_stride < max_pages_per_row) return TWL_EINVAL;
+  if ((uint64_t)batch * num_q_heads > 65535u) return TWL_EINVAL;
+  if ((((uintptr_t)q) & 15u) || (((uintptr_t)k_int4) & 15u) || (((uintptr_t)out) & 3u))
+    return TWL_EALIGN;
+  twl::GemvArgs a{};
+  a.q = q; a.out = out; a.out_stride = out_stride; a.out_count = out_count;
+  a.k_int4 = (const uint8_t*)k_int4; a.sel_pages = sel_pages; a.sel_count = sel_count;
+  a.sel_stride = sel_stride; a.kv_page_indices = kv_page_indices; a.kv_page_indptr = kv_page_indptr;
+  a.kv_last_page_len = kv_last_page_len; a.num_q_heads = num_q_heads;
+  a.num_kv_heads = num_kv_heads; a.max_pages = max_pages_per_row; a.sm_scale = sm_scale;
+  const uint32_t gx = (max_pages_per_row + twl::kGemvPagesPerBlock - 1) / twl::kGemvPagesPerBlock;
+  dim3 grid(gx, batch * num_q_heads);
+  if (q_dtype == TWL_F16)
+    hipLaunchKernelGGL((twl::gemv_int4_kernel<TWL_F16>), grid, dim3(twl::kGemvThreads), 0,
+                       (hipStream_t)stream, a);
+  else
+    hipLaunchKernelGGL((twl::gemv_int4_kernel<TWL_BF16>), grid, dim3(twl::kGemvThreads), 0,
+                       (hipStream_t)stream, a);
+  return hipGetLastError() == hipSuccess ? TWL_OK : TWL_ELAUNCH;
+}
+
+extern "C" int twl_gemv_int4_nhd(const void* q, void* o, uint32_t o_stride, const uint8_t* k_u8,
+                                 const void* scales, const void* zeros,
+                                 const int32_t* kv_page_indices, const int32_t* kv_page_indptr,
+                                 const int32_t* kv_last_page_len, uint32_t batch,
+                                 uint32_t num_heads, uint32_t page_size,
+                                 uint32_t max_pages_per_req, float sm_scale, void* stream) {
+  if (!q || !o || !k_u8 || !scales || !zeros || !kv_page_indices || !kv_page_indptr ||
+      !kv_last_page_len)
+    return TWL_ENULL;
+  if (batch == 0 || num_heads == 0 || page_size == 0 || max_pages_per_req == 0) return TWL_EINVAL;
+  if ((uint64_t)max_pages_per_req * page_size > o_stride) return TWL_EINVAL;
+  if ((uint64_t)batch * num_heads > 65535u) return TWL_EINVAL;
+  if ((((uintptr_t)k_u8) & 15u) || (((uintptr_t)q) & 1u) || (((uintptr_t)o) & 1u))
+    return TWL_EALIGN;
+  twl::GemvNhdArgs a{};
+  a.q = (const uint16_t*)q; a.o = (uint16_t*)o; a.o_stride = o_stride; a.k_u8 = k_u8;
+  a.scales = (const uint16_t*)scales; a.zeros = (const uint16_t*)zeros;
+  a.kv_page_indices = kv_page_indices; a.kv_page_indptr = kv_page_indptr;
+  a.kv_last_page_len = kv_last_page_len; a.num_heads = num_heads; a.page_size = page_size;
+  a.sm_scale = sm_scale;
+  const uint64_t max_tok = (uint64_t)max_pages_per_req * page_size;
+  if (max_tok > 0x7FFFFFFFull) return TWL_EINVAL;
+  a.max_tok = (uint32_t)max_tok;
+  dim3 grid((uint32_t)((max_tok + 255) / 256), batch * num_heads);
+  hipLaunchKernelGGL(twl::gemv_int4_nhd_kernel, grid, dim3(twl::kGemvThreads), 0,
+                     (hipStream_t)stream, a);
+  return hipGetLastError() == hipSuccess ? TWL_OK : TWL_ELAUNCH;
+}

@@ -1,0 +1,173 @@
+// KV-append side of the path: INT4 shadow records and Quest min/max metadata from paged K.
+//
+// The quantiser restates twilight/pyimpl/quantize.py:4-13 (asymmetric min/max, 4 bits) per group
+// of 32 channels, storing scale and zero (= group minimum) as fp16 and computing the code from the
+// ROUNDED scale / zero so that code * scale + zero is what the GEMV will see. The reference
+// re-quantises all of K on every decode step (twilight/pyimpl/attention.py:247-251); here it runs
+// once per page when the page is written. The metadata is the channel-wise min / max over the
+// page's valid tokens, the stored form of the per-chunk amax of twilight/pyimpl/quest.py:68-74.
+//
+// One wavefront per (page, kv head): lane l = token l/4, group l%4 reads its 32 channels
+// (4 x 16 B), quantises them in registers and writes 16 B of nibbles + one (scale, zero) pair;
+// the page tile is staged through LDS once for the per-channel min / max.
+#include "twl_common.h"
+
+namespace twl {
+
+struct ShadowArgs {
+  const void* k_cache;
+  uint64_t page_stride, token_stride, head_stride;
+  const int32_t* page_ids;
+  const int32_t* valid_len;
+  uint32_t num_pages, num_kv_heads;
+  uint8_t* k_int4;
+  uint8_t* meta;
+};
+
+constexpr int kShThreads = 256;
+constexpr int kShWaves = kShThreads / kWave;
+
+template <int DT>
+__global__ __launch_bounds__(kShThreads) void kv_shadow_kernel(ShadowArgs a) {
+  __shared__ float tile[kShWaves][TWL_PAGE][TWL_HEAD_DIM + 4];
+  const int lane = lane_id();
+  const int wave = threadIdx.x / kWave;
+  const uint32_t item = blockIdx.x * kShWaves + wave;
+  const bool active = item < a.num_pages * a.num_kv_heads;  // wave-uniform
+  const uint32_t pi = active ? item / a.num_kv_heads : 0;
+  const uint32_t kvh = active ? item - pi * a.num_kv_heads : 0;
+  const int page = a.page_ids ? a.page_ids[pi] : (int)pi;
+  const int valid = a.valid_len ? min(max(a.valid_len[pi], 0), TWL_PAGE) : TWL_PAGE;
+  const int t = lane >> 2, g = lane & 3;
+
+  float x[32];
+  if (active) {
+    const uint16_t* src = (const uint16_t*)a.k_cache + (size_t)page * a.page_stride +
+                          (size_t)t * a.token_stride + (size_t)kvh * a.head_stride + 32 * g;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      u32x4 v = *(const u32x4*)(src + 8 * i);
+      const uint32_t ws[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        x[8 * i + 2 * j] = bits16_to_f32<DT>(ws[j] & 0xFFFFu);
+        x[8 * i + 2 * j + 1] = bits16_to_f32<DT>(ws[j] >> 16);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 32; ++i) x[i] = 0.0f;
+  }
+
+  if (active && a.k_int4) {
+    uint8_t* rec = a.k_int4 + ((size_t)page * a.num_kv_heads + kvh) * TWL_INT4_RECORD_BYTES;
+    u32x4 packed = {0u, 0u, 0u, 0u};
+    uint32_t sz = 0;
+    if (t < valid) {
+      float mn = x[0], mx = x[0];
+#pragma unroll
+      for (int i = 1; i < 32; ++i) {
+        mn = fminf(mn, x[i]);
+        mx = fmaxf(mx, x[i]);
+      }
+      const float range = fmaxf(mx - mn, 1e-9f);
+      float sh = round_to<TWL_F16>(range / 15.0f);
+      sh = fminf(fmaxf(sh, 6.103515625e-05f), 65504.0f);
+      float zh = round_to<TWL_F16>(mn);
+      zh = fminf(fmaxf(zh, -65504.0f), 65504.0f);
+      uint32_t w[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+      for (int i = 0; i < 32; ++i) {
+        float c = rintf((x[i] - zh) / sh);
+        c = fminf(fmaxf(c, 0.0f), 15.0f);
+        w[i >> 3] |= (uint32_t)c << (4 * (i & 7));
+      }
+      packed.x = w[0]; packed.y = w[1]; packed.z = w[2]; packed.w = w[3];
+      sz = f32_to_f16_bits(sh) | (f32_to_f16_bits(zh) << 16);
+    }
+    *(u32x4*)(rec + 16 * lane) = packed;
+    *(uint32_t*)(rec + 1024 + 4 * lane) = sz;
+  }
+
+  if (a.meta) {  // uniform across the block: barriers below are reached by every thread
+#pragma unroll
+    for (int i = 0; i < 32; ++i) tile[wave][t][32 * g + i] = x[i];
+    __syncthreads();
+    if (active) {
+      // lane l reduces channels 2l and 2l+1 over the valid tokens
+      float mn0 = __builtin_inff(), mn1 = __builtin_inff();
+      float mx0 = -__builtin_inff(), mx1 = -__builtin_inff();
+      for (int tt = 0; tt < valid; ++tt) {
+        const float v0 = tile[wave][tt][2 * lane], v1 = tile[wave][tt][2 * lane + 1];
+        mn0 = fminf(mn0, v0); mx0 = fmaxf(mx0, v0);
+        mn1 = fminf(mn1, v1); mx1 = fmaxf(mx1, v1);
+      }
+      if (valid == 0) { mn0 = mn1 = mx0 = mx1 = 0.0f; }
+      uint8_t* rec = a.meta + ((size_t)page * a.num_kv_heads + kvh) * TWL_META_RECORD_BYTES;
+      const int c = lane >> 1, o = (lane & 1) * 4;
+      *(uint32_t*)(rec + 16 * c + o) = f32_to_bits16<DT>(mn0) | (f32_to_bits16<DT>(mn1) << 16);
+      *(uint32_t*)(rec + 16 * c + 8 + o) = f32_to_bits16<DT>(mx0) | (f32_to_bits16<DT>(mx1) << 16);
+    }
+  }
+}
+
+// one thread per (record, token, group): 32 outputs
+__global__ __launch_bounds__(256) void dequant_int4_kernel(const uint8_t* k_int4,
+                                                           uint32_t num_records, float* out) {
+  const uint64_t gid = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+  const uint64_t rec_i = gid >> 6;
+  if (rec_i >= num_records) return;
+  const int l = (int)(gid & 63);
+  const uint8_t* rec = k_int4 + rec_i * TWL_INT4_RECORD_BYTES;
+  u32x4 v = *(const u32x4*)(rec + 16 * l);
+  const uint32_t sz = *(const uint32_t*)(rec + 1024 + 4 * l);
+  const float scale = f16_bits_to_f32(sz & 0xFFFFu), zero = f16_bits_to_f32(sz >> 16);
+  const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+  float* dst = out + rec_i * (TWL_PAGE * TWL_HEAD_DIM) + 32 * l;  // token l/4, group l%4
+#pragma unroll
+  for (int i = 0; i < 32; ++i) {
+    const float c = (float)((w[i >> 3] >> (4 * (i & 7))) & 0xFu);
+    dst[i] = fmaf(c, scale, zero);
+  }
+}
+
+}  // namespace twl
+
+extern "C" int twl_kv_shadow_build(const void* k_cache, int kv_dtype, uint64_t page_stride,
+                                   uint64_t token_stride, uint64_t head_stride,
+                                   const int32_t* page_ids, const int32_t* valid_len,
+                                   uint32_t num_pages, uint32_t num_kv_heads, void* k_int4,
+                                   void* meta, void* stream) {
+  if (!k_cache || (!k_int4 && !meta)) return TWL_ENULL;
+  if (kv_dtype != TWL_F16 && kv_dtype != TWL_BF16) return TWL_EDTYPE;
+  if (num_pages == 0 || num_kv_heads == 0) return TWL_EINVAL;
+  if ((uint64_t)num_pages * num_kv_heads > 0x7FFFFFFFull) return TWL_EINVAL;
+  if ((page_stride | token_stride | head_stride) & 7u) return TWL_EALIGN;
+  if ((((uintptr_t)k_cache) & 15u) || (((uintptr_t)k_int4) & 15u) || (((uintptr_t)meta) & 15u))
+    return TWL_EALIGN;
+  twl::ShadowArgs a{};
+  a.k_cache = k_cache; a.page_stride = page_stride; a.token_stride = token_stride;
+  a.head_stride = head_stride; a.page_ids = page_ids; a.valid_len = valid_len;
+  a.num_pages = num_pages; a.num_kv_heads = num_kv_heads; a.k_int4 = (uint8_t*)k_int4;
+  a.meta = (uint8_t*)meta;
+  const uint32_t items = num_pages * num_kv_heads;
+  dim3 grid((items + twl::kShWaves - 1) / twl::kShWaves);
+  if (kv_dtype == TWL_F16)
+    hipLaunchKernelGGL((twl::kv_shadow_kernel<TWL_F16>), grid, dim3(twl::kShThreads), 0,
+                       (hipStream_t)stream, a);
+  else
+    hipLaunchKernelGGL((twl::kv_shadow_kernel<TWL_BF16>), grid, dim3(twl::kShThreads), 0,
+                       (hipStream_t)stream, a);
+  return hipGetLastError() == hipSuccess ? TWL_OK : TWL_ELAUNCH;
+}
+
+extern "C" int twl_dequant_int4(const void* k_int4, uint32_t num_records, float* out,
+                                void* stream) {
+  if (!k_int4 || !out) return TWL_ENULL;
+  if (num_records == 0 || num_records > (1u << 25)) return TWL_EINVAL;
+  if ((((uintptr_t)k_int4) & 15u) || (((uintptr_t)out) & 3u)) return TWL_EALIGN;
+  const uint64_t threads = (uint64_t)num_records * 64;
+  hipLaunchKernelGGL(twl::dequant_int4_kernel, dim3((uint32_t)((threads + 255) / 256)), dim3(256),
+                     0, (hipStream_t)stream, (const uint8_t*)k_int4, num_records, out);
+  return hipGetLastError() == hipSuccess ? TWL_OK : TWL_ELAUNCH;
+}

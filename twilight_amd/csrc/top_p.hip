@@ -1,0 +1,367 @@
+// Top-p pruner: one workgroup per (batch, head) row, the row held in registers.
+//
+// Follows the bisection of csrc/include/sampling.cuh:156-231 iteration by iteration
+// (low = 0, high = probs[row][0] or the row maximum; mid = (low+high)/2; S = sum of probs > mid;
+// min_gt_low / max_le_high bracket; stop when the bracket is narrower than 1e-5; keep
+// probs > low), but reads the row from HBM exactly once: every thread keeps VPT values in
+// VGPRs, the three block reductions of an iteration are DPP wave reductions plus one LDS hop,
+// and the result is emitted as a byte mask and/or as an ascending index list with its count
+// (the stream compaction that replaces `mask & pruned_mask`, twilight/pyimpl/attention.py:280-281).
+//
+// The fused entry additionally computes the fp32 softmax of raw scores in the same registers
+// (twilight/pyimpl/top_p.py:10-15), so scores are read once and probabilities never hit HBM.
+#include "twl_common.h"
+
+namespace twl {
+
+struct TopPArgs {
+  const void* in;        // probs (any dtype) or raw fp32 scores
+  uint32_t in_stride;    // elements between rows
+  const int32_t* lens;   // nullable: per-row length (<= d)
+  uint32_t d;
+  const float* p_arr;    // nullable
+  float p;
+  int high_mode;
+  uint8_t* mask;         // nullable [rows, d]
+  int32_t* idx;          // nullable [rows, idx_stride]
+  uint32_t idx_stride;
+  int32_t* count;        // nullable [rows]
+  const int32_t* sel_pages;  // nullable: position -> token mapping through a page list
+  uint32_t sel_stride;
+  float* probs_out;      // nullable [rows, in_stride] (fused entry only)
+  float* low_out;        // nullable [rows]
+  int32_t* iters_out;    // nullable [rows]
+};
+
+// Element e of the row is held by thread (e/4) % THREADS, slot 4*((e/4)/THREADS) + e%4:
+// consecutive threads read consecutive 16-byte groups.
+template <int DT, int THREADS, int VPT, bool FUSED_SOFTMAX>
+__global__ __launch_bounds__(THREADS) void top_p_kernel(TopPArgs a) {
+  constexpr int NWAVES = THREADS / kWave;
+  constexpr int CHUNKS = VPT / 4;
+  __shared__ float red[2][3][16];
+  __shared__ int wave_tot[16];
+
+  const uint32_t row = blockIdx.x;
+  const int tx = threadIdx.x;
+  const int lane = lane_id();
+  const int wave = tx / kWave;
+  const uint32_t len = a.lens ? min((uint32_t)max(a.lens[row], 0), a.d) : a.d;
+
+  // ---- load the row once ----------------------------------------------------------------
+  float x[VPT];
+  const float fill = FUSED_SOFTMAX ? -__builtin_inff() : 0.0f;
+  if (DT == TWL_F32) {
+    const float* src = (const float*)a.in + (size_t)row * a.in_stride;
+    const bool vec_ok = ((((uintptr_t)src) & 15u) == 0);
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+      const uint32_t e0 = 4u * (uint32_t)(tx + THREADS * c);
+      if (vec_ok && e0 + 4 <= len) {
+        f32x4 v = *(const f32x4*)(src + e0);
+        x[4 * c + 0] = v.x; x[4 * c + 1] = v.y; x[4 * c + 2] = v.z; x[4 * c + 3] = v.w;
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) x[4 * c + j] = (e0 + j < len) ? src[e0 + j] : fill;
+      }
+    }
+  } else {
+    const uint16_t* src = (const uint16_t*)a.in + (size_t)row * a.in_stride;
+    const bool vec_ok = ((((uintptr_t)src) & 7u) == 0);
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+      const uint32_t e0 = 4u * (uint32_t)(tx + THREADS * c);
+      if (vec_ok && e0 + 4 <= len) {
+        u32x2 v = *(const u32x2*)(src + e0);
+        x[4 * c + 0] = bits16_to_f32<DT == TWL_F32 ? TWL_F16 : DT>(v.x & 0xFFFFu);
+        x[4 * c + 1] = bits16_to_f32<DT == TWL_F32 ? TWL_F16 : DT>(v.x >> 16);
+        x[4 * c + 2] = bits16_to_f32<DT == TWL_F32 ? TWL_F16 : DT>(v.y & 0xFFFFu);
+        x[4 * c + 3] = bits16_to_f32<DT == TWL_F32 ? TWL_F16 : DT>(v.y >> 16);
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          x[4 * c + j] = (e0 + j < len)
+                             ? bits16_to_f32<DT == TWL_F32 ? TWL_F16 : DT>(src[e0 + j])
+                             : fill;
+      }
+    }
+  }
+
+  int buf = 0;
+  // ---- softmax in registers (fused entry) -------------------------------------------------
+  if (FUSED_SOFTMAX) {
+    float m = -__builtin_inff();
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) m = fmaxf(m, x[k]);
+    m = block_allreduce<OpMax, NWAVES>(m, red[buf][0]);
+    buf ^= 1;
+    float z = 0.0f;
+    if (m == -__builtin_inff()) {
+      // empty row or all candidates masked: every probability is 0
+#pragma unroll
+      for (int k = 0; k < VPT; ++k) x[k] = 0.0f;
+    } else {
+#pragma unroll
+      for (int k = 0; k < VPT; ++k) {
+        x[k] = expf(x[k] - m);  // exp(-inf) == 0 for masked / out-of-row slots
+        z += x[k];
+      }
+      z = block_allreduce<OpSum, NWAVES>(z, red[buf][0]);
+      buf ^= 1;
+#pragma unroll
+      for (int k = 0; k < VPT; ++k) x[k] = x[k] / z;
+    }
+    if (a.probs_out) {
+      float* dst = a.probs_out + (size_t)row * a.in_stride;
+#pragma unroll
+      for (int c = 0; c < CHUNKS; ++c) {
+        const uint32_t e0 = 4u * (uint32_t)(tx + THREADS * c);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if (e0 + j < len) dst[e0 + j] = x[4 * c + j];
+      }
+    }
+  }
+
+  // ---- bisection (sampling.cuh:156-217) ----------------------------------------------------
+  const float p = round_to<DT>(a.p_arr ? a.p_arr[row] : a.p);
+  float low = 0.0f;
+  float high;
+  if (a.high_mode == TWL_HIGH_FIRST) {
+    // element 0 lives in thread 0, slot 0
+    __shared__ float first;
+    if (tx == 0) first = (len > 0) ? x[0] : 0.0f;
+    __syncthreads();
+    high = first;
+  } else {
+    float m = 0.0f;
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) m = fmaxf(m, x[k]);
+    high = block_allreduce<OpMax, NWAVES>(m, red[buf][0]);
+    buf ^= 1;
+  }
+  high = as_f32(__builtin_amdgcn_readfirstlane(as_i32(high)));
+  const float eps = round_to<DT>(1e-5f);
+  float min_gt_low, max_le_high;
+  int iters = 0;
+  do {
+    const float mid = round_to<DT>((low + high) * 0.5f);
+    float s = 0.0f, mn = high, mx = low;
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) {
+      const float v = x[k];
+      s += (v > mid) ? v : 0.0f;
+      mn = (v > low) ? fminf(mn, v) : mn;
+      mx = (v <= high) ? fmaxf(mx, v) : mx;
+    }
+    // three reductions, one barrier
+    s = wave_allreduce<OpSum>(s);
+    mn = wave_allreduce<OpMin>(mn);
+    mx = wave_allreduce<OpMax>(mx);
+    if (NWAVES > 1) {
+      if (lane == 0) {
+        red[buf][0][wave] = s;
+        red[buf][1][wave] = mn;
+        red[buf][2][wave] = mx;
+      }
+      __syncthreads();
+      float ts = red[buf][0][lane & (NWAVES - 1)];
+      float tn = red[buf][1][lane & (NWAVES - 1)];
+      float tm = red[buf][2][lane & (NWAVES - 1)];
+      if (NWAVES >= 2) {
+        ts += dpp<kDppXor1>(0.0f, ts);
+        tn = fminf(tn, dpp<kDppXor1>(tn, tn));
+        tm = fmaxf(tm, dpp<kDppXor1>(tm, tm));
+      }
+      if (NWAVES >= 4) {
+        ts += dpp<kDppXor2>(0.0f, ts);
+        tn = fminf(tn, dpp<kDppXor2>(tn, tn));
+        tm = fmaxf(tm, dpp<kDppXor2>(tm, tm));
+      }
+      if (NWAVES >= 8) {
+        ts += dpp<kDppHalfMirror>(0.0f, ts);
+        tn = fminf(tn, dpp<kDppHalfMirror>(tn, tn));
+        tm = fmaxf(tm, dpp<kDppHalfMirror>(tm, tm));
+      }
+      if (NWAVES >= 16) {
+        ts += dpp<kDppMirror>(0.0f, ts);
+        tn = fminf(tn, dpp<kDppMirror>(tn, tn));
+        tm = fmaxf(tm, dpp<kDppMirror>(tm, tm));
+      }
+      s = ts; mn = tn; mx = tm;
+      buf ^= 1;
+    }
+    // identical in every lane of every wave; make that explicit for the branch below
+    s = as_f32(__builtin_amdgcn_readfirstlane(as_i32(s)));
+    min_gt_low = as_f32(__builtin_amdgcn_readfirstlane(as_i32(mn)));
+    max_le_high = as_f32(__builtin_amdgcn_readfirstlane(as_i32(mx)));
+    if (s >= p) {
+      low = mid;
+    } else {
+      high = fminf(mid, max_le_high);
+    }
+    ++iters;
+  } while (round_to<DT>(max_le_high - min_gt_low) > eps && iters < 4096);
+
+  if (tx == 0) {
+    if (a.low_out) a.low_out[row] = low;
+    if (a.iters_out) a.iters_out[row] = iters;
+  }
+
+  // ---- emit: mask and / or ordered index list ----------------------------------------------
+  if (a.mask) {
+    uint8_t* dst = a.mask + (size_t)row * a.d;
+    const bool vec_ok = ((((uintptr_t)dst) & 3u) == 0);
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+      const uint32_t e0 = 4u * (uint32_t)(tx + THREADS * c);
+      if (vec_ok && e0 + 4 <= a.d) {
+        uint32_t w = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) w |= (x[4 * c + j] > low ? 1u : 0u) << (8 * j);
+        *(uint32_t*)(dst + e0) = w;
+      } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          if (e0 + j < a.d) dst[e0 + j] = (x[4 * c + j] > low) ? 1 : 0;
+      }
+    }
+  }
+  if (a.idx || a.count) {
+    int32_t* dst = a.idx ? a.idx + (size_t)row * a.idx_stride : nullptr;
+    const int32_t* pages = a.sel_pages ? a.sel_pages + (size_t)row * a.sel_stride : nullptr;
+    int base = 0;  // survivors emitted by earlier chunks (uniform)
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+      const uint32_t e0 = 4u * (uint32_t)(tx + THREADS * c);
+      bool k0 = x[4 * c + 0] > low, k1 = x[4 * c + 1] > low;
+      bool k2 = x[4 * c + 2] > low, k3 = x[4 * c + 3] > low;
+      const int mine = (int)k0 + (int)k1 + (int)k2 + (int)k3;
+      // inclusive scan of `mine` across the wave, in lane order
+      int scan = mine;
+      {
+        int t;
+        t = dpp<0x111>(0, scan); scan += t;                    // row_shr:1
+        t = dpp<0x112>(0, scan); scan += t;                    // row_shr:2
+        t = dpp<0x114>(0, scan); scan += t;                    // row_shr:4
+        t = dpp<0x118>(0, scan); scan += t;                    // row_shr:8
+        t = dpp<kDppBcast15, 0xA>(0, scan); scan += t;         // rows 1,3 += end of rows 0,2
+        t = dpp<kDppBcast31, 0xC>(0, scan); scan += t;         // rows 2,3 += end of row 1
+      }
+      const int wtot = __builtin_amdgcn_readlane(scan, 63);
+      if (NWAVES > 1) {
+        __syncthreads();  // previous chunk's readers are done with wave_tot
+        if (lane == 0) wave_tot[wave] = wtot;
+        __syncthreads();
+      }
+      int before = 0, total = wtot;
+      if (NWAVES > 1) {
+        total = 0;
+#pragma unroll
+        for (int w = 0; w < NWAVES; ++w) {
+          const int t = wave_tot[w];
+          before += (w < wave) ? t : 0;
+          total += t;
+        }
+      }
+      if (dst && mine) {
+        int pos = base + before + scan - mine;
+        const bool kk[4] = {k0, k1, k2, k3};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          if (kk[j]) {
+            const uint32_t e = e0 + j;
+            dst[pos++] = pages ? (pages[e >> 4] * TWL_PAGE + (int)(e & 15u)) : (int)e;
+          }
+        }
+      }
+      base += total;
+    }
+    if (tx == 0 && a.count) a.count[row] = base;
+  }
+}
+
+template <int DT, bool FUSED>
+static int launch_top_p(const TopPArgs& a, uint32_t rows, hipStream_t s) {
+  const uint32_t d = a.d;
+  if (d <= 1024) {
+    hipLaunchKernelGGL((top_p_kernel<DT, 256, 4, FUSED>), dim3(rows), dim3(256), 0, s, a);
+  } else if (d <= 2048) {
+    hipLaunchKernelGGL((top_p_kernel<DT, 512, 4, FUSED>), dim3(rows), dim3(512), 0, s, a);
+  } else if (d <= 4096) {
+    hipLaunchKernelGGL((top_p_kernel<DT, 1024, 4, FUSED>), dim3(rows), dim3(1024), 0, s, a);
+  } else if (d <= 8192) {
+    hipLaunchKernelGGL((top_p_kernel<DT, 1024, 8, FUSED>), dim3(rows), dim3(1024), 0, s, a);
+  } else if (d <= 16384) {
+    hipLaunchKernelGGL((top_p_kernel<DT, 1024, 16, FUSED>), dim3(rows), dim3(1024), 0, s, a);
+  } else {
+    hipLaunchKernelGGL((top_p_kernel<DT, 1024, 32, FUSED>), dim3(rows), dim3(1024), 0, s, a);
+  }
+  return hipGetLastError() == hipSuccess ? TWL_OK : TWL_ELAUNCH;
+}
+
+}  // namespace twl
+
+using twl::TopPArgs;
+
+static int check_top_p_common(const void* in, uint8_t* mask, int32_t* idx, int32_t* count,
+                              float p, const float* p_arr, uint32_t rows, uint32_t d,
+                              uint32_t idx_stride, int high_mode) {
+  if (!in) return TWL_ENULL;
+  if (!mask && !idx && !count) return TWL_ENULL;
+  if (idx && !count) return TWL_ENULL;
+  if (rows == 0 || d == 0 || d > TWL_MAX_CANDIDATES) return TWL_EINVAL;
+  if (idx && idx_stride < d) return TWL_EINVAL;
+  if (high_mode != TWL_HIGH_FIRST && high_mode != TWL_HIGH_MAX) return TWL_EINVAL;
+  if (!p_arr && !(p > 0.0f && p <= 1.0f)) return TWL_EINVAL;
+  return TWL_OK;
+}
+
+extern "C" int twl_top_p_f32(const float* probs, uint8_t* mask, int32_t* idx, int32_t* count,
+                             const float* p_arr, float p, uint32_t rows, uint32_t d,
+                             uint32_t idx_stride, int high_mode, float* low_out,
+                             int32_t* iters_out, void* stream) {
+  int rc = check_top_p_common(probs, mask, idx, count, p, p_arr, rows, d, idx_stride, high_mode);
+  if (rc != TWL_OK) return rc;
+  if (((uintptr_t)probs) & 3u) return TWL_EALIGN;
+  TopPArgs a{};
+  a.in = probs; a.in_stride = d; a.lens = nullptr; a.d = d; a.p_arr = p_arr; a.p = p;
+  a.high_mode = high_mode; a.mask = mask; a.idx = idx; a.idx_stride = idx_stride; a.count = count;
+  a.low_out = low_out; a.iters_out = iters_out;
+  return twl::launch_top_p<TWL_F32, false>(a, rows, (hipStream_t)stream);
+}
+
+extern "C" int twl_top_p_f16(const void* probs, int dtype, uint8_t* mask, int32_t* idx,
+                             int32_t* count, const float* p_arr, float p, uint32_t rows,
+                             uint32_t d, uint32_t idx_stride, int high_mode, float* low_out,
+                             int32_t* iters_out, void* stream) {
+  int rc = check_top_p_common(probs, mask, idx, count, p, p_arr, rows, d, idx_stride, high_mode);
+  if (rc != TWL_OK) return rc;
+  if (dtype != TWL_F16 && dtype != TWL_BF16) return TWL_EDTYPE;
+  if (((uintptr_t)probs) & 1u) return TWL_EALIGN;
+  TopPArgs a{};
+  a.in = probs; a.in_stride = d; a.lens = nullptr; a.d = d; a.p_arr = p_arr; a.p = p;
+  a.high_mode = high_mode; a.mask = mask; a.idx = idx; a.idx_stride = idx_stride; a.count = count;
+  a.low_out = low_out; a.iters_out = iters_out;
+  if (dtype == TWL_F16) return twl::launch_top_p<TWL_F16, false>(a, rows, (hipStream_t)stream);
+  return twl::launch_top_p<TWL_BF16, false>(a, rows, (hipStream_t)stream);
+}
+
+extern "C" int twl_softmax_top_p_f32(const float* scores, uint32_t score_stride,
+                                     const int32_t* lens, uint32_t rows, uint32_t d,
+                                     const float* p_arr, float p, int high_mode,
+                                     const int32_t* sel_pages, uint32_t sel_stride, int32_t* idx,
+                                     uint32_t idx_stride, int32_t* count, float* probs_out,
+                                     float* low_out, void* stream) {
+  int rc = check_top_p_common(scores, nullptr, idx, count, p, p_arr, rows, d, idx_stride, high_mode);
+  if (rc != TWL_OK) return rc;
+  if (score_stride < d) return TWL_EINVAL;
+  if (sel_pages && (uint64_t)sel_stride * TWL_PAGE < d) return TWL_EINVAL;
+  if (((uintptr_t)scores) & 3u) return TWL_EALIGN;
+  TopPArgs a{};
+  a.in = scores; a.in_stride = score_stride; a.lens = lens; a.d = d; a.p_arr = p_arr; a.p = p;
+  a.high_mode = high_mode; a.mask = nullptr; a.idx = idx; a.idx_stride = idx_stride;
+  a.count = count; a.sel_pages = sel_pages; a.sel_stride = sel_stride; a.probs_out = probs_out;
+  a.low_out = low_out;
+  return twl::launch_top_p<TWL_F32, true>(a, rows, (hipStream_t)stream);
+}

@@ -1,0 +1,133 @@
+// Device-side helpers shared by the kernels of libtwilight_hip (gfx950, wave64 only).
+#ifndef TWL_COMMON_H_
+#define TWL_COMMON_H_
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/twilight_hip.h"
+
+namespace twl {
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kWave = 64;
+
+__device__ __forceinline__ float as_f32(int v) { return __builtin_bit_cast(float, v); }
+__device__ __forceinline__ float as_f32(uint32_t v) { return __builtin_bit_cast(float, v); }
+__device__ __forceinline__ int as_i32(float v) { return __builtin_bit_cast(int, v); }
+__device__ __forceinline__ uint32_t as_u32(float v) { return __builtin_bit_cast(uint32_t, v); }
+
+__device__ __forceinline__ int lane_id() {
+  return __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+}
+
+// ---- 16-bit float conversions (exact widenings; narrowing is round-to-nearest-even) ----------
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return as_f32(b << 16); }
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+  uint32_t x = as_u32(f);
+  if ((x & 0x7FFFFFFFu) > 0x7F800000u) return (x >> 16) | 0x40u;
+  return (x + 0x7FFFu + ((x >> 16) & 1u)) >> 16;
+}
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t b) {
+  return (float)__builtin_bit_cast(_Float16, (uint16_t)b);
+}
+__device__ __forceinline__ uint32_t f32_to_f16_bits(float f) {
+  return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)f);
+}
+template <int DT>
+__device__ __forceinline__ float bits16_to_f32(uint32_t b) {
+  return DT == TWL_F16 ? f16_bits_to_f32(b) : bf16_bits_to_f32(b);
+}
+template <int DT>
+__device__ __forceinline__ uint32_t f32_to_bits16(float f) {
+  return DT == TWL_F16 ? f32_to_f16_bits(f) : f32_to_bf16_bits(f);
+}
+// round a float to the value set of element type DT (TWL_F32: identity)
+template <int DT>
+__device__ __forceinline__ float round_to(float f) {
+  if (DT == TWL_F16) return f16_bits_to_f32(f32_to_f16_bits(f));
+  if (DT == TWL_BF16) return bf16_bits_to_f32(f32_to_bf16_bits(f));
+  return f;
+}
+
+// ---- DPP data movement -----------------------------------------------------------------------
+// Lanes disabled by ROW_MASK / out-of-range sources receive `old`.
+template <int CTRL, int ROW_MASK = 0xF>
+__device__ __forceinline__ float dpp(float old, float v) {
+  return as_f32(__builtin_amdgcn_update_dpp(as_i32(old), as_i32(v), CTRL, ROW_MASK, 0xF, false));
+}
+template <int CTRL, int ROW_MASK = 0xF>
+__device__ __forceinline__ int dpp(int old, int v) {
+  return __builtin_amdgcn_update_dpp(old, v, CTRL, ROW_MASK, 0xF, false);
+}
+constexpr int kDppXor1 = 0xB1;        // quad_perm [1,0,3,2]
+constexpr int kDppXor2 = 0x4E;        // quad_perm [2,3,0,1]
+constexpr int kDppHalfMirror = 0x141; // lane i <-> 7-i inside each 8 lanes
+constexpr int kDppMirror = 0x140;     // lane i <-> 15-i inside each row of 16
+constexpr int kDppBcast15 = 0x142;    // lane 15 of each row -> next row
+constexpr int kDppBcast31 = 0x143;    // lane 31 -> rows 2 and 3
+
+struct OpSum {
+  static __device__ __forceinline__ float id() { return 0.0f; }
+  static __device__ __forceinline__ float ap(float a, float b) { return a + b; }
+};
+struct OpMax {
+  static __device__ __forceinline__ float id() { return -__builtin_inff(); }
+  static __device__ __forceinline__ float ap(float a, float b) { return fmaxf(a, b); }
+};
+struct OpMin {
+  static __device__ __forceinline__ float id() { return __builtin_inff(); }
+  static __device__ __forceinline__ float ap(float a, float b) { return fminf(a, b); }
+};
+
+// After this every lane of a quad holds the quad's reduction.
+template <class Op>
+__device__ __forceinline__ float quad_allreduce(float v) {
+  v = Op::ap(v, dpp<kDppXor1>(Op::id(), v));
+  v = Op::ap(v, dpp<kDppXor2>(Op::id(), v));
+  return v;
+}
+// After this every lane of a 16-lane row holds the row's reduction (fixed order: deterministic).
+template <class Op>
+__device__ __forceinline__ float row16_allreduce(float v) {
+  v = quad_allreduce<Op>(v);
+  v = Op::ap(v, dpp<kDppHalfMirror>(Op::id(), v));
+  v = Op::ap(v, dpp<kDppMirror>(Op::id(), v));
+  return v;
+}
+// Reduction over the 64 lanes, returned in every lane (wave-uniform value).
+template <class Op>
+__device__ __forceinline__ float wave_allreduce(float v) {
+  v = row16_allreduce<Op>(v);
+  v = Op::ap(v, dpp<kDppBcast15, 0xA>(Op::id(), v));  // rows 1,3 += rows 0,2
+  v = Op::ap(v, dpp<kDppBcast31, 0xC>(Op::id(), v));  // row 3 += rows 0,1
+  return as_f32(__builtin_amdgcn_readlane(as_i32(v), 63));
+}
+
+// Block-wide reduction through a caller-provided LDS slot array of `NWAVES` floats.
+// All threads receive the result. Callers alternate between two slot arrays (or put a barrier
+// between uses) so that a fast wave cannot overwrite values a slow wave still has to read.
+template <class Op, int NWAVES>
+__device__ __forceinline__ float block_allreduce(float v, float* slots) {
+  static_assert(NWAVES <= 16 && (NWAVES & (NWAVES - 1)) == 0, "NWAVES must be a power of 2 <= 16");
+  v = wave_allreduce<Op>(v);
+  if (NWAVES == 1) return v;
+  const int lane = lane_id();
+  const int wave = threadIdx.x / kWave;
+  if (lane == 0) slots[wave] = v;
+  __syncthreads();
+  float t = slots[lane & (NWAVES - 1)];
+  // lanes hold NWAVES distinct partials, repeated with period NWAVES inside each row of 16
+  if (NWAVES >= 2) t = Op::ap(t, dpp<kDppXor1>(Op::id(), t));
+  if (NWAVES >= 4) t = Op::ap(t, dpp<kDppXor2>(Op::id(), t));
+  if (NWAVES >= 8) t = Op::ap(t, dpp<kDppHalfMirror>(Op::id(), t));
+  if (NWAVES >= 16) t = Op::ap(t, dpp<kDppMirror>(Op::id(), t));
+  return t;
+}
+
+}  // namespace twl
+#endif  // TWL_COMMON_H_

@@ -1,0 +1,18 @@
+"""Op surface of the Select-then-Prune decode path.
+
+The first two names are the reference's own (twilight/kernel/__init__.py:1-3); the rest are the
+index-list / paged forms the decode layer needs, including the call shape of the INT4 GEMV the
+reference benchmarks (benchmark/efficiency/bench_gemv.py:445-454).
+"""
+from .sampling import (top_p_fp16_return_mask, top_p_fp32_return_mask, top_p_select,
+                       softmax_top_p)
+from .gemv import batched_sparse_gemv_int4_k, sparse_gemv_int4
+from .attention import sparse_paged_decode_attention
+from .quest import quest_num_pages, quest_select
+from .kv_shadow import dequant_int4, kv_shadow_build
+
+__all__ = [
+    "top_p_fp16_return_mask", "top_p_fp32_return_mask", "top_p_select", "softmax_top_p",
+    "batched_sparse_gemv_int4_k", "sparse_gemv_int4", "sparse_paged_decode_attention",
+    "quest_num_pages", "quest_select", "dequant_int4", "kv_shadow_build",
+]

@@ -1,0 +1,78 @@
+"""Sparse paged decode attention op (twilight/pyimpl/attention.py:188-190,299-306 over survivors)."""
+from __future__ import annotations
+
+import math
+from typing import Optional
+
+import torch
+
+from .. import _lib
+from ._check import (check_cuda, check_dim, check_dtype, check_input, check_same_device,
+                     dtype_code, ptr, stream_of)
+
+
+def _cache_strides(cache: torch.Tensor, name: str):
+    """``cache`` is a 4-D view [pages, 16, Hkv, 128] with a contiguous last dim (any page /
+    token / head strides: both NHD and HND storage work)."""
+    check_cuda(cache, name)
+    check_dim(4, cache, name)
+    if cache.size(1) != _lib.PAGE or cache.size(3) != _lib.HEAD_DIM:
+        raise RuntimeError(f"{name} must be viewed as [pages, 16, kv_heads, 128]")
+    if cache.stride(3) != 1:
+        raise RuntimeError(f"{name}: head_dim must be contiguous")
+    return cache.stride(0), cache.stride(1), cache.stride(2)
+
+
+def sparse_paged_decode_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                                  idx: torch.Tensor, count: torch.Tensor,
+                                  kv_page_indices: torch.Tensor, kv_page_indptr: torch.Tensor,
+                                  sm_scale: Optional[float] = None, return_lse: bool = False,
+                                  out: Optional[torch.Tensor] = None):
+    """Exact softmax attention of one decode token restricted to per-row survivor lists.
+
+    ``q`` [B,H,128] fp16/bf16; ``k_cache`` / ``v_cache`` [pages,16,Hkv,128] of the same dtype;
+    ``idx`` int32 [B,H,S] ascending logical token positions, ``count`` int32 [B,H]. Returns
+    ``out`` [B,H,128] in q's dtype (and ``lse`` fp32 [B,H] when asked). Probabilities are rounded
+    to q's dtype before the V product as at attention.py:302-304.
+    """
+    check_input(q, "q")
+    check_dim(3, q, "q")
+    B, H, D = q.shape
+    if D != _lib.HEAD_DIM:
+        raise RuntimeError(f"head_dim must be {_lib.HEAD_DIM}, got {D}")
+    ks = _cache_strides(k_cache, "k_cache")
+    vs = _cache_strides(v_cache, "v_cache")
+    if ks != vs or k_cache.shape != v_cache.shape:
+        raise RuntimeError("k_cache and v_cache must share shape and strides")
+    if k_cache.dtype != q.dtype or v_cache.dtype != q.dtype:
+        raise RuntimeError("q, k_cache and v_cache must share one dtype (float16 or bfloat16)")
+    Hkv = k_cache.size(2)
+    if H % Hkv != 0:
+        raise RuntimeError(f"num_q_heads {H} must be a multiple of num_kv_heads {Hkv}")
+    check_input(idx, "idx"); check_dtype(idx, torch.int32, "idx"); check_dim(3, idx, "idx")
+    check_input(count, "count"); check_dtype(count, torch.int32, "count")
+    if idx.size(0) != B or idx.size(1) != H or count.numel() != B * H:
+        raise RuntimeError("idx must be [B,H,S] and count [B,H]")
+    for name, t in (("kv_page_indices", kv_page_indices), ("kv_page_indptr", kv_page_indptr)):
+        check_input(t, name); check_dtype(t, torch.int32, name)
+    if kv_page_indptr.numel() != B + 1:
+        raise RuntimeError("kv_page_indptr must have B+1 elements")
+    check_same_device(q, ("k_cache", k_cache), ("v_cache", v_cache), ("idx", idx),
+                      ("count", count), ("kv_page_indices", kv_page_indices),
+                      ("kv_page_indptr", kv_page_indptr))
+    dev = q.device
+    with torch.cuda.device(dev):
+        if out is None:
+            out = torch.empty_like(q)
+        else:
+            check_input(out, "out")
+            if out.shape != q.shape or out.dtype != q.dtype:
+                raise RuntimeError("out must match q")
+        lse = torch.empty((B, H), dtype=torch.float32, device=dev) if return_lse else None
+        scale = 1.0 / math.sqrt(D) if sm_scale is None else float(sm_scale)
+        rc = _lib.lib().twl_sparse_attn(
+            ptr(q), ptr(out), dtype_code(q.dtype, "q"), ptr(k_cache), ptr(v_cache), ks[0], ks[1],
+            ks[2], ptr(idx), idx.size(2), ptr(count), ptr(kv_page_indices), ptr(kv_page_indptr),
+            B, H, Hkv, scale, ptr(lse), stream_of(q))
+    _lib.check(rc, "SparsePagedDecodeAttention")
+    return (out, lse) if return_lse else out

@@ -1,0 +1,131 @@
+"""INT4-K score GEMV ops (estimator of twilight/pyimpl/attention.py:252-255)."""
+from __future__ import annotations
+
+import math
+from typing import Optional
+
+import torch
+
+from .. import _lib
+from ._check import (check_dim, check_dtype, check_input, check_same_device, dtype_code, ptr,
+                     stream_of)
+
+
+def sparse_gemv_int4(q: torch.Tensor, k_int4: torch.Tensor, kv_page_indices: torch.Tensor,
+                     kv_page_indptr: torch.Tensor, kv_last_page_len: torch.Tensor,
+                     sel_pages: Optional[torch.Tensor] = None,
+                     sel_count: Optional[torch.Tensor] = None,
+                     max_pages: Optional[int] = None, sm_scale: Optional[float] = None,
+                     out: Optional[torch.Tensor] = None, out_count: Optional[torch.Tensor] = None):
+    """``scores[b,h,c] = sm_scale * q[b,h,:] . dequant(K_int4[candidate c])`` in fp32.
+
+    ``q`` [B,H,128] fp16/bf16; ``k_int4`` uint8 [pages, Hkv, 1280] INT4 shadow records;
+    the CSR page table of the batch; ``sel_pages`` int32 [B,H,S] per-row ascending logical page
+    lists with ``sel_count`` int32 [B,H] (both None: every page of the request, ``max_pages``
+    = the longest request's page count). Candidate slots past a request's length are ``-inf``.
+    Returns ``(scores fp32 [B,H,16*max_pages], cand_count int32 [B,H])``.
+    """
+    check_input(q, "q")
+    check_dim(3, q, "q")
+    B, H, D = q.shape
+    if D != _lib.HEAD_DIM:
+        raise RuntimeError(f"head_dim must be {_lib.HEAD_DIM}, got {D}")
+    check_input(k_int4, "k_int4")
+    check_dtype(k_int4, torch.uint8, "k_int4")
+    if k_int4.dim() != 3 or k_int4.size(2) != _lib.INT4_RECORD_BYTES:
+        raise RuntimeError("k_int4 must be uint8 [pages, kv_heads, 1280]")
+    Hkv = k_int4.size(1)
+    if H % Hkv != 0:
+        raise RuntimeError(f"num_q_heads {H} must be a multiple of num_kv_heads {Hkv}")
+    for name, t in (("kv_page_indices", kv_page_indices), ("kv_page_indptr", kv_page_indptr),
+                    ("kv_last_page_len", kv_last_page_len)):
+        check_input(t, name)
+        check_dtype(t, torch.int32, name)
+    if kv_page_indptr.numel() != B + 1 or kv_last_page_len.numel() != B:
+        raise RuntimeError("kv_page_indptr must have B+1 and kv_last_page_len B elements")
+    sel_stride = 0
+    if sel_pages is not None:
+        check_input(sel_pages, "sel_pages")
+        check_dtype(sel_pages, torch.int32, "sel_pages")
+        if sel_pages.dim() != 3 or sel_pages.size(0) != B or sel_pages.size(1) != H:
+            raise RuntimeError("sel_pages must be int32 [B, H, S]")
+        sel_stride = sel_pages.size(2)
+        if max_pages is None:
+            max_pages = sel_stride
+        if sel_count is not None:
+            check_input(sel_count, "sel_count")
+            check_dtype(sel_count, torch.int32, "sel_count")
+            if sel_count.numel() != B * H:
+                raise RuntimeError("sel_count must have B*H elements")
+    elif sel_count is not None:
+        raise RuntimeError("sel_count given without sel_pages")
+    if max_pages is None:
+        raise RuntimeError("max_pages is required when sel_pages is None")
+    check_same_device(q, ("k_int4", k_int4), ("kv_page_indices", kv_page_indices),
+                      ("kv_page_indptr", kv_page_indptr), ("kv_last_page_len", kv_last_page_len),
+                      ("sel_pages", sel_pages), ("sel_count", sel_count))
+    dev = q.device
+    M = max_pages * _lib.PAGE
+    with torch.cuda.device(dev):
+        if out is None:
+            out = torch.empty((B, H, M), dtype=torch.float32, device=dev)
+        else:
+            check_input(out, "out")
+            check_dtype(out, torch.float32, "out")
+            if out.dim() != 3 or out.size(0) != B or out.size(1) != H or out.size(2) < M:
+                raise RuntimeError("out must be fp32 [B, H, >= 16*max_pages]")
+        if out_count is None:
+            out_count = torch.empty((B, H), dtype=torch.int32, device=dev)
+        scale = 1.0 / math.sqrt(D) if sm_scale is None else float(sm_scale)
+        rc = _lib.lib().twl_gemv_int4(
+            ptr(q), dtype_code(q.dtype, "q"), ptr(out), out.size(2), ptr(out_count), ptr(k_int4),
+            ptr(sel_pages), ptr(sel_count), sel_stride, ptr(kv_page_indices), ptr(kv_page_indptr),
+            ptr(kv_last_page_len), B, H, Hkv, max_pages, scale, stream_of(q))
+    _lib.check(rc, "SparseGemvInt4")
+    return out, out_count
+
+
+def batched_sparse_gemv_int4_k(q: torch.Tensor, o: torch.Tensor, k_u8: torch.Tensor,
+                               quant_scales: torch.Tensor, quant_zeros: torch.Tensor,
+                               kv_page_indices: torch.Tensor, kv_page_indptr: torch.Tensor,
+                               kv_last_page_len: torch.Tensor,
+                               sm_scale: float = 1.0) -> None:
+    """Same call shape as ``ftka.cuda_ops.gemv.batched_sparse_gemv_int4_k`` at
+    benchmark/efficiency/bench_gemv.py:445-454 (tensors built at :390-443).
+
+    ``q`` fp16 [B,H,128]; ``o`` fp16 [B,H,N] filled in place; ``k_u8`` uint8
+    [max_pages, page_size, H, 64] (low nibble = even element); ``quant_scales`` / ``quant_zeros``
+    fp16 [max_pages, page_size, H] with dequant ``k*scale + zero`` (bench_gemv.py:181); one page
+    list per request shared by all heads. ``sm_scale`` defaults to 1 (the bench compares against
+    a plain ``q @ k``, bench_gemv.py:491).
+    """
+    check_input(q, "q"); check_dim(3, q, "q"); check_dtype(q, torch.float16, "q")
+    check_input(o, "o"); check_dim(3, o, "o"); check_dtype(o, torch.float16, "o")
+    check_input(k_u8, "k_cache"); check_dim(4, k_u8, "k_cache"); check_dtype(k_u8, torch.uint8, "k_cache")
+    B, H, D = q.shape
+    if D != _lib.HEAD_DIM or k_u8.size(3) != D // 2 or k_u8.size(2) != H:
+        raise RuntimeError("k_cache must be uint8 [max_pages, page_size, num_heads, 64]")
+    page_size = k_u8.size(1)
+    for name, t in (("quant_scales", quant_scales), ("quant_zeros", quant_zeros)):
+        check_input(t, name); check_dtype(t, torch.float16, name)
+        if tuple(t.shape) != tuple(k_u8.shape[:3]):
+            raise RuntimeError(f"{name} must be fp16 [max_pages, page_size, num_heads]")
+    for name, t in (("kv_page_indices", kv_page_indices), ("kv_page_indptr", kv_page_indptr),
+                    ("kv_last_page_len", kv_last_page_len)):
+        check_input(t, name); check_dtype(t, torch.int32, name)
+    if o.size(0) != B or o.size(1) != H:
+        raise RuntimeError("o must be fp16 [B, H, N]")
+    if kv_page_indptr.numel() != B + 1 or kv_last_page_len.numel() != B:
+        raise RuntimeError("kv_page_indptr must have B+1 and kv_last_page_len B elements")
+    check_same_device(q, ("o", o), ("k_cache", k_u8), ("quant_scales", quant_scales),
+                      ("quant_zeros", quant_zeros), ("kv_page_indices", kv_page_indices),
+                      ("kv_page_indptr", kv_page_indptr), ("kv_last_page_len", kv_last_page_len))
+    max_pages_per_req = o.size(2) // page_size
+    if max_pages_per_req == 0:
+        raise RuntimeError("o is shorter than one page")
+    with torch.cuda.device(q.device):
+        rc = _lib.lib().twl_gemv_int4_nhd(
+            ptr(q), ptr(o), o.size(2), ptr(k_u8), ptr(quant_scales), ptr(quant_zeros),
+            ptr(kv_page_indices), ptr(kv_page_indptr), ptr(kv_last_page_len), B, H, page_size,
+            max_pages_per_req, float(sm_scale), stream_of(q))
+    _lib.check(rc, "BatchedSparseGemvInt4K")

@@ -1,0 +1,65 @@
+"""KV-append ops: INT4 shadow + Quest metadata builder, and the INT4 unpacker used by tests."""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from .. import _lib
+from ._check import check_dtype, check_input, check_same_device, dtype_code, ptr, stream_of
+from .attention import _cache_strides
+
+
+def kv_shadow_build(k_cache: torch.Tensor, k_int4: Optional[torch.Tensor],
+                    meta: Optional[torch.Tensor], page_ids: Optional[torch.Tensor] = None,
+                    valid_len: Optional[torch.Tensor] = None) -> None:
+    """Quantise whole pages of ``k_cache`` [pages,16,Hkv,128] into ``k_int4`` uint8
+    [pages,Hkv,1280] (twilight/pyimpl/quantize.py:4-13 per group of 32, fp16 scale/zero) and
+    write their channel-wise min/max into ``meta`` uint8 [pages,Hkv,512]
+    (twilight/pyimpl/quest.py:68-74). ``page_ids`` int32 selects physical pages (default all);
+    ``valid_len`` int32 gives the valid tokens of each listed page (default 16)."""
+    ps, ts, hs = _cache_strides(k_cache, "k_cache")
+    Hkv = k_cache.size(2)
+    if k_int4 is None and meta is None:
+        raise RuntimeError("at least one of k_int4 / meta is required")
+    if k_int4 is not None:
+        check_input(k_int4, "k_int4"); check_dtype(k_int4, torch.uint8, "k_int4")
+        if k_int4.dim() != 3 or k_int4.size(1) != Hkv or k_int4.size(2) != _lib.INT4_RECORD_BYTES \
+                or k_int4.size(0) != k_cache.size(0):
+            raise RuntimeError("k_int4 must be uint8 [pages, kv_heads, 1280]")
+    if meta is not None:
+        check_input(meta, "meta"); check_dtype(meta, torch.uint8, "meta")
+        if meta.dim() != 3 or meta.size(1) != Hkv or meta.size(2) != _lib.META_RECORD_BYTES \
+                or meta.size(0) != k_cache.size(0):
+            raise RuntimeError("meta must be uint8 [pages, kv_heads, 512]")
+    n = k_cache.size(0)
+    if page_ids is not None:
+        check_input(page_ids, "page_ids"); check_dtype(page_ids, torch.int32, "page_ids")
+        n = page_ids.numel()
+    if valid_len is not None:
+        check_input(valid_len, "valid_len"); check_dtype(valid_len, torch.int32, "valid_len")
+        if valid_len.numel() != n:
+            raise RuntimeError("valid_len must have one entry per processed page")
+    check_same_device(k_cache, ("k_int4", k_int4), ("meta", meta), ("page_ids", page_ids),
+                      ("valid_len", valid_len))
+    if n == 0:
+        return
+    with torch.cuda.device(k_cache.device):
+        rc = _lib.lib().twl_kv_shadow_build(
+            ptr(k_cache), dtype_code(k_cache.dtype, "k_cache"), ps, ts, hs, ptr(page_ids),
+            ptr(valid_len), n, Hkv, ptr(k_int4), ptr(meta), stream_of(k_cache))
+    _lib.check(rc, "KvShadowBuild")
+
+
+def dequant_int4(k_int4: torch.Tensor) -> torch.Tensor:
+    """uint8 [pages,Hkv,1280] records -> fp32 [pages,Hkv,16,128] (nibble*scale + zero)."""
+    check_input(k_int4, "k_int4"); check_dtype(k_int4, torch.uint8, "k_int4")
+    if k_int4.dim() != 3 or k_int4.size(2) != _lib.INT4_RECORD_BYTES:
+        raise RuntimeError("k_int4 must be uint8 [pages, kv_heads, 1280]")
+    P, Hkv, _ = k_int4.shape
+    with torch.cuda.device(k_int4.device):
+        out = torch.empty((P, Hkv, _lib.PAGE, _lib.HEAD_DIM), dtype=torch.float32,
+                          device=k_int4.device)
+        rc = _lib.lib().twl_dequant_int4(ptr(k_int4), P * Hkv, ptr(out), stream_of(k_int4))
+    _lib.check(rc, "DequantInt4")
+    return out

@@ -1,0 +1,118 @@
+"""Host-side driver of one Select-then-Prune decode layer.
+
+Mirrors the decode branch of twilight/pyimpl/attention.py:188-306 (selector -> weight estimator
+-> weight pruner -> attention) with the configuration keys of benchmark/configs/*.json:
+``selector: {type: quest, token_budget, chunk_size}``, ``weight_estimator: {type: min_max_quant,
+quant_bit: 4}``, ``weight_pruner: {type: top_p, threshold}``. All buffers are allocated once; a
+step is a single call into ``twl_decode_layer`` which enqueues the kernels on the current stream.
+"""
+from __future__ import annotations
+
+import ctypes
+import math
+from typing import Optional
+
+import torch
+
+from . import _lib
+from .cache import PagedKVCache
+from .kernel._check import check_dim, check_input, dtype_code, ptr, stream_of
+from .kernel.quest import quest_num_pages
+
+
+def parse_sparse_config(cfg: dict) -> dict:
+    """Validate a reference-style algorithm config (twilight/pyimpl/attention.py:360-400) and
+    return the parameters of the path this package implements."""
+    sel = dict(cfg.get("selector", {}))
+    est = dict(cfg.get("weight_estimator", {}))
+    prn = dict(cfg.get("weight_pruner", {}))
+    if sel.get("type", "quest") != "quest":
+        raise RuntimeError(f"selector type {sel.get('type')!r} is not supported (only 'quest')")
+    if sel.get("chunk_size", _lib.PAGE) != _lib.PAGE:
+        raise RuntimeError(f"quest chunk_size must equal the page size {_lib.PAGE}")
+    if est.get("type", "min_max_quant") != "min_max_quant" or est.get("quant_bit", 4) != 4:
+        raise RuntimeError("weight_estimator must be {type: min_max_quant, quant_bit: 4}")
+    if prn.get("type", "top_p") != "top_p":
+        raise RuntimeError(f"weight_pruner type {prn.get('type')!r} is not supported (only 'top_p')")
+    if cfg.get("use_estimated_weights_in_attn", False):
+        raise RuntimeError("use_estimated_weights_in_attn=True is not supported")
+    return dict(token_budget=int(sel.get("token_budget", 8192)),
+                top_p=float(prn.get("threshold", 0.85)))
+
+
+class TwilightDecodeLayer:
+    """One attention layer's decode step over a :class:`PagedKVCache`."""
+
+    def __init__(self, cache: PagedKVCache, num_q_heads: int, token_budget: int = 8192,
+                 top_p: float = 0.85, high: str = "max", sm_scale: Optional[float] = None):
+        if num_q_heads % cache.num_kv_heads != 0:
+            raise RuntimeError("num_q_heads must be a multiple of the cache's kv heads")
+        if not (0.0 < top_p <= 1.0):
+            raise RuntimeError(f"top_p must be in (0, 1], got {top_p}")
+        if high not in ("first", "max"):
+            raise RuntimeError("high must be 'first' or 'max'")
+        self.cache, self.H = cache, num_q_heads
+        self.token_budget, self.top_p = int(token_budget), float(top_p)
+        self.high_mode = _lib.TWL_HIGH_FIRST if high == "first" else _lib.TWL_HIGH_MAX
+        self.sm_scale = 1.0 / math.sqrt(_lib.HEAD_DIM) if sm_scale is None else float(sm_scale)
+        self._alloc()
+
+    @classmethod
+    def from_config(cls, cache: PagedKVCache, num_q_heads: int, cfg: dict, **kw):
+        return cls(cache, num_q_heads, **parse_sparse_config(cfg), **kw)
+
+    def _alloc(self) -> None:
+        c = self.cache
+        B, H, dev = c.batch, self.H, c.device
+        self.k_pages = quest_num_pages(self.token_budget, c.max_pages_per_req)
+        M = self.k_pages * _lib.PAGE
+        if M > _lib.MAX_CANDIDATES:
+            raise RuntimeError(f"token budget {M} exceeds the supported maximum {_lib.MAX_CANDIDATES}")
+        i32, f32 = torch.int32, torch.float32
+        self.sel_pages = torch.zeros((B, H, self.k_pages), dtype=i32, device=dev)
+        self.sel_count = torch.zeros((B, H), dtype=i32, device=dev)
+        self.page_scores = torch.zeros((B, H, c.max_pages_per_req), dtype=f32, device=dev)
+        self.scores = torch.zeros((B, H, M), dtype=f32, device=dev)
+        self.cand_count = torch.zeros((B, H), dtype=i32, device=dev)
+        self.idx = torch.zeros((B, H, M), dtype=i32, device=dev)
+        self.count = torch.zeros((B, H), dtype=i32, device=dev)
+        self.out = torch.zeros((B, H, _lib.HEAD_DIM), dtype=c.dtype, device=dev)
+        self._shape = (B, c.max_pages_per_req)
+
+    def forward(self, q: torch.Tensor) -> torch.Tensor:
+        """``q`` [B, H, 128] in the cache dtype -> attention output [B, H, 128] (same buffer every
+        call). Intermediates stay readable as ``sel_pages/sel_count/scores/idx/count``."""
+        c = self.cache
+        check_input(q, "q")
+        check_dim(3, q, "q")
+        if (c.batch, c.max_pages_per_req) != self._shape:
+            self._alloc()
+        if tuple(q.shape) != (c.batch, self.H, _lib.HEAD_DIM) or q.dtype != c.dtype:
+            raise RuntimeError(f"q must be [{c.batch}, {self.H}, {_lib.HEAD_DIM}] of {c.dtype}")
+        if q.device != c.device:
+            raise RuntimeError(f"q must be on {c.device}")
+        ks = c.k_cache.stride()
+        a = _lib.LayerArgs()
+        a.q, a.dtype = ptr(q), dtype_code(q.dtype, "q")
+        a.k_cache, a.v_cache = ptr(c.k_cache), ptr(c.v_cache)
+        a.page_stride, a.token_stride, a.head_stride = ks[0], ks[1], ks[2]
+        a.k_int4, a.meta = ptr(c.k_int4), ptr(c.meta)
+        a.kv_page_indices, a.kv_page_indptr = ptr(c.kv_page_indices), ptr(c.kv_page_indptr)
+        a.kv_last_page_len = ptr(c.kv_last_page_len)
+        a.batch, a.num_q_heads, a.num_kv_heads = c.batch, self.H, c.num_kv_heads
+        a.max_pages_per_req, a.token_budget = c.max_pages_per_req, self.token_budget
+        a.top_p, a.high_mode, a.sm_scale = self.top_p, self.high_mode, self.sm_scale
+        a.sel_pages, a.sel_stride = ptr(self.sel_pages), self.sel_pages.size(2)
+        a.sel_count = ptr(self.sel_count)
+        a.page_scores, a.page_score_stride = ptr(self.page_scores), self.page_scores.size(2)
+        a.scores, a.score_stride = ptr(self.scores), self.scores.size(2)
+        a.cand_count = ptr(self.cand_count)
+        a.idx, a.idx_stride = ptr(self.idx), self.idx.size(2)
+        a.count = ptr(self.count)
+        a.out = ptr(self.out)
+        with torch.cuda.device(c.device):
+            rc = _lib.lib().twl_decode_layer(ctypes.byref(a), stream_of(q))
+        _lib.check(rc, "TwilightDecodeLayer")
+        return self.out
+
+    __call__ = forward
