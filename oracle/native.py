@@ -38,10 +38,10 @@ def lib() -> ctypes.CDLL:
         f32p = ctypes.POINTER(ctypes.c_float)
         i32p = ctypes.POINTER(ctypes.c_int32)
         L.twl_oracle_top_p_f32.argtypes = [f32p, u8p, f32p, ctypes.c_float, ctypes.c_uint32,
-                                           ctypes.c_uint32, ctypes.c_int, f32p, i32p]
+                                           ctypes.c_uint32, ctypes.c_int, f32p, i32p, f32p]
         L.twl_oracle_top_p_f32.restype = None
         L.twl_oracle_top_p_f16.argtypes = [u16p, ctypes.c_int, u8p, f32p, ctypes.c_float,
-                                           ctypes.c_uint32, ctypes.c_uint32, ctypes.c_int, f32p, i32p]
+                                           ctypes.c_uint32, ctypes.c_uint32, ctypes.c_int, f32p, i32p, f32p]
         L.twl_oracle_top_p_f16.restype = None
         L.twl_oracle_nucleus.argtypes = [f32p, ctypes.c_uint32, ctypes.c_double, u8p, f32p,
                                          ctypes.POINTER(ctypes.c_double)]
@@ -68,11 +68,13 @@ HIGH_FIRST = 0  # csrc/include/sampling.cuh:156-159 as written
 HIGH_MAX = 1    # paper Algorithm 1
 
 
-def top_p_mask_f32(probs: np.ndarray, p, high_mode: int = HIGH_FIRST):
+def top_p_mask_f32(probs: np.ndarray, p, high_mode: int = HIGH_FIRST, return_margin: bool = False):
     """csrc/include/sampling.cuh:156-231 on a [rows, d] fp32 array.
 
     ``p`` is a float or a per-row array (``top_p_arr``, sampling.cuh:125).
-    Returns ``(mask uint8 [rows,d], low float32 [rows], iters int32 [rows])``.
+    Returns ``(mask uint8 [rows,d], low float32 [rows], iters int32 [rows])``; with
+    ``return_margin`` also the smallest ``|S - p|`` met per row (a decision with a margin of a few
+    fp32 ulps may flip under another summation order).
     """
     probs = np.ascontiguousarray(probs, dtype=np.float32)
     assert probs.ndim == 2
@@ -80,6 +82,7 @@ def top_p_mask_f32(probs: np.ndarray, p, high_mode: int = HIGH_FIRST):
     mask = np.zeros((rows, d), dtype=np.uint8)
     low = np.zeros(rows, dtype=np.float32)
     iters = np.zeros(rows, dtype=np.int32)
+    margin = np.zeros(rows, dtype=np.float32)
     if isinstance(p, np.ndarray):
         p_arr = np.ascontiguousarray(p, dtype=np.float32)
         assert p_arr.shape == (rows,)
@@ -88,7 +91,9 @@ def top_p_mask_f32(probs: np.ndarray, p, high_mode: int = HIGH_FIRST):
         pp, pv = None, float(p)
     lib().twl_oracle_top_p_f32(_ptr(probs, ctypes.c_float), _ptr(mask, ctypes.c_uint8), pp, pv,
                                rows, d, int(high_mode), _ptr(low, ctypes.c_float),
-                               _ptr(iters, ctypes.c_int32))
+                               _ptr(iters, ctypes.c_int32), _ptr(margin, ctypes.c_float))
+    if return_margin:
+        return mask, low, iters, margin
     return mask, low, iters
 
 
@@ -106,7 +111,7 @@ def top_p_mask_f16(bits: np.ndarray, dtype: int, p, high_mode: int = HIGH_FIRST)
         pp, pv = None, float(p)
     lib().twl_oracle_top_p_f16(_ptr(bits, ctypes.c_uint16), int(dtype), _ptr(mask, ctypes.c_uint8),
                                pp, pv, rows, d, int(high_mode), _ptr(low, ctypes.c_float),
-                               _ptr(iters, ctypes.c_int32))
+                               _ptr(iters, ctypes.c_int32), None)
     return mask, low, iters
 
 

@@ -120,7 +120,7 @@ static float round_to(float v, int dtype) {
 /* One row of csrc/include/sampling.cuh:156-231. x[] already holds the row as floats (for 16-bit
  * inputs: the exact values of the 16-bit numbers). dtype selects the arithmetic of the pivots. */
 static void top_p_row(const float* x, uint32_t d, float p_in, int high_mode, int dtype,
-                      uint8_t* mask, float* low_out, int32_t* iters_out) {
+                      uint8_t* mask, float* low_out, int32_t* iters_out, float* margin_out) {
   float p = round_to(p_in, dtype); /* DType p = DType(top_p...)            sampling.cuh:125 */
   float low = 0.0f;                /*                                       sampling.cuh:159 */
   float high;
@@ -133,6 +133,7 @@ static void top_p_row(const float* x, uint32_t d, float p_in, int high_mode, int
   const float eps = round_to(1e-5f, dtype); /*                              sampling.cuh:162 */
   float min_gt_low, max_le_high;
   int32_t iters = 0;
+  double margin = 1e30; /* smallest |S - p| met: how close a decision came to a rounding flip */
   do {                                       /*                             sampling.cuh:171 */
     float mid = round_to((low + high) / 2.0f, dtype); /*                    sampling.cuh:173 */
     min_gt_low = high;                       /*                             sampling.cuh:174 */
@@ -144,7 +145,8 @@ static void top_p_row(const float* x, uint32_t d, float p_in, int high_mode, int
       if (v > low && v < min_gt_low) min_gt_low = v;          /* :184-186 */
       if (v <= high && v > max_le_high) max_le_high = v;      /* :187-189 */
     }
-    float s = (dtype == 2) ? (float)sum : (float)sum; /* fp32 partial sums for every dtype */
+    float s = (float)sum; /* fp32 partial sums for every dtype */
+    if (fabs(sum - (double)p) < margin) margin = fabs(sum - (double)p);
     if (s >= p) {                            /*                             sampling.cuh:211-213 */
       low = mid;
     } else {                                 /*                             sampling.cuh:214-216 */
@@ -158,29 +160,31 @@ static void top_p_row(const float* x, uint32_t d, float p_in, int high_mode, int
   }
   if (low_out) *low_out = low;
   if (iters_out) *iters_out = iters;
+  if (margin_out) *margin_out = (float)margin;
 }
 
 void twl_oracle_top_p_f32(const float* probs, uint8_t* mask, const float* p_arr, float p,
                           uint32_t rows, uint32_t d, int high_mode, float* low_out,
-                          int32_t* iters_out) {
+                          int32_t* iters_out, float* margin_out) {
   for (uint32_t r = 0; r < rows; ++r) {
     top_p_row(probs + (size_t)r * d, d, p_arr ? p_arr[r] : p, high_mode, 2,
               mask ? mask + (size_t)r * d : NULL, low_out ? low_out + r : NULL,
-              iters_out ? iters_out + r : NULL);
+              iters_out ? iters_out + r : NULL, margin_out ? margin_out + r : NULL);
   }
 }
 
 /* probs: 16-bit patterns, dtype 0 = fp16, 1 = bf16 */
 void twl_oracle_top_p_f16(const uint16_t* probs, int dtype, uint8_t* mask, const float* p_arr,
                           float p, uint32_t rows, uint32_t d, int high_mode, float* low_out,
-                          int32_t* iters_out) {
+                          int32_t* iters_out, float* margin_out) {
   float* x = (float*)malloc(sizeof(float) * (size_t)d);
   for (uint32_t r = 0; r < rows; ++r) {
     const uint16_t* src = probs + (size_t)r * d;
     for (uint32_t j = 0; j < d; ++j)
       x[j] = dtype == 0 ? f16_bits_to_f32(src[j]) : bf16_bits_to_f32(src[j]);
     top_p_row(x, d, p_arr ? p_arr[r] : p, high_mode, dtype, mask ? mask + (size_t)r * d : NULL,
-              low_out ? low_out + r : NULL, iters_out ? iters_out + r : NULL);
+              low_out ? low_out + r : NULL, iters_out ? iters_out + r : NULL,
+              margin_out ? margin_out + r : NULL);
   }
   free(x);
 }

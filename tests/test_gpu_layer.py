@@ -1,0 +1,114 @@
+"""End-to-end GPU parity of the decode layer (select -> INT4 estimate -> top-p -> attention)
+against the oracle's dense-masked restatement of twilight/pyimpl/attention.py:188-306."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import native
+from oracle import pyimpl_port as P
+from twilight_amd import synth
+from twilight_amd.cache import PagedKVCache
+from twilight_amd.layer import TwilightDecodeLayer
+from _checks import assert_scores_close, assert_top_p_parity
+
+pytestmark = pytest.mark.gpu
+
+
+def _lists_to_mask(idx, count, N):
+    rows = idx.shape[0]
+    m = np.zeros((rows, N), dtype=bool)
+    for r in range(rows):
+        m[r, idx[r, :count[r]]] = True
+    return m
+
+
+def _run_case(dev, B, H, Hkv, N, budget, p, dt, seed, shuffle=True, n_heavy=16):
+    q, k, v = synth.heavy_hitter_qkv(B, H, N, n_heavy=n_heavy, mass=0.6, seed=seed, dtype=dt)
+    group = H // Hkv
+    kk, vv = k[:, ::group].contiguous(), v[:, ::group].contiguous()        # one K/V per kv head
+    npg = (N + 15) // 16
+    perm = torch.randperm(B * npg, generator=torch.Generator().manual_seed(seed)) if shuffle else None
+    cache = PagedKVCache.from_dense(kk.to(dt), vv.to(dt), dev, page_perm=perm)
+    layer = TwilightDecodeLayer(cache, H, token_budget=budget, top_p=p, high="max")
+    out = layer(q[:, :, 0].to(dt).to(dev)).cpu().float()
+    krep = kk.repeat_interleave(group, dim=1)                               # attention.py:124-126
+    vrep = vv.repeat_interleave(group, dim=1)
+    ref = P.decode_layer_dense(q, krep, vrep, top_p=p, token_budget=budget if budget < N else None,
+                               high_mode=native.HIGH_MAX, quant="storage", prob_dtype=dt)
+    rows = B * H
+    # 1. selector: same pages (a page whose score ties the k-th within rounding may differ)
+    sel = layer.sel_pages.cpu().numpy().reshape(rows, -1)
+    selc = layer.sel_count.cpu().numpy().reshape(rows)
+    mask0 = ref["mask0"].reshape(rows, N).numpy()
+    same_sel = np.zeros(rows, dtype=bool)
+    for r in range(rows):
+        m = np.zeros(npg * 16, dtype=bool)
+        for pg in sel[r, :selc[r]]:
+            m[pg * 16:(pg + 1) * 16] = True
+        same_sel[r] = np.array_equal(m[:N], mask0[r])
+    assert same_sel.mean() >= 0.9, same_sel.mean()
+    # 2. estimator scores on the selected candidates (1e-3 relative)
+    scores = layer.scores.cpu().numpy().reshape(rows, -1)
+    est = ref["scores"].reshape(rows, N).double().numpy()
+    cand_tok = (sel[:, :, None] * 16 + np.arange(16)[None, None, :]).reshape(rows, -1)
+    for r in np.nonzero(same_sel)[0]:
+        n = selc[r] * 16
+        tok = cand_tok[r, :n]
+        inside = tok < N
+        assert_scores_close(scores[r, :n][inside][None], est[r, tok[inside]][None])
+        assert np.all(np.isneginf(scores[r, :n][~inside]))
+    # 3. pruned index lists (identical except within 1e-5 of the threshold; kept mass >= p)
+    idx = layer.idx.cpu().numpy().reshape(rows, -1)
+    cnt = layer.count.cpu().numpy().reshape(rows)
+    gm = _lists_to_mask(idx, cnt, N)
+    probs = ref["probs"].reshape(rows, N).numpy()
+    _, _, _, margin = native.top_p_mask_f32(probs, p, native.HIGH_MAX, return_margin=True)
+    ok = np.nonzero(same_sel)[0]
+    n_exact = assert_top_p_parity(probs[ok], p, gm[ok], ref["mask"].reshape(rows, N).numpy()[ok],
+                                  ref["low"][ok], margin[ok], margin_tol=5e-6)
+    assert n_exact >= 0.9 * len(ok)
+    # 4. attention: exact over the GPU's own survivors, and end to end against the oracle
+    tol = 1e-3 if dt == torch.float16 else 8e-3
+    own = P.masked_attention(q, krep, vrep, torch.from_numpy(gm).reshape(B, H, 1, N), prob_dtype=dt)
+    assert torch.allclose(out, own[:, :, 0], rtol=tol, atol=tol)
+    e2e = (out.reshape(rows, 128)[ok] - ref["out"].reshape(rows, 128)[ok]).abs().max().item()
+    assert e2e < 5 * tol, e2e
+    return layer, ref
+
+
+def test_cfg1_full_context(dev):
+    # BASELINE config 1: B=1, 32 heads MHA, D=128, N=4096, 16 heavy hitters with ~60 % of the mass,
+    # all tokens are candidates, p = 0.95
+    layer, ref = _run_case(dev, 1, 32, 32, 4096, 4096, 0.95, torch.float16, seed=0)
+    cnt = layer.count.cpu().float()
+    assert 16 <= cnt.min() and cnt.mean() < 4096 * 0.8
+
+
+@pytest.mark.parametrize("B,H,Hkv,N,budget,p,dt", [
+    (2, 8, 8, 2048, 512, 0.95, torch.float16),     # Longchat-7B shape in the small (MHA)
+    (2, 8, 2, 2048, 512, 0.90, torch.bfloat16),    # Llama-3-8B shape in the small (GQA 4:1, bf16)
+    (3, 4, 4, 1000, 250, 0.85, torch.float16),     # ragged: partial last page, budget not /16
+    (1, 4, 1, 100, 8192, 0.95, torch.float16),     # budget larger than the context
+])
+def test_small_layer_configs(dev, B, H, Hkv, N, budget, p, dt):
+    _run_case(dev, B, H, Hkv, N, budget, p, dt, seed=B * 100 + H, n_heavy=8)
+
+
+def test_decode_append_keeps_shadow_fresh(dev):
+    # append tokens one at a time (crossing a page boundary) and compare with a cache built at once
+    g = torch.Generator().manual_seed(0)
+    B, Hkv, N0, steps = 2, 2, 60, 9
+    k = torch.randn((B, Hkv, N0 + steps, 128), generator=g).half()
+    v = torch.randn((B, Hkv, N0 + steps, 128), generator=g).half()
+    cache = PagedKVCache.from_dense(k[:, :, :N0].contiguous(), v[:, :, :N0].contiguous(), dev,
+                                    spare_pages=4)
+    free = [8, 9, 10, 11]
+    for s in range(steps):
+        cache.append(k[:, :, N0 + s], v[:, :, N0 + s], free)
+    full = PagedKVCache.from_dense(k, v, dev)
+    q = torch.randn((B, 4, 128), generator=g).half().to(dev)
+    a = TwilightDecodeLayer(cache, 4, token_budget=32, top_p=0.9)
+    b = TwilightDecodeLayer(full, 4, token_budget=32, top_p=0.9)
+    oa, ob = a(q).clone(), b(q).clone()
+    assert torch.equal(a.sel_pages, b.sel_pages) and torch.equal(a.count, b.count)
+    assert torch.equal(oa, ob)

@@ -1,0 +1,164 @@
+"""GPU parity of the top-p pruner (through the C-ABI) against the oracle's restatement of
+csrc/include/sampling.cuh:156-231 and twilight/pyimpl/top_p.py:10-15."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import native
+from oracle import pyimpl_port as P
+from twilight_amd import synth
+import twilight_amd.kernel as K
+from _checks import assert_top_p_parity
+
+pytestmark = pytest.mark.gpu
+
+
+def _softmax(x):
+    return torch.softmax(x, dim=-1, dtype=torch.float32)
+
+
+@pytest.mark.parametrize("p", [0.85, 0.95])
+@pytest.mark.parametrize("first_is_max", [True, False])
+def test_mask_dropin_cfg3(dev, p, first_is_max):
+    # BASELINE config 3: [8, 32, 8192] Zipf-spiked rows
+    x = synth.topp_scores(8, 32, 8192, seed=0, first_is_max=first_is_max)
+    probs = _softmax(x).reshape(8, 32, 1, 8192)
+    pn = probs.reshape(256, 8192).numpy()
+    for high, mode in (("first", native.HIGH_FIRST), ("max", native.HIGH_MAX)):
+        om, ol, oi, og = native.top_p_mask_f32(pn, p, mode, return_margin=True)
+        idx, count, mask, low, iters = K.top_p_select(probs.to(dev), p, high=high,
+                                                      return_mask=True, return_stats=True)
+        gm = mask.cpu().numpy().reshape(256, 8192)
+        assert mask.dtype == torch.bool and mask.shape == probs.shape
+        n_exact = assert_top_p_parity(pn, p, gm, om, ol, og, gpu_low=low.cpu().numpy())
+        assert n_exact >= 250
+        ok = og >= 2e-6
+        assert np.array_equal(iters.cpu().numpy()[ok], oi[ok])
+        # index list == positions of the mask, ascending
+        cn = count.cpu().numpy().reshape(256)
+        ix = idx.cpu().numpy().reshape(256, 8192)
+        assert np.array_equal(cn, gm.sum(-1))
+        for r in range(256):
+            assert np.array_equal(ix[r, :cn[r]], np.nonzero(gm[r])[0])
+        # the reference entry point itself
+        m2 = K.top_p_fp32_return_mask(probs.to(dev), p, high=high)
+        assert torch.equal(m2, mask)
+
+
+@pytest.mark.parametrize("d", [1, 3, 17, 1000, 1024, 1025, 4097, 9000, 20000, 32768])
+def test_ragged_lengths(dev, d):
+    g = torch.Generator().manual_seed(d)
+    x = torch.randn((3, 2, d), generator=g) * 3
+    probs = _softmax(x).reshape(3, 2, 1, d)
+    pn = probs.reshape(6, d).numpy()
+    om, ol, oi, og = native.top_p_mask_f32(pn, 0.9, native.HIGH_MAX, return_margin=True)
+    idx, count, mask = K.top_p_select(probs.to(dev), 0.9, high="max", return_mask=True)
+    gm = mask.cpu().numpy().reshape(6, d)
+    assert_top_p_parity(pn, 0.9, gm, om, ol, og)
+    assert np.array_equal(count.cpu().numpy().reshape(6), gm.sum(-1))
+
+
+def test_per_row_p_and_degenerate_rows(dev):
+    d = 2048
+    g = torch.Generator().manual_seed(1)
+    probs = _softmax(torch.randn((2, 4, d), generator=g) * 4)
+    probs[0, 0] = 0; probs[0, 0, 77] = 1.0            # one-hot
+    probs[0, 1] = 1.0 / d                              # uniform: everything ties, all kept
+    probs[0, 2] = 0                                    # all zero: nothing kept
+    probs = probs.reshape(2, 4, 1, d).contiguous()
+    ps = torch.tensor([0.95, 0.5, 0.9, 0.3, 0.6, 0.85, 0.99, 1.0])
+    pn = probs.reshape(8, d).numpy()
+    om, ol, oi, og = native.top_p_mask_f32(pn, ps.numpy(), native.HIGH_MAX, return_margin=True)
+    mask = K.top_p_fp32_return_mask(probs.to(dev), ps.to(dev), high="max")
+    gm = mask.cpu().numpy().reshape(8, d)
+    assert gm[0].sum() == 1 and gm[0, 77] and gm[1].sum() == d and gm[2].sum() == 0
+    assert_top_p_parity(pn[3:], ps.numpy()[3:], gm[3:], om[3:], ol[3:], og[3:])
+
+
+def test_sink_quirk_first_mode(dev):
+    # probs[...,0] == 0 under high="first": the reference prunes nothing (mask = probs > 0)
+    g = torch.Generator().manual_seed(2)
+    probs = _softmax(torch.randn((1, 4, 1, 512), generator=g) * 3)
+    probs[..., 0] = 0
+    m = K.top_p_fp32_return_mask(probs.to(dev), 0.5, high="first")
+    assert torch.equal(m.cpu(), probs > 0)
+
+
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
+def test_16bit_entry(dev, dt):
+    # pivots live in the 16-bit type; partial sums are fp32 in both implementations
+    g = torch.Generator().manual_seed(3)
+    probs = _softmax(torch.randn((2, 8, 1, 3000), generator=g) * 4).to(dt)
+    bits = probs.view(torch.int16).numpy().view(np.uint16).reshape(16, 3000)
+    om, ol, _ = native.top_p_mask_f16(bits, 0 if dt == torch.float16 else 1, 0.9, native.HIGH_MAX)
+    m = K.top_p_fp16_return_mask(probs.to(dev), 0.9, high="max")
+    gm = m.cpu().numpy().reshape(16, 3000)
+    pf = probs.float().numpy().reshape(16, 3000)
+    same = (gm == om.astype(bool)).all(-1)
+    assert same.mean() >= 0.8
+    for r in np.nonzero(~same)[0]:   # a differing row still is a threshold set with mass >= p
+        assert pf[r][gm[r]].astype(np.float64).sum() >= 0.9 - 4e-3
+        assert pf[r][~gm[r]].max() <= pf[r][gm[r]].min()
+
+
+def test_fused_softmax_top_p_lists(dev):
+    # twilight/pyimpl/top_p.py:10-15 on candidate scores with -inf slots, ragged lens, page mapping
+    B, H, S = 2, 4, 40
+    M = S * 16
+    x = synth.topp_scores(B, H, M, seed=5, max_spikes=40)
+    lens = torch.tensor([[640, 600, 16, 333], [1, 640, 500, 48]], dtype=torch.int32)
+    x[0, 0, 5:9] = float("-inf")
+    g = torch.Generator().manual_seed(9)
+    sel = torch.stack([torch.sort(torch.randperm(200, generator=g)[:S]).values
+                       for _ in range(B * H)]).reshape(B, H, S).to(torch.int32)
+    xm = x.clone()
+    for b in range(B):
+        for h in range(H):
+            xm[b, h, lens[b, h]:] = float("-inf")
+    ref_in = xm.masked_fill(torch.isinf(xm), torch.finfo(torch.float32).min).reshape(B, H, 1, M)
+    om, oprobs, ol, _ = P.top_p_unnormalized(ref_in, 0.9, native.HIGH_MAX)
+    pn = oprobs.reshape(B * H, M).numpy()
+    _, _, _, og = native.top_p_mask_f32(pn, 0.9, native.HIGH_MAX, return_margin=True)
+    idx, count, probs, low = K.softmax_top_p(x.to(dev), 0.9, lens=lens.to(dev), sel_pages=sel.to(dev),
+                                             high="max", return_probs=True, return_low=True)
+    gp = probs.cpu().numpy().reshape(B * H, M)
+    for r in range(B * H):
+        n = int(lens.reshape(-1)[r])
+        np.testing.assert_allclose(gp[r, :n], pn[r, :n], rtol=2e-6, atol=1e-12)
+    cn = count.cpu().numpy().reshape(-1)
+    ix = idx.cpu().numpy().reshape(B * H, M)
+    gm = np.zeros((B * H, M), dtype=bool)
+    selr = sel.reshape(B * H, S).numpy()
+    for r in range(B * H):
+        toks = ix[r, :cn[r]]
+        assert np.all(np.diff(toks) > 0)
+        # invert the page mapping: token -> candidate position
+        pos = np.searchsorted(selr[r], toks // 16) * 16 + toks % 16
+        assert np.array_equal(selr[r][pos // 16] * 16 + pos % 16, toks)
+        gm[r, pos] = True
+    assert_top_p_parity(pn, 0.9, gm, om.reshape(B * H, M).numpy(), ol, og, margin_tol=5e-6)
+
+
+def test_repeatable(dev):
+    x = synth.topp_scores(2, 8, 8192, seed=11).to(dev)
+    a = K.softmax_top_p(x, 0.95, return_low=True)
+    b = K.softmax_top_p(x, 0.95, return_low=True)
+    assert torch.equal(a[1], b[1]) and torch.equal(a[2], b[2])
+    ca = a[1].reshape(-1).cpu()
+    ia, ib = a[0].reshape(16, -1).cpu(), b[0].reshape(16, -1).cpu()
+    for r in range(16):
+        assert torch.equal(ia[r, :ca[r]], ib[r, :ca[r]])
+
+
+def test_errors(dev):
+    p = torch.rand(2, 3, 1, 64, device=dev)
+    with pytest.raises(RuntimeError):
+        K.top_p_fp32_return_mask(p[..., ::2], 0.9)           # not contiguous
+    with pytest.raises(RuntimeError):
+        K.top_p_fp32_return_mask(p.reshape(6, 64), 0.9)       # not 4-D
+    with pytest.raises(RuntimeError):
+        K.top_p_fp32_return_mask(p.half(), 0.9)               # wrong dtype for the fp32 entry
+    with pytest.raises(RuntimeError):
+        K.top_p_fp32_return_mask(p, 1.5)
+    with pytest.raises(RuntimeError):
+        K.top_p_fp32_return_mask(p, torch.rand(5, device=dev))
