@@ -1,0 +1,230 @@
+#!/usr/bin/env python3
+"""Benchmark of the Select-then-Prune decode layer on one MI355X.
+
+A step is one pass of the hot path (Quest page selection -> INT4-K score GEMV -> softmax + top-p
+prune -> sparse paged attention) over one batch of synthetic decode queries, enqueued by a single
+``twl_decode_layer`` call with every input already resident in HBM.
+
+Workload (``config.workload``): the Longchat-7B-shaped layer of the reference's headline figure at
+the batch the target is quoted on — 32 MHA heads, head_dim 128, fp16 paged KV (page 16), batch 8,
+context 32768, Quest budget 8192, top-p 0.95.
+
+Prints ONE JSON line. ``value`` is microseconds per layer (lower is better). ``roofline`` is for
+the kernel with the largest HBM term (the Quest metadata stream); ``kernels`` lists every kernel of
+the layer with its algorithmic bytes, time and fraction of the 8 TB/s peak, and ``gemv_cfg2`` the
+stand-alone INT4 GEMV at 8 x 32 x 32768 candidates. ``cpu_baseline`` is the CPU oracle (a port of
+the reference's torch path) timed on this host on one of the 8 batch elements and scaled by 8.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+
+
+def _time_calls(fn, iters: int, warmup: int) -> float:
+    """Average microseconds per call of ``fn`` (which enqueues on the current stream), measured
+    with events on that stream around ``iters`` back-to-back calls."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1000.0 / iters
+
+
+def cpu_baseline(N: int, H: int, budget: int, top_p: float, batch_scale: int, seed: int = 0):
+    """Times the CPU oracle (torch fp32 + the C top-p restatement) on one batch element."""
+    from oracle import native, pyimpl_port as P
+    from twilight_amd import synth
+    threads = torch.get_num_threads()
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn((1, H, 1, 128), generator=g).half().float()
+    k = torch.randn((1, H, N, 128), generator=g).half().float()
+    v = torch.randn((1, H, N, 128), generator=g).half().float()
+    pos = torch.randint(0, N, (H, 24), generator=g)
+    for h in range(H):
+        k[0, h, pos[h]] += 0.9 * q[0, h, 0]
+    k = k.half().float()
+    # (A) as the reference does it: K is re-quantised inside every decode step
+    t0 = time.perf_counter()
+    ra = P.decode_layer_dense(q, k, v, top_p=top_p, token_budget=budget, high_mode=native.HIGH_MAX,
+                              quant="storage", prob_dtype=torch.float16)
+    ta = time.perf_counter() - t0
+    # (B) K quantised once on append, as the GPU path does
+    k_deq = torch.from_numpy(P.int4_quant_storage(k)[3])
+    t0 = time.perf_counter()
+    P.decode_layer_dense(q, k, v, top_p=top_p, token_budget=budget, high_mode=native.HIGH_MAX,
+                         k_deq=k_deq, prob_dtype=torch.float16)
+    tb = time.perf_counter() - t0
+    return {
+        "value": ta * 1e6 * batch_scale, "unit": "us/layer", "cores": threads, "kind": "port",
+        "value_k_prequantised": tb * 1e6 * batch_scale,
+        "sample": (f"1 of {batch_scale} batch elements (32 heads x {N} tokens, budget {budget}, "
+                   f"p {top_p}) through oracle.pyimpl_port.decode_layer_dense, one run each, "
+                   f"time x {batch_scale}; `value` re-quantises K every step like "
+                   "twilight/pyimpl/attention.py:247-251, `value_k_prequantised` does not; torch "
+                   f"uses {threads} threads, the C quantiser / top-p one"),
+        "survivors_mean": float(ra["mask"].sum(-1).float().mean()),
+    }
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--context", type=int, default=32768)
+    ap.add_argument("--budget", type=int, default=8192)
+    ap.add_argument("--top-p", type=float, default=0.95)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel breakdown")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this path has no multi-GPU part (every (batch, head) "
+              "row is independent); run with --gpus 1", file=sys.stderr)
+        return 2
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        return 2
+
+    from twilight_amd import _lib, build, synth
+    from twilight_amd.cache import PagedKVCache
+    from twilight_amd.layer import TwilightDecodeLayer
+    if not os.path.exists(build.LIB_PATH):
+        build.build_library()
+    L = _lib.lib()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    B, H, Hkv, N, D = args.batch, 32, 32, args.context, 128
+    npg = N // 16
+    dt = torch.float16
+
+    # ---- inputs, resident in HBM before anything is timed ----------------------------------
+    q, k, v, (ids, indptr, last) = synth.layer_inputs_device(B, H, Hkv, N, dt, dev, seed=0)
+    cache = PagedKVCache(B * npg, Hkv, dt, dev)
+    cache.k_cache, cache.v_cache = k, v
+    cache.set_page_table(ids, indptr, last)
+    cache.rebuild_shadow()
+    layer = TwilightDecodeLayer(cache, H, token_budget=args.budget, top_p=args.top_p, high="max")
+    torch.cuda.synchronize()
+
+    # ---- the timed region: K steps of the whole layer --------------------------------------
+    step = lambda: layer.forward(q)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    wall_us = (time.perf_counter() - t0) * 1e6 / args.steps
+    n_bar = float(layer.count.float().mean())
+    n_max = int(layer.count.max())
+    kp = layer.k_pages
+    M = kp * 16
+    rows = B * H
+
+    # ---- per-kernel times through the stand-alone entry points, same buffers ----------------
+    kernels = {}
+    stream = torch.cuda.current_stream().cuda_stream
+    p = lambda t: 0 if t is None else t.data_ptr()
+    ks = cache.k_cache.stride()
+    sm = 1.0 / math.sqrt(D)
+    if not args.no_kernels:
+        it, wu = max(args.steps, 50), 10
+        calls = {
+            "quest_score": (lambda: L.twl_quest_page_scores(
+                p(q), 0, p(cache.meta), p(cache.kv_page_indices), p(cache.kv_page_indptr), B, H, Hkv,
+                npg, p(layer.page_scores), npg, stream), rows * npg * (512 + 4) + rows * D * 2),
+            "quest_topk": (lambda: L.twl_quest_topk_pages(
+                p(layer.page_scores), npg, p(cache.kv_page_indptr), B, H, args.budget, npg,
+                p(layer.sel_pages), kp, p(layer.sel_count), stream), rows * (npg * 4 + kp * 4 + 4)),
+            "gemv_int4": (lambda: L.twl_gemv_int4(
+                p(q), 0, p(layer.scores), M, p(layer.cand_count), p(cache.k_int4), p(layer.sel_pages),
+                p(layer.sel_count), kp, p(cache.kv_page_indices), p(cache.kv_page_indptr),
+                p(cache.kv_last_page_len), B, H, Hkv, kp, sm, stream),
+                rows * M * (64 + 16 + 4) + rows * D * 2 + rows * kp * 8),
+            "softmax_top_p": (lambda: L.twl_softmax_top_p_f32(
+                p(layer.scores), M, p(layer.cand_count), rows, M, 0, args.top_p, 1, p(layer.sel_pages),
+                kp, p(layer.idx), M, p(layer.count), 0, 0, stream),
+                rows * M * 4 + int(rows * n_bar) * 4 + rows * 4),
+            "sparse_attn": (lambda: L.twl_sparse_attn(
+                p(q), p(layer.out), 0, p(cache.k_cache), p(cache.v_cache), ks[0], ks[1], ks[2],
+                p(layer.idx), M, p(layer.count), p(cache.kv_page_indices), p(cache.kv_page_indptr),
+                B, H, Hkv, sm, 0, p(layer.attn_workspace), layer.attn_workspace.numel(), stream),
+                int(rows * n_bar) * (2 * D * 2 + 4) + rows * D * 4),
+        }
+        for name, (fn, nbytes) in calls.items():
+            us = _time_calls(fn, it, wu)
+            kernels[name] = {"us": round(us, 2), "bytes": nbytes,
+                             "GBps": round(nbytes / us / 1e3, 1),
+                             "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+        layer.forward(q)  # leave the buffers as a whole step leaves them
+        torch.cuda.synchronize()
+
+    layer_bytes = sum(kv["bytes"] for kv in kernels.values()) if kernels else None
+    dom = kernels.get("quest_score")
+    roofline = None
+    if dom:
+        roofline = {"bound": "hbm", "kernel": "quest_score_kernel", "achieved": dom["GBps"],
+                    "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": dom["frac_of_hbm_peak"],
+                    "bytes_per_launch": dom["bytes"], "us_per_launch": dom["us"], "traffic": None}
+
+    # ---- stand-alone INT4 GEMV at 8 x 32 x 32768 candidates (all pages of every request) ----
+    gemv_cfg2 = None
+    if not args.no_kernels and B == 8 and N == 32768:
+        out2 = torch.empty((B, H, N), dtype=torch.float32, device=dev)
+        cnt2 = torch.empty((B, H), dtype=torch.int32, device=dev)
+        fn = lambda: L.twl_gemv_int4(p(q), 0, p(out2), N, p(cnt2), p(cache.k_int4), 0, 0, 0,
+                                     p(cache.kv_page_indices), p(cache.kv_page_indptr),
+                                     p(cache.kv_last_page_len), B, H, Hkv, npg, sm, stream)
+        us = _time_calls(fn, 50, 10)
+        nbytes = rows * N * 84 + rows * D * 2
+        gemv_cfg2 = {"us": round(us, 2), "bytes": nbytes, "GBps": round(nbytes / us / 1e3, 1),
+                     "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
+                     "workload": "INT4 GEMV alone, B=8 H=32 D=128, 32768 candidates per head, "
+                                 "shuffled pages"}
+        del out2
+
+    cpu = None
+    if not args.no_cpu_baseline:
+        cpu = cpu_baseline(N, H, args.budget, args.top_p, B)
+
+    line = {
+        "metric": "us/decode-layer at 32k ctx (select+prune+attn)",
+        "value": round(wall_us, 2), "unit": "us", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(wall_us / 1e3, 5), "higher_is_better": False,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": f"Select-then-Prune decode layer, Longchat-7B shape: B={B}, 32 MHA "
+                               f"heads, head_dim 128, fp16 paged KV (page 16), context {N}, Quest "
+                               f"budget {args.budget}, INT4 K estimate (group 32), top-p "
+                               f"{args.top_p}",
+                   "batch": B, "context": N, "budget": args.budget, "top_p": args.top_p,
+                   "survivors_mean": round(n_bar, 1), "survivors_max": n_max},
+        "layer_bytes": layer_bytes,
+        "layer_frac_of_hbm_peak": (round(layer_bytes / wall_us / 1e3 / HBM_PEAK_GBS, 4)
+                                   if layer_bytes else None),
+        "roofline": roofline, "kernels": kernels, "gemv_cfg2": gemv_cfg2, "cpu_baseline": cpu,
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -149,13 +149,20 @@ int twl_gemv_int4_nhd(const void* q, void* o, uint32_t o_stride, const uint8_t* 
  * [rows] receives log(sum exp(logit)) of the row.
  * k_cache / v_cache: element type kv_dtype (TWL_F16 / TWL_BF16, must equal q's type); element
  * (page, token, kv_head, d) lives at page*page_stride + token*token_stride + kv_head*head_stride + d.
+ * Rows longer than 128 survivors are split over several workgroups that meet in `workspace`
+ * (256-byte aligned, at least twl_sparse_attn_workspace_bytes(rows, idx_stride) bytes). Its first
+ * rows*4 bytes are ticket counters that must be zero before the first call; every call leaves
+ * them zero again. Two calls that share a workspace must not overlap in time. In a split row the
+ * softmax weights are not rounded to the q dtype before the V product (the partial sums are
+ * merged in fp32); a row of at most 128 survivors follows the reference rounding exactly.
  * ------------------------------------------------------------------------------------------- */
+uint64_t twl_sparse_attn_workspace_bytes(uint32_t rows, uint32_t idx_stride);
 int twl_sparse_attn(const void* q, void* out, int dtype, const void* k_cache, const void* v_cache,
                     uint64_t page_stride, uint64_t token_stride, uint64_t head_stride,
                     const int32_t* idx, uint32_t idx_stride, const int32_t* count,
                     const int32_t* kv_page_indices, const int32_t* kv_page_indptr, uint32_t batch,
                     uint32_t num_q_heads, uint32_t num_kv_heads, float sm_scale, float* lse_out,
-                    void* stream);
+                    void* workspace, uint64_t workspace_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Quest page selector: page score + top-k pages per row.
@@ -171,6 +178,17 @@ int twl_quest_select(const void* q, int q_dtype, const void* meta, const int32_t
                      uint32_t num_kv_heads, uint32_t token_budget, uint32_t max_pages_per_req,
                      int32_t* sel_pages, uint32_t sel_stride, int32_t* sel_count,
                      float* page_scores, uint32_t score_stride, void* stream);
+/* The two kernels of twl_quest_select as separate calls: page scores only (quest.py:36-84), and
+ * top-k page selection over given scores (quest.py:93-122). */
+int twl_quest_page_scores(const void* q, int q_dtype, const void* meta,
+                          const int32_t* kv_page_indices, const int32_t* kv_page_indptr,
+                          uint32_t batch, uint32_t num_q_heads, uint32_t num_kv_heads,
+                          uint32_t max_pages_per_req, float* page_scores, uint32_t score_stride,
+                          void* stream);
+int twl_quest_topk_pages(const float* page_scores, uint32_t score_stride,
+                         const int32_t* kv_page_indptr, uint32_t batch, uint32_t num_q_heads,
+                         uint32_t token_budget, uint32_t max_pages_per_req, int32_t* sel_pages,
+                         uint32_t sel_stride, int32_t* sel_count, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * KV-append side: build the INT4 shadow and the Quest metadata of whole pages from the paged K.
@@ -223,6 +241,7 @@ typedef struct twl_layer_args {
   int32_t* cand_count;                       /* [rows] */
   int32_t* idx;        uint32_t idx_stride;  /* [rows, idx_stride], >= 16 * selected pages */
   int32_t* count;                            /* [rows] */
+  void* attn_workspace; uint64_t attn_workspace_bytes; /* see twl_sparse_attn */
   /* output */
   void* out;                /* [batch, num_q_heads, 128], dtype */
 } twl_layer_args;

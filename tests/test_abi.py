@@ -16,7 +16,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 def test_header_symbols_are_exported(hip_lib):
     hdr = open(os.path.join(ROOT, "include", "twilight_hip.h")).read()
     declared = set(re.findall(r"\b(twl_[a-z0-9_]+)\s*\(", hdr))
-    declared -= {"twl_top_p_"}  # no partial names
+    declared -= {"twl_top_p_"}  # a prefix used in a comment, not a symbol
     assert declared == set(_lib.EXPORTS)
     for name in declared:
         assert hasattr(hip_lib, name), name
@@ -73,12 +73,18 @@ def test_c_level_validation_without_gpu(hip_lib):
     assert L.twl_gemv_int4(fake, 0, fake, 16, 0, fake, 0, 0, 0, fake, fake, fake, 1, 3, 2, 1, 1.0, 0) == -2
     assert L.twl_gemv_int4(fake, 0, fake, 8, 0, fake, 0, 0, 0, fake, fake, fake, 1, 1, 1, 1, 1.0, 0) == -2
     assert L.twl_gemv_int4(fake + 4, 0, fake, 16, 0, fake, 0, 0, 0, fake, fake, fake, 1, 1, 1, 1, 1.0, 0) == -4
+    ws = L.twl_sparse_attn_workspace_bytes(1, 8)
+    assert ws == 256 + 130 * 4 and L.twl_sparse_attn_workspace_bytes(256, 8192) == 1024 + 256 * 64 * 520
     assert L.twl_sparse_attn(fake, fake, 0, fake, fake, 4096, 256, 128, 0, 8, fake, fake, fake,
-                             1, 1, 1, 1.0, 0, 0) == -1
+                             1, 1, 1, 1.0, 0, fake, ws, 0) == -1
     assert L.twl_sparse_attn(fake, fake, 0, fake, fake, 4096, 256, 130, fake, 8, fake, fake, fake,
-                             1, 1, 1, 1.0, 0, 0) == -4
+                             1, 1, 1, 1.0, 0, fake, ws, 0) == -4
     assert L.twl_sparse_attn(fake, fake, 0, fake, fake, 4096, 256, 128, fake, 0, fake, fake, fake,
-                             1, 1, 1, 1.0, 0, 0) == -2
+                             1, 1, 1, 1.0, 0, fake, ws, 0) == -2
+    assert L.twl_sparse_attn(fake, fake, 0, fake, fake, 4096, 256, 128, fake, 8, fake, fake, fake,
+                             1, 1, 1, 1.0, 0, fake, ws - 1, 0) == -2      # workspace too small
+    assert L.twl_sparse_attn(fake, fake, 0, fake, fake, 4096, 256, 128, fake, 8, fake, fake, fake,
+                             1, 1, 1, 1.0, 0, 0, ws, 0) == -1             # workspace NULL
     assert L.twl_quest_select(fake, 0, fake, fake, fake, 1, 1, 1, 0, 4, fake, 4, fake, fake, 4, 0) == -2
     assert L.twl_quest_select(fake, 0, fake, fake, fake, 1, 1, 1, 64, 4, fake, 2, fake, fake, 4, 0) == -2
     assert L.twl_kv_shadow_build(fake, 0, 4096, 256, 128, 0, 0, 1, 1, 0, 0, 0) == -1

@@ -108,3 +108,28 @@ def test_sparse_attention_hnd_layout_view(dev):
     b = K.sparse_paged_decode_attention(q, k_hnd, v_hnd, idx, cnt, cache.kv_page_indices,
                                         cache.kv_page_indptr)
     assert torch.equal(a, b)
+
+
+def test_sparse_attention_split_rows_share_a_workspace(dev):
+    # rows of 1..3000 survivors (1 to 24 chunks of 128), two calls in a row on one workspace:
+    # the ticket counters must come back to zero and both results must match the reference
+    B, H, N = 1, 8, 3000
+    g = torch.Generator().manual_seed(8)
+    q = torch.randn((B, H, 1, 128), generator=g).half()
+    k = torch.randn((B, H, N, 128), generator=g).half()
+    v = torch.randn((B, H, N, 128), generator=g).half()
+    cache = PagedKVCache.from_dense(k, v, dev, page_perm=torch.randperm(188, generator=g))
+    ws = torch.zeros(K.attention_workspace_bytes(B * H, N), dtype=torch.uint8, device=dev)
+    for trial, lens in enumerate(([1, 127, 128, 129, 256, 257, 1000, 3000], [3000, 5, 640, 128, 2, 1999, 384, 129])):
+        mask = torch.zeros((B, H, 1, N), dtype=torch.bool)
+        for h, n in enumerate(lens):
+            mask[0, h, 0, torch.randperm(N, generator=g)[:n]] = True
+        idx, count = P.mask_to_lists(mask)
+        out = K.sparse_paged_decode_attention(
+            q[:, :, 0].contiguous().to(dev), cache.k_cache, cache.v_cache,
+            torch.from_numpy(np.maximum(idx, 0)).reshape(B, H, N).to(dev),
+            torch.from_numpy(count).reshape(B, H).to(dev), cache.kv_page_indices,
+            cache.kv_page_indptr, workspace=ws)
+        ref = P.masked_attention(q.float(), k.float(), v.float(), mask, prob_dtype=torch.float16)[:, :, 0]
+        assert torch.allclose(out.cpu().float(), ref, rtol=1e-3, atol=1e-3), trial
+        assert int(ws[:B * H * 4].view(torch.int32).abs().sum()) == 0

@@ -24,7 +24,7 @@ MAX_CANDIDATES = 32768
 EXPORTS = (
     "twl_strerror", "twl_abi_version", "twl_device_count", "twl_top_p_f32", "twl_top_p_f16",
     "twl_softmax_top_p_f32", "twl_gemv_int4", "twl_gemv_int4_nhd", "twl_sparse_attn",
-    "twl_quest_select", "twl_kv_shadow_build", "twl_dequant_int4", "twl_decode_layer",
+    "twl_sparse_attn_workspace_bytes", "twl_quest_select", "twl_quest_page_scores", "twl_quest_topk_pages", "twl_kv_shadow_build", "twl_dequant_int4", "twl_decode_layer",
 )
 
 
@@ -45,6 +45,7 @@ class LayerArgs(ctypes.Structure):
         ("cand_count", c_void_p),
         ("idx", c_void_p), ("idx_stride", c_uint32),
         ("count", c_void_p),
+        ("attn_workspace", c_void_p), ("attn_workspace_bytes", c_uint64),
         ("out", c_void_p),
     ]
 
@@ -75,15 +76,19 @@ def lib() -> ctypes.CDLL:
                                 u32, f32, vp]
     L.twl_gemv_int4_nhd.argtypes = [vp, vp, u32, vp, vp, vp, vp, vp, vp, u32, u32, u32, u32, f32, vp]
     L.twl_sparse_attn.argtypes = [vp, vp, i32, vp, vp, u64, u64, u64, vp, u32, vp, vp, vp, u32, u32,
-                                  u32, f32, vp, vp]
+                                  u32, f32, vp, vp, u64, vp]
+    L.twl_sparse_attn_workspace_bytes.argtypes = [u32, u32]
     L.twl_quest_select.argtypes = [vp, i32, vp, vp, vp, u32, u32, u32, u32, u32, vp, u32, vp, vp,
                                    u32, vp]
+    L.twl_quest_page_scores.argtypes = [vp, i32, vp, vp, vp, u32, u32, u32, u32, vp, u32, vp]
+    L.twl_quest_topk_pages.argtypes = [vp, u32, vp, u32, u32, u32, u32, vp, u32, vp, vp]
     L.twl_kv_shadow_build.argtypes = [vp, i32, u64, u64, u64, vp, vp, u32, u32, vp, vp, vp]
     L.twl_dequant_int4.argtypes = [vp, u32, vp, vp]
     L.twl_decode_layer.argtypes = [POINTER(LayerArgs), vp]
     for name in EXPORTS:
-        if name != "twl_strerror":
+        if name not in ("twl_strerror", "twl_sparse_attn_workspace_bytes"):
             getattr(L, name).restype = c_int
+    L.twl_sparse_attn_workspace_bytes.restype = c_uint64
     _lib = L
     return L
 

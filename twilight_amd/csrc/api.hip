@@ -68,5 +68,6 @@ extern "C" int twl_decode_layer(const twl_layer_args* a, void* stream) {
   return twl_sparse_attn(a->q, a->out, a->dtype, a->k_cache, a->v_cache, a->page_stride,
                          a->token_stride, a->head_stride, a->idx, a->idx_stride, a->count,
                          a->kv_page_indices, a->kv_page_indptr, a->batch, a->num_q_heads,
-                         a->num_kv_heads, a->sm_scale, nullptr, stream);
+                         a->num_kv_heads, a->sm_scale, nullptr, a->attn_workspace,
+                         a->attn_workspace_bytes, stream);
 }

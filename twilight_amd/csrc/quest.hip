@@ -123,18 +123,6 @@ __device__ __forceinline__ uint32_t order_key(float f) {
   return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 
-// inclusive scan of an int across the 64 lanes, in lane order
-__device__ __forceinline__ int wave_inclusive_scan(int v) {
-  int t;
-  t = dpp<0x111>(0, v); v += t;
-  t = dpp<0x112>(0, v); v += t;
-  t = dpp<0x114>(0, v); v += t;
-  t = dpp<0x118>(0, v); v += t;
-  t = dpp<kDppBcast15, 0xA>(0, v); v += t;
-  t = dpp<kDppBcast31, 0xC>(0, v); v += t;
-  return v;
-}
-
 // Thread t holds pages [t*VPT, (t+1)*VPT) of the row.
 template <int THREADS, int VPT>
 __global__ __launch_bounds__(THREADS) void quest_select_kernel(QuestSelectArgs a) {
@@ -238,18 +226,56 @@ __global__ __launch_bounds__(THREADS) void quest_select_kernel(QuestSelectArgs a
 
 }  // namespace twl
 
-extern "C" int twl_quest_select(const void* q, int q_dtype, const void* meta,
-                                const int32_t* kv_page_indices, const int32_t* kv_page_indptr,
-                                uint32_t batch, uint32_t num_q_heads, uint32_t num_kv_heads,
-                                uint32_t token_budget, uint32_t max_pages_per_req,
-                                int32_t* sel_pages, uint32_t sel_stride, int32_t* sel_count,
-                                float* page_scores, uint32_t score_stride, void* stream) {
-  if (!q || !meta || !kv_page_indices || !kv_page_indptr || !sel_pages || !sel_count ||
-      !page_scores)
-    return TWL_ENULL;
+static int check_quest_common(const void* q, int q_dtype, const void* meta,
+                              const int32_t* kv_page_indices, const int32_t* kv_page_indptr,
+                              uint32_t batch, uint32_t num_q_heads, uint32_t num_kv_heads,
+                              uint32_t max_pages_per_req, const float* page_scores,
+                              uint32_t score_stride) {
+  if (!q || !meta || !kv_page_indices || !kv_page_indptr || !page_scores) return TWL_ENULL;
   if (q_dtype != TWL_F16 && q_dtype != TWL_BF16) return TWL_EDTYPE;
   if (batch == 0 || num_q_heads == 0 || num_kv_heads == 0 || num_q_heads % num_kv_heads != 0)
     return TWL_EINVAL;
+  if (max_pages_per_req == 0 || max_pages_per_req > 16384 || score_stride < max_pages_per_req)
+    return TWL_EINVAL;
+  if ((uint64_t)batch * num_q_heads > 65535u) return TWL_EINVAL;
+  if ((((uintptr_t)q) & 7u) || (((uintptr_t)meta) & 15u) || (((uintptr_t)page_scores) & 3u))
+    return TWL_EALIGN;
+  return TWL_OK;
+}
+
+extern "C" int twl_quest_page_scores(const void* q, int q_dtype, const void* meta,
+                                     const int32_t* kv_page_indices,
+                                     const int32_t* kv_page_indptr, uint32_t batch,
+                                     uint32_t num_q_heads, uint32_t num_kv_heads,
+                                     uint32_t max_pages_per_req, float* page_scores,
+                                     uint32_t score_stride, void* stream) {
+  int rc = check_quest_common(q, q_dtype, meta, kv_page_indices, kv_page_indptr, batch,
+                              num_q_heads, num_kv_heads, max_pages_per_req, page_scores,
+                              score_stride);
+  if (rc != TWL_OK) return rc;
+  twl::QuestScoreArgs sa{};
+  sa.q = q; sa.meta = (const uint8_t*)meta; sa.kv_page_indices = kv_page_indices;
+  sa.kv_page_indptr = kv_page_indptr; sa.num_q_heads = num_q_heads; sa.num_kv_heads = num_kv_heads;
+  sa.max_pages = max_pages_per_req;
+  sa.page_scores = page_scores; sa.score_stride = score_stride;
+  dim3 grid((max_pages_per_req + twl::kQsPagesPerBlock - 1) / twl::kQsPagesPerBlock,
+            batch * num_q_heads);
+  if (q_dtype == TWL_F16)
+    hipLaunchKernelGGL((twl::quest_score_kernel<TWL_F16>), grid, dim3(twl::kQsThreads), 0,
+                       (hipStream_t)stream, sa);
+  else
+    hipLaunchKernelGGL((twl::quest_score_kernel<TWL_BF16>), grid, dim3(twl::kQsThreads), 0,
+                       (hipStream_t)stream, sa);
+  return hipGetLastError() == hipSuccess ? TWL_OK : TWL_ELAUNCH;
+}
+
+extern "C" int twl_quest_topk_pages(const float* page_scores, uint32_t score_stride,
+                                    const int32_t* kv_page_indptr, uint32_t batch,
+                                    uint32_t num_q_heads, uint32_t token_budget,
+                                    uint32_t max_pages_per_req, int32_t* sel_pages,
+                                    uint32_t sel_stride, int32_t* sel_count, void* stream) {
+  if (!page_scores || !kv_page_indptr || !sel_pages || !sel_count) return TWL_ENULL;
+  if (batch == 0 || num_q_heads == 0) return TWL_EINVAL;
   if (max_pages_per_req == 0 || max_pages_per_req > 16384 || score_stride < max_pages_per_req)
     return TWL_EINVAL;
   if (token_budget == 0) return TWL_EINVAL;
@@ -260,26 +286,13 @@ extern "C" int twl_quest_select(const void* q, int q_dtype, const void* meta,
     if (sel_stride < k) return TWL_EINVAL;
   }
   if ((uint64_t)batch * num_q_heads > 65535u) return TWL_EINVAL;
-  if ((((uintptr_t)q) & 7u) || (((uintptr_t)meta) & 15u) || (((uintptr_t)page_scores) & 3u))
-    return TWL_EALIGN;
+  if (((uintptr_t)page_scores) & 3u) return TWL_EALIGN;
   hipStream_t s = (hipStream_t)stream;
   const uint32_t rows = batch * num_q_heads;
-  twl::QuestScoreArgs sa{};
-  sa.q = q; sa.meta = (const uint8_t*)meta; sa.kv_page_indices = kv_page_indices;
-  sa.kv_page_indptr = kv_page_indptr; sa.num_q_heads = num_q_heads; sa.num_kv_heads = num_kv_heads;
-  sa.max_pages = max_pages_per_req;
-  sa.page_scores = page_scores; sa.score_stride = score_stride;
-  dim3 grid((max_pages_per_req + twl::kQsPagesPerBlock - 1) / twl::kQsPagesPerBlock, rows);
-  if (q_dtype == TWL_F16)
-    hipLaunchKernelGGL((twl::quest_score_kernel<TWL_F16>), grid, dim3(twl::kQsThreads), 0, s, sa);
-  else
-    hipLaunchKernelGGL((twl::quest_score_kernel<TWL_BF16>), grid, dim3(twl::kQsThreads), 0, s, sa);
-  if (hipGetLastError() != hipSuccess) return TWL_ELAUNCH;
-
   twl::QuestSelectArgs ta{};
   ta.page_scores = page_scores; ta.score_stride = score_stride; ta.kv_page_indptr = kv_page_indptr;
-  ta.num_q_heads = num_q_heads; ta.max_pages = max_pages_per_req; ta.token_budget = token_budget; ta.sel_pages = sel_pages;
-  ta.sel_stride = sel_stride; ta.sel_count = sel_count;
+  ta.num_q_heads = num_q_heads; ta.max_pages = max_pages_per_req; ta.token_budget = token_budget;
+  ta.sel_pages = sel_pages; ta.sel_stride = sel_stride; ta.sel_count = sel_count;
   const uint32_t n = max_pages_per_req;
   if (n <= 512)
     hipLaunchKernelGGL((twl::quest_select_kernel<256, 2>), dim3(rows), dim3(256), 0, s, ta);
@@ -292,4 +305,27 @@ extern "C" int twl_quest_select(const void* q, int q_dtype, const void* meta,
   else
     hipLaunchKernelGGL((twl::quest_select_kernel<1024, 16>), dim3(rows), dim3(1024), 0, s, ta);
   return hipGetLastError() == hipSuccess ? TWL_OK : TWL_ELAUNCH;
+}
+
+extern "C" int twl_quest_select(const void* q, int q_dtype, const void* meta,
+                                const int32_t* kv_page_indices, const int32_t* kv_page_indptr,
+                                uint32_t batch, uint32_t num_q_heads, uint32_t num_kv_heads,
+                                uint32_t token_budget, uint32_t max_pages_per_req,
+                                int32_t* sel_pages, uint32_t sel_stride, int32_t* sel_count,
+                                float* page_scores, uint32_t score_stride, void* stream) {
+  if (!sel_pages || !sel_count) return TWL_ENULL;
+  if (token_budget == 0) return TWL_EINVAL;
+  {
+    uint64_t k = (token_budget / TWL_PAGE ? token_budget / TWL_PAGE : 1) +
+                 (token_budget % TWL_PAGE ? 1 : 0);
+    if (k > max_pages_per_req) k = max_pages_per_req;
+    if (sel_stride < k) return TWL_EINVAL;
+  }
+  int rc = twl_quest_page_scores(q, q_dtype, meta, kv_page_indices, kv_page_indptr, batch,
+                                 num_q_heads, num_kv_heads, max_pages_per_req, page_scores,
+                                 score_stride, stream);
+  if (rc != TWL_OK) return rc;
+  return twl_quest_topk_pages(page_scores, score_stride, kv_page_indptr, batch, num_q_heads,
+                              token_budget, max_pages_per_req, sel_pages, sel_stride, sel_count,
+                              stream);
 }

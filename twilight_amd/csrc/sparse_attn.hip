@@ -1,15 +1,22 @@
 // Sparse paged decode attention over per-row survivor lists.
 //
 // Restates the masked softmax.V of twilight/pyimpl/attention.py:188-190,299-306 restricted to the
-// surviving tokens: logits = sm_scale * q.K in fp32, fp32 softmax over the survivors,
-// probabilities rounded to the q dtype (attention.py:302-304), fp32 accumulation of p.V, output
-// rounded to the q dtype.
+// surviving tokens: logits = sm_scale * q.K in fp32, fp32 softmax over the survivors, fp32
+// accumulation of p.V, output rounded to the q dtype.
 //
-// One workgroup (4 wavefronts) per (batch, head) row — after pruning a row keeps tens to a few
-// hundred tokens, so rows are short and many. 16 lanes share a token: each lane owns 8 of the
-// 128 head dims (one 16-byte load from K, one from V), a wavefront covers 4 tokens per step and
-// the workgroup 16. Logits are staged in LDS so that the softmax normaliser is known before any
-// probability is rounded, exactly as the reference does.
+// After pruning a row keeps tens to a few hundred tokens, with a long tail of rows that keep
+// thousands, so the work is split by tokens, not by rows: workgroup (s, row) owns survivors
+// [128 s, 128 s + 128) of its row and exits at once when the row is shorter (split-K across CUs).
+// Inside a workgroup (4 wavefronts) 16 lanes share a token: each lane owns 8 of the 128 head dims,
+// i.e. one 16-byte load from K and one from V; token addresses are resolved once into LDS and then
+// all K and V loads of the chunk are issued before any arithmetic, so a chunk costs about one HBM
+// round trip.
+//   - A row that fits one chunk is finished in place: probabilities are normalised and rounded to
+//     the q dtype before the V product, exactly as attention.py:302-304 does.
+//   - A longer row leaves (max, sum, unnormalised acc[128]) per chunk in the workspace; the chunk
+//     that finishes last (ticket counter) merges them FlashDecoding-style. There the weights
+//     stay in fp32 (no intermediate rounding to the q dtype): the difference is below the output
+//     rounding.
 #include "twl_common.h"
 
 namespace twl {
@@ -28,13 +35,18 @@ struct AttnArgs {
   uint32_t num_q_heads, num_kv_heads;
   float sm_scale;
   float* lse_out;
-  uint32_t lds_tokens;  // capacity of the logit staging area
+  int32_t* tickets;   // [rows], zero between calls
+  float* partials;    // [rows, max_splits, kAttnPartial]
+  uint32_t max_splits;
+  uint32_t rows;
+  uint32_t pool;      // workgroups that serve chunks 1.. of long rows
 };
 
 constexpr int kAttnThreads = 256;
 constexpr int kAttnWaves = kAttnThreads / kWave;
-constexpr int kAttnTokPerStep = 4 * kAttnWaves;  // 16
-constexpr int kAttnUnroll = 4;
+constexpr int kAttnChunk = 128;                        // survivors per workgroup
+constexpr int kAttnSteps = kAttnChunk / (4 * kAttnWaves);  // 8 tokens per lane-group
+constexpr int kAttnPartial = TWL_HEAD_DIM + 2;         // m, l, acc[128]
 
 template <int DT>
 __device__ __forceinline__ void unpack8(const u32x4& v, float* f) {
@@ -46,130 +58,258 @@ __device__ __forceinline__ void unpack8(const u32x4& v, float* f) {
   }
 }
 
-template <int DT>
-__global__ __launch_bounds__(kAttnThreads) void sparse_attn_kernel(AttnArgs a) {
-  extern __shared__ float lds[];  // [lds_tokens] logits, then probabilities
-  __shared__ float red[2][16];
-  __shared__ float oacc[kAttnWaves][TWL_HEAD_DIM];
+struct AttnSmem {
+  int slot_id[kAttnChunk];      // physical token slot = page * 16 + slot
+  float w[kAttnChunk];          // logits, then weights
+  float red[2][16];
+  float oacc[4 * kAttnWaves][TWL_HEAD_DIM];
+  int is_last;
+};
 
-  const uint32_t row = blockIdx.x;
+// One chunk (survivors [128*split, 128*split+128) of `row`, which has n > 128*split survivors).
+// Called by all threads of the workgroup.
+template <int DT>
+__device__ __forceinline__ void attn_chunk(const AttnArgs& a, AttnSmem& sm, uint32_t row,
+                                           int split, int n) {
+  int (&slot_id)[kAttnChunk] = sm.slot_id;
+  float (&w)[kAttnChunk] = sm.w;
+  float (&red)[2][16] = sm.red;
+  float (&oacc)[4 * kAttnWaves][TWL_HEAD_DIM] = sm.oacc;
+  int& is_last = sm.is_last;
+  const int j0 = split * kAttnChunk;
+  const int tx = threadIdx.x;
+  uint16_t* orow = (uint16_t*)a.out + (size_t)row * TWL_HEAD_DIM;
+  const int cn = min(kAttnChunk, n - j0);            // survivors of this chunk
+  const int n_splits = (n + kAttnChunk - 1) / kAttnChunk;
+
   const uint32_t b = row / a.num_q_heads;
   const uint32_t h = row - b * a.num_q_heads;
   const uint32_t kvh = h / (a.num_q_heads / a.num_kv_heads);
-  const int tx = threadIdx.x;
   const int lane = lane_id();
   const int wave = tx / kWave;
   const int sub = lane & 15;   // which 8 dims
-  const int slot = lane >> 4;  // which of the wave's 4 tokens
-  const int n = min(max(a.count[row], 0), (int)min(a.idx_stride, a.lds_tokens));
-  uint16_t* orow = (uint16_t*)a.out + (size_t)row * TWL_HEAD_DIM;
+  const int grp = lane >> 4;   // which of the wave's 4 concurrent tokens
 
-  if (n == 0) {
-    if (tx < TWL_HEAD_DIM) orow[tx] = 0;
-    if (tx == 0 && a.lse_out) a.lse_out[row] = -__builtin_inff();
-    return;
+  // ---- resolve token addresses once ---------------------------------------------------------
+  if (tx < kAttnChunk) {
+    int sid = 0;
+    if (tx < cn) {
+      const int tok = a.idx[(size_t)row * a.idx_stride + j0 + tx];
+      sid = a.kv_page_indices[a.kv_page_indptr[b] + (tok >> 4)] * TWL_PAGE + (tok & 15);
+    }
+    slot_id[tx] = sid;
   }
-
   float qf[8];
   {
     u32x4 v = *(const u32x4*)((const uint16_t*)a.q + (size_t)row * TWL_HEAD_DIM + 8 * sub);
     unpack8<DT>(v, qf);
   }
-  const int32_t* irow = a.idx + (size_t)row * a.idx_stride;
-  const int32_t* ptab = a.kv_page_indices + a.kv_page_indptr[b];
+  __syncthreads();
+
+  // ---- issue every K and V load of the chunk -------------------------------------------------
   const size_t head_off = (size_t)kvh * a.head_stride + 8 * sub;
   const uint16_t* kc = (const uint16_t*)a.k_cache;
   const uint16_t* vc = (const uint16_t*)a.v_cache;
+  u32x4 kreg[kAttnSteps], vreg[kAttnSteps];
+  int tloc[kAttnSteps];
+#pragma unroll
+  for (int i = 0; i < kAttnSteps; ++i) {
+    const int t = i * (4 * kAttnWaves) + wave * 4 + grp;  // local token of this lane group
+    tloc[i] = t;
+    const int sid = slot_id[min(t, cn - 1)];
+    const size_t off = (size_t)(sid >> 4) * a.page_stride + (size_t)(sid & 15) * a.token_stride +
+                       head_off;
+    kreg[i] = *(const u32x4*)(kc + off);
+  }
+#pragma unroll
+  for (int i = 0; i < kAttnSteps; ++i) {
+    const int sid = slot_id[min(tloc[i], cn - 1)];
+    const size_t off = (size_t)(sid >> 4) * a.page_stride + (size_t)(sid & 15) * a.token_stride +
+                       head_off;
+    vreg[i] = *(const u32x4*)(vc + off);
+  }
 
-  // ---- phase 1: logits -> LDS -------------------------------------------------------------
+  // ---- logits -------------------------------------------------------------------------------
   float wmax = -__builtin_inff();
-  for (int j0 = 0; j0 < n; j0 += kAttnTokPerStep * kAttnUnroll) {
-    u32x4 kv[kAttnUnroll];
-    int jj[kAttnUnroll];
 #pragma unroll
-    for (int u = 0; u < kAttnUnroll; ++u) {
-      const int j = j0 + u * kAttnTokPerStep + wave * 4 + slot;
-      jj[u] = j;
-      const int tok = irow[min(j, n - 1)];
-      const size_t off = (size_t)ptab[tok >> 4] * a.page_stride +
-                         (size_t)(tok & 15) * a.token_stride + head_off;
-      kv[u] = *(const u32x4*)(kc + off);
-    }
+  for (int i = 0; i < kAttnSteps; ++i) {
+    float kf[8];
+    unpack8<DT>(kreg[i], kf);
+    float acc = 0.0f;
 #pragma unroll
-    for (int u = 0; u < kAttnUnroll; ++u) {
-      float kf[8];
-      unpack8<DT>(kv[u], kf);
-      float acc = 0.0f;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) acc = fmaf(qf[i], kf[i], acc);
-      acc = row16_allreduce<OpSum>(acc) * a.sm_scale;
-      if (jj[u] < n) {
-        wmax = fmaxf(wmax, acc);
-        if (sub == 0) lds[jj[u]] = acc;
-      }
+    for (int d = 0; d < 8; ++d) acc = fmaf(qf[d], kf[d], acc);
+    acc = row16_allreduce<OpSum>(acc) * a.sm_scale;
+    if (tloc[i] < cn) {
+      wmax = fmaxf(wmax, acc);
+      if (sub == 0) w[tloc[i]] = acc;
     }
   }
-  const float m = block_allreduce<OpMax, kAttnWaves>(wmax, red[0]);  // barrier inside: LDS visible
+  const float m = block_allreduce<OpMax, kAttnWaves>(wmax, red[0]);  // barrier: w[] visible
 
-  // ---- phase 2: normaliser, probabilities rounded to the q dtype ---------------------------
+  // ---- weights ------------------------------------------------------------------------------
   float z = 0.0f;
-  for (int j = tx; j < n; j += kAttnThreads) {
-    const float e = expf(lds[j] - m);
-    lds[j] = e;
-    z += e;
+  float e = 0.0f;
+  if (tx < cn) {
+    e = expf(w[tx] - m);
+    z = e;
   }
   z = block_allreduce<OpSum, kAttnWaves>(z, red[1]);
-  if (tx == 0 && a.lse_out) a.lse_out[row] = m + logf(z);
-  for (int j = tx; j < n; j += kAttnThreads) lds[j] = round_to<DT>(lds[j] / z);
+  const bool single = (n_splits == 1);
+  if (tx < cn) w[tx] = single ? round_to<DT>(e / z) : e;
   __syncthreads();
 
-  // ---- phase 3: out = sum_j p_j * V_j -------------------------------------------------------
+  // ---- acc = sum_t w_t * V_t ----------------------------------------------------------------
   float acc[8];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
-  for (int j0 = 0; j0 < n; j0 += kAttnTokPerStep * kAttnUnroll) {
-    u32x4 vv[kAttnUnroll];
-    float pj[kAttnUnroll];
+  for (int d = 0; d < 8; ++d) acc[d] = 0.0f;
 #pragma unroll
-    for (int u = 0; u < kAttnUnroll; ++u) {
-      const int j = j0 + u * kAttnTokPerStep + wave * 4 + slot;
-      const int jc = min(j, n - 1);
-      const int tok = irow[jc];
-      const size_t off = (size_t)ptab[tok >> 4] * a.page_stride +
-                         (size_t)(tok & 15) * a.token_stride + head_off;
-      vv[u] = *(const u32x4*)(vc + off);
-      pj[u] = (j < n) ? lds[jc] : 0.0f;
-    }
+  for (int i = 0; i < kAttnSteps; ++i) {
+    const float wt = (tloc[i] < cn) ? w[tloc[i]] : 0.0f;
+    float vf[8];
+    unpack8<DT>(vreg[i], vf);
 #pragma unroll
-    for (int u = 0; u < kAttnUnroll; ++u) {
-      float vf[8];
-      unpack8<DT>(vv[u], vf);
-#pragma unroll
-      for (int i = 0; i < 8; ++i) acc[i] = fmaf(pj[u], vf[i], acc[i]);
-    }
+    for (int d = 0; d < 8; ++d) acc[d] = fmaf(wt, vf[d], acc[d]);
   }
-  // fold the 4 token slots of the wave (lanes l, l^16, l^32, l^48), then the 4 waves
+  // fold the 16 lane groups (4 per wave x 4 waves) through LDS
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    float v = acc[i];
-    v += __shfl_xor(v, 16, kWave);
-    v += __shfl_xor(v, 32, kWave);
-    acc[i] = v;
+  for (int d = 0; d < 8; ++d) oacc[wave * 4 + grp][8 * sub + d] = acc[d];
+  __syncthreads();
+  float o = 0.0f;
+  if (tx < TWL_HEAD_DIM) {
+#pragma unroll
+    for (int gi = 0; gi < 4 * kAttnWaves; ++gi) o += oacc[gi][tx];
   }
-  if (slot == 0) {
-#pragma unroll
-    for (int i = 0; i < 8; ++i) oacc[wave][8 * sub + i] = acc[i];
+
+  if (single) {
+    if (tx < TWL_HEAD_DIM) orow[tx] = (uint16_t)f32_to_bits16<DT>(o);
+    if (tx == 0 && a.lse_out) a.lse_out[row] = m + logf(z);
+    return;
+  }
+
+  // ---- split row: publish the partial, the last chunk to finish merges -------------------------
+  // The chunks of a row run on different XCDs, whose L2 caches are not coherent with each other
+  // inside a kernel. Partials therefore travel as device-scope relaxed atomics (write-through
+  // stores, cache-bypassing loads) ordered by the barrier's wait for outstanding stores and by the
+  // ticket increment; no cache-wide write-back / invalidate fence is needed.
+  float* part = a.partials + ((size_t)row * a.max_splits + split) * kAttnPartial;
+  if (tx < TWL_HEAD_DIM)
+    __hip_atomic_store(part + 2 + tx, o, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (tx == 0) {
+    __hip_atomic_store(part + 0, m, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(part + 1, z, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  __builtin_amdgcn_s_waitcnt(0);  // every counter to zero: this thread's stores have been acknowledged
+  __syncthreads();
+  if (tx == 0) {
+    const int ticket =
+        __hip_atomic_fetch_add(&a.tickets[row], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    is_last = (ticket == n_splits - 1);
   }
   __syncthreads();
-  if (tx < TWL_HEAD_DIM) {
-    float v = 0.0f;
+  if (!is_last) return;
+  // The partials are read back with device-scope loads that bypass this XCD's caches.
+  const float* prow = a.partials + (size_t)row * a.max_splits * kAttnPartial;
+  float* fm = &oacc[0][0];   // [n_splits <= 256] chunk maxima, then rescale factors
+  float* fl = &oacc[2][0];   // [n_splits] chunk sums
+  float lm = -__builtin_inff();
+  for (int s = tx; s < n_splits; s += kAttnThreads) {
+    const float ms = __hip_atomic_load(prow + (size_t)s * kAttnPartial, __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+    const float ls = __hip_atomic_load(prow + (size_t)s * kAttnPartial + 1, __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+    fm[s] = ms;
+    fl[s] = ls;
+    lm = fmaxf(lm, ms);
+  }
+  const float gm = block_allreduce<OpMax, kAttnWaves>(lm, red[0]);
+  float lsum = 0.0f;
+  for (int s = tx; s < n_splits; s += kAttnThreads) {
+    const float f = expf(fm[s] - gm);
+    fm[s] = f;
+    lsum = fmaf(fl[s], f, lsum);
+  }
+  const float gl = block_allreduce<OpSum, kAttnWaves>(lsum, red[1]);  // barrier: factors visible
+  const int d = tx & (TWL_HEAD_DIM - 1), half = tx >> 7;
+  float go = 0.0f;
+#pragma unroll 4
+  for (int s = half; s < n_splits; s += 2)
+    go = fmaf(__hip_atomic_load(prow + (size_t)s * kAttnPartial + 2 + d, __ATOMIC_RELAXED,
+                                __HIP_MEMORY_SCOPE_AGENT), fm[s], go);
+  if (half == 1) oacc[8][d] = go;
+  __syncthreads();
+  if (half == 0) go += oacc[8][d];
+  if (tx < TWL_HEAD_DIM) orow[tx] = (uint16_t)f32_to_bits16<DT>(go / gl);
+  if (tx == 0) {
+    if (a.lse_out) a.lse_out[row] = gm + logf(gl);
+    // ready for the next call
+    __hip_atomic_store(&a.tickets[row], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
+// Workgroup g < rows serves chunk 0 of row g. The remaining `pool` workgroups serve the chunks
+// 1.. of rows with more than 128 survivors: pool workgroup j takes overflow chunks j, j+pool, ...
+// in row-major order, locating each with a block-wide prefix sum over the rows' chunk counts
+// (a few KB from L2), so a launch never contains more than rows + pool workgroups however long
+// the longest row is.
+template <int DT>
+__global__ __launch_bounds__(kAttnThreads) void sparse_attn_kernel(AttnArgs a) {
+  __shared__ AttnSmem sm;
+  __shared__ int wave_tot[kAttnWaves];
+  __shared__ int found[3];  // row, split, n
+  const int tx = threadIdx.x;
+  if (blockIdx.x < a.rows) {
+    const uint32_t row = blockIdx.x;
+    const int n = min(max(a.count[row], 0), (int)a.idx_stride);
+    if (n == 0) {
+      if (tx < TWL_HEAD_DIM) ((uint16_t*)a.out)[(size_t)row * TWL_HEAD_DIM + tx] = 0;
+      if (tx == 0 && a.lse_out) a.lse_out[row] = -__builtin_inff();
+      return;
+    }
+    attn_chunk<DT>(a, sm, row, 0, n);
+    return;
+  }
+  const int lane = lane_id();
+  const int wave = tx / kWave;
+  for (int j = (int)(blockIdx.x - a.rows);; j += (int)a.pool) {
+    int running = 0;   // overflow chunks of the rows before the current tile
+    bool hit = false;
+    for (uint32_t r0 = 0; r0 < a.rows && !hit; r0 += kAttnThreads) {
+      const uint32_t r = r0 + tx;
+      int n = 0, ov = 0;
+      if (r < a.rows) {
+        n = min(max(a.count[r], 0), (int)a.idx_stride);
+        ov = max((n + kAttnChunk - 1) / kAttnChunk - 1, 0);
+      }
+      const int incl = wave_inclusive_scan(ov);
+      if (lane == kWave - 1) wave_tot[wave] = incl;
+      __syncthreads();
+      int before = running, total = running;
 #pragma unroll
-    for (int w = 0; w < kAttnWaves; ++w) v += oacc[w][tx];
-    orow[tx] = (uint16_t)f32_to_bits16<DT>(v);
+      for (int wv = 0; wv < kAttnWaves; ++wv) {
+        before += (wv < wave) ? wave_tot[wv] : 0;
+        total += wave_tot[wv];
+      }
+      const int lo = before + incl - ov;  // first overflow chunk index owned by row r
+      if (ov > 0 && j >= lo && j < lo + ov) {
+        found[0] = (int)r; found[1] = j - lo + 1; found[2] = n;
+      }
+      hit = (j < total);
+      running = total;
+      __syncthreads();
+    }
+    if (!hit) return;  // j is past the last overflow chunk: nothing left for this workgroup
+    attn_chunk<DT>(a, sm, (uint32_t)found[0], found[1], found[2]);
+    __syncthreads();
   }
 }
 
 }  // namespace twl
+
+extern "C" uint64_t twl_sparse_attn_workspace_bytes(uint32_t rows, uint32_t idx_stride) {
+  const uint64_t splits = (idx_stride + twl::kAttnChunk - 1) / twl::kAttnChunk;
+  uint64_t tickets = ((uint64_t)rows * sizeof(int32_t) + 255) & ~255ull;
+  return tickets + (uint64_t)rows * splits * twl::kAttnPartial * sizeof(float);
+}
 
 extern "C" int twl_sparse_attn(const void* q, void* out, int dtype, const void* k_cache,
                                const void* v_cache, uint64_t page_stride, uint64_t token_stride,
@@ -177,37 +317,43 @@ extern "C" int twl_sparse_attn(const void* q, void* out, int dtype, const void* 
                                const int32_t* count, const int32_t* kv_page_indices,
                                const int32_t* kv_page_indptr, uint32_t batch,
                                uint32_t num_q_heads, uint32_t num_kv_heads, float sm_scale,
-                               float* lse_out, void* stream) {
-  if (!q || !out || !k_cache || !v_cache || !idx || !count || !kv_page_indices || !kv_page_indptr)
+                               float* lse_out, void* workspace, uint64_t workspace_bytes,
+                               void* stream) {
+  if (!q || !out || !k_cache || !v_cache || !idx || !count || !kv_page_indices ||
+      !kv_page_indptr || !workspace)
     return TWL_ENULL;
   if (dtype != TWL_F16 && dtype != TWL_BF16) return TWL_EDTYPE;
   if (batch == 0 || num_q_heads == 0 || num_kv_heads == 0 || num_q_heads % num_kv_heads != 0)
     return TWL_EINVAL;
   if (idx_stride == 0 || idx_stride > TWL_MAX_CANDIDATES) return TWL_EINVAL;
+  const uint64_t rows64 = (uint64_t)batch * num_q_heads;
+  if (rows64 > 65535u) return TWL_EINVAL;
+  const uint32_t rows = (uint32_t)rows64;
+  if (workspace_bytes < twl_sparse_attn_workspace_bytes(rows, idx_stride)) return TWL_EINVAL;
   if ((page_stride | token_stride | head_stride) & 7u) return TWL_EALIGN;  // 16-byte loads
   if ((((uintptr_t)q) & 15u) || (((uintptr_t)k_cache) & 15u) || (((uintptr_t)v_cache) & 15u) ||
-      (((uintptr_t)out) & 1u))
+      (((uintptr_t)out) & 1u) || (((uintptr_t)workspace) & 255u))
     return TWL_EALIGN;
   twl::AttnArgs a{};
   a.q = q; a.out = out; a.k_cache = k_cache; a.v_cache = v_cache; a.page_stride = page_stride;
   a.token_stride = token_stride; a.head_stride = head_stride; a.idx = idx;
   a.idx_stride = idx_stride; a.count = count; a.kv_page_indices = kv_page_indices;
   a.kv_page_indptr = kv_page_indptr; a.num_q_heads = num_q_heads; a.num_kv_heads = num_kv_heads;
-  a.sm_scale = sm_scale; a.lse_out = lse_out; a.lds_tokens = idx_stride;
-  const size_t lds_bytes = (size_t)idx_stride * sizeof(float);
-  dim3 grid(batch * num_q_heads);
-  if (dtype == TWL_F16) {
-    if (lds_bytes > 48 * 1024)
-      (void)hipFuncSetAttribute((const void*)twl::sparse_attn_kernel<TWL_F16>,
-                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-    hipLaunchKernelGGL((twl::sparse_attn_kernel<TWL_F16>), grid, dim3(twl::kAttnThreads),
-                       lds_bytes, (hipStream_t)stream, a);
-  } else {
-    if (lds_bytes > 48 * 1024)
-      (void)hipFuncSetAttribute((const void*)twl::sparse_attn_kernel<TWL_BF16>,
-                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-    hipLaunchKernelGGL((twl::sparse_attn_kernel<TWL_BF16>), grid, dim3(twl::kAttnThreads),
-                       lds_bytes, (hipStream_t)stream, a);
+  a.sm_scale = sm_scale; a.lse_out = lse_out;
+  a.max_splits = (idx_stride + twl::kAttnChunk - 1) / twl::kAttnChunk;
+  a.tickets = (int32_t*)workspace;
+  a.partials = (float*)((uint8_t*)workspace + (((uint64_t)rows * sizeof(int32_t) + 255) & ~255ull));
+  a.rows = rows;
+  {
+    const uint64_t overflow_max = (uint64_t)rows * (a.max_splits - 1);
+    a.pool = (uint32_t)(overflow_max < 1024 ? overflow_max : 1024);
   }
+  dim3 grid(rows + a.pool);
+  if (dtype == TWL_F16)
+    hipLaunchKernelGGL((twl::sparse_attn_kernel<TWL_F16>), grid, dim3(twl::kAttnThreads), 0,
+                       (hipStream_t)stream, a);
+  else
+    hipLaunchKernelGGL((twl::sparse_attn_kernel<TWL_BF16>), grid, dim3(twl::kAttnThreads), 0,
+                       (hipStream_t)stream, a);
   return hipGetLastError() == hipSuccess ? TWL_OK : TWL_ELAUNCH;
 }

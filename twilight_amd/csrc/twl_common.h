@@ -129,5 +129,17 @@ __device__ __forceinline__ float block_allreduce(float v, float* slots) {
   return t;
 }
 
+// inclusive scan of an int across the 64 lanes, in lane order
+__device__ __forceinline__ int wave_inclusive_scan(int v) {
+  int t;
+  t = dpp<0x111>(0, v); v += t;
+  t = dpp<0x112>(0, v); v += t;
+  t = dpp<0x114>(0, v); v += t;
+  t = dpp<0x118>(0, v); v += t;
+  t = dpp<kDppBcast15, 0xA>(0, v); v += t;
+  t = dpp<kDppBcast31, 0xC>(0, v); v += t;
+  return v;
+}
+
 }  // namespace twl
 #endif  // TWL_COMMON_H_

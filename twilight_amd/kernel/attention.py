@@ -23,17 +23,27 @@ def _cache_strides(cache: torch.Tensor, name: str):
     return cache.stride(0), cache.stride(1), cache.stride(2)
 
 
+def attention_workspace_bytes(rows: int, idx_stride: int) -> int:
+    """Bytes of scratch :func:`sparse_paged_decode_attention` needs for ``rows`` = B*H rows of at
+    most ``idx_stride`` survivors."""
+    return int(_lib.lib().twl_sparse_attn_workspace_bytes(rows, idx_stride))
+
+
 def sparse_paged_decode_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                                   idx: torch.Tensor, count: torch.Tensor,
                                   kv_page_indices: torch.Tensor, kv_page_indptr: torch.Tensor,
                                   sm_scale: Optional[float] = None, return_lse: bool = False,
-                                  out: Optional[torch.Tensor] = None):
+                                  out: Optional[torch.Tensor] = None,
+                                  workspace: Optional[torch.Tensor] = None):
     """Exact softmax attention of one decode token restricted to per-row survivor lists.
 
     ``q`` [B,H,128] fp16/bf16; ``k_cache`` / ``v_cache`` [pages,16,Hkv,128] of the same dtype;
     ``idx`` int32 [B,H,S] ascending logical token positions, ``count`` int32 [B,H]. Returns
     ``out`` [B,H,128] in q's dtype (and ``lse`` fp32 [B,H] when asked). Probabilities are rounded
-    to q's dtype before the V product as at attention.py:302-304.
+    to q's dtype before the V product as at attention.py:302-304 (rows of more than 128 survivors
+    are split over workgroups and merged in fp32 instead). ``workspace`` is a zero-initialised
+    uint8 tensor of :func:`attention_workspace_bytes` bytes that calls on one stream may share;
+    by default a fresh one is allocated.
     """
     check_input(q, "q")
     check_dim(3, q, "q")
@@ -70,9 +80,16 @@ def sparse_paged_decode_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cach
                 raise RuntimeError("out must match q")
         lse = torch.empty((B, H), dtype=torch.float32, device=dev) if return_lse else None
         scale = 1.0 / math.sqrt(D) if sm_scale is None else float(sm_scale)
+        need = attention_workspace_bytes(B * H, idx.size(2))
+        if workspace is None:
+            workspace = torch.zeros(need, dtype=torch.uint8, device=dev)
+        else:
+            check_input(workspace, "workspace"); check_dtype(workspace, torch.uint8, "workspace")
+            if workspace.numel() < need or workspace.device != dev:
+                raise RuntimeError(f"workspace must hold {need} bytes on {dev}")
         rc = _lib.lib().twl_sparse_attn(
             ptr(q), ptr(out), dtype_code(q.dtype, "q"), ptr(k_cache), ptr(v_cache), ks[0], ks[1],
             ks[2], ptr(idx), idx.size(2), ptr(count), ptr(kv_page_indices), ptr(kv_page_indptr),
-            B, H, Hkv, scale, ptr(lse), stream_of(q))
+            B, H, Hkv, scale, ptr(lse), ptr(workspace), workspace.numel(), stream_of(q))
     _lib.check(rc, "SparsePagedDecodeAttention")
     return (out, lse) if return_lse else out

@@ -77,20 +77,13 @@ class TwilightDecodeLayer:
         self.idx = torch.zeros((B, H, M), dtype=i32, device=dev)
         self.count = torch.zeros((B, H), dtype=i32, device=dev)
         self.out = torch.zeros((B, H, _lib.HEAD_DIM), dtype=c.dtype, device=dev)
+        ws = int(_lib.lib().twl_sparse_attn_workspace_bytes(B * H, M))
+        self.attn_workspace = torch.zeros(ws, dtype=torch.uint8, device=dev)
         self._shape = (B, c.max_pages_per_req)
+        self._args, self._args_key = None, None
 
-    def forward(self, q: torch.Tensor) -> torch.Tensor:
-        """``q`` [B, H, 128] in the cache dtype -> attention output [B, H, 128] (same buffer every
-        call). Intermediates stay readable as ``sel_pages/sel_count/scores/idx/count``."""
+    def _build_args(self, q: torch.Tensor) -> "_lib.LayerArgs":
         c = self.cache
-        check_input(q, "q")
-        check_dim(3, q, "q")
-        if (c.batch, c.max_pages_per_req) != self._shape:
-            self._alloc()
-        if tuple(q.shape) != (c.batch, self.H, _lib.HEAD_DIM) or q.dtype != c.dtype:
-            raise RuntimeError(f"q must be [{c.batch}, {self.H}, {_lib.HEAD_DIM}] of {c.dtype}")
-        if q.device != c.device:
-            raise RuntimeError(f"q must be on {c.device}")
         ks = c.k_cache.stride()
         a = _lib.LayerArgs()
         a.q, a.dtype = ptr(q), dtype_code(q.dtype, "q")
@@ -109,7 +102,28 @@ class TwilightDecodeLayer:
         a.cand_count = ptr(self.cand_count)
         a.idx, a.idx_stride = ptr(self.idx), self.idx.size(2)
         a.count = ptr(self.count)
+        a.attn_workspace, a.attn_workspace_bytes = ptr(self.attn_workspace), self.attn_workspace.numel()
         a.out = ptr(self.out)
+        return a
+
+    def forward(self, q: torch.Tensor) -> torch.Tensor:
+        """``q`` [B, H, 128] in the cache dtype -> attention output [B, H, 128] (same buffer every
+        call). Intermediates stay readable as ``sel_pages/sel_count/scores/idx/count``."""
+        c = self.cache
+        check_input(q, "q")
+        check_dim(3, q, "q")
+        if (c.batch, c.max_pages_per_req) != self._shape:
+            self._alloc()
+        if tuple(q.shape) != (c.batch, self.H, _lib.HEAD_DIM) or q.dtype != c.dtype:
+            raise RuntimeError(f"q must be [{c.batch}, {self.H}, {_lib.HEAD_DIM}] of {c.dtype}")
+        if q.device != c.device:
+            raise RuntimeError(f"q must be on {c.device}")
+        key = (q.data_ptr(), c.k_cache.data_ptr(), c.v_cache.data_ptr(), c.k_int4.data_ptr(),
+               c.meta.data_ptr(), c.kv_page_indices.data_ptr(), c.kv_page_indptr.data_ptr(),
+               c.kv_last_page_len.data_ptr())
+        if self._args_key != key:
+            self._args, self._args_key = self._build_args(q), key
+        a = self._args
         with torch.cuda.device(c.device):
             rc = _lib.lib().twl_decode_layer(ctypes.byref(a), stream_of(q))
         _lib.check(rc, "TwilightDecodeLayer")
