@@ -92,6 +92,8 @@ def main() -> int:
     ap.add_argument("--context", type=int, default=32768)
     ap.add_argument("--budget", type=int, default=8192)
     ap.add_argument("--top-p", type=float, default=0.95)
+    ap.add_argument("--layers", type=int, default=4,
+                    help="independent layer caches visited round-robin (cold-cache steps)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel breakdown")
     args = ap.parse_args()
@@ -116,58 +118,78 @@ def main() -> int:
     dt = torch.float16
 
     # ---- inputs, resident in HBM before anything is timed ----------------------------------
-    q, k, v, (ids, indptr, last) = synth.layer_inputs_device(B, H, Hkv, N, dt, dev, seed=0)
-    cache = PagedKVCache(B * npg, Hkv, dt, dev)
-    cache.k_cache, cache.v_cache = k, v
-    cache.set_page_table(ids, indptr, last)
-    cache.rebuild_shadow()
-    layer = TwilightDecodeLayer(cache, H, token_budget=args.budget, top_p=args.top_p, high="max")
+    # `--layers` independent caches (different data, same shape) are visited round-robin, as the
+    # layers of a model are during decode: no step finds its KV, INT4 shadow or Quest metadata
+    # left in the 256 MB last-level cache by the previous step.
+    layers, qs = [], []
+    for li in range(args.layers):
+        q, k, v, (ids, indptr, last) = synth.layer_inputs_device(B, H, Hkv, N, dt, dev, seed=10 * li)
+        cache = PagedKVCache(B * npg, Hkv, dt, dev)
+        cache.k_cache, cache.v_cache = k, v
+        cache.set_page_table(ids, indptr, last)
+        cache.rebuild_shadow()
+        layers.append(TwilightDecodeLayer(cache, H, token_budget=args.budget, top_p=args.top_p,
+                                          high="max"))
+        qs.append(q)
     torch.cuda.synchronize()
+    nl = len(layers)
 
     # ---- the timed region: K steps of the whole layer --------------------------------------
-    step = lambda: layer.forward(q)
-    for _ in range(args.warmup):
-        step()
+    for i in range(args.warmup):
+        layers[i % nl].forward(qs[i % nl])
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
+    for i in range(args.steps):
+        layers[i % nl].forward(qs[i % nl])
     torch.cuda.synchronize()
     wall_us = (time.perf_counter() - t0) * 1e6 / args.steps
-    n_bar = float(layer.count.float().mean())
-    n_max = int(layer.count.max())
-    kp = layer.k_pages
+    for i in range(nl):                      # leave every layer's buffers as a whole step does
+        layers[i].forward(qs[i])
+    torch.cuda.synchronize()
+    counts = torch.stack([l.count for l in layers]).float()
+    n_bar = float(counts.mean())
+    n_max = int(counts.max())
+    kp = layers[0].k_pages
     M = kp * 16
     rows = B * H
 
-    # ---- per-kernel times through the stand-alone entry points, same buffers ----------------
+    # ---- per-kernel times through the stand-alone entry points, same buffers, same rotation ----
     kernels = {}
     stream = torch.cuda.current_stream().cuda_stream
     p = lambda t: 0 if t is None else t.data_ptr()
-    ks = cache.k_cache.stride()
     sm = 1.0 / math.sqrt(D)
+
+    def rotating(make):
+        fns = [make(layers[i], layers[i].cache, qs[i]) for i in range(nl)]
+        state = {"i": 0}
+
+        def call():
+            fns[state["i"] % nl]()
+            state["i"] += 1
+        return call
+
     if not args.no_kernels:
-        it, wu = max(args.steps, 50), 10
+        it, wu = max(args.steps, 50), 2 * nl
         calls = {
-            "quest_score": (lambda: L.twl_quest_page_scores(
-                p(q), 0, p(cache.meta), p(cache.kv_page_indices), p(cache.kv_page_indptr), B, H, Hkv,
-                npg, p(layer.page_scores), npg, stream), rows * npg * (512 + 4) + rows * D * 2),
-            "quest_topk": (lambda: L.twl_quest_topk_pages(
-                p(layer.page_scores), npg, p(cache.kv_page_indptr), B, H, args.budget, npg,
-                p(layer.sel_pages), kp, p(layer.sel_count), stream), rows * (npg * 4 + kp * 4 + 4)),
-            "gemv_int4": (lambda: L.twl_gemv_int4(
-                p(q), 0, p(layer.scores), M, p(layer.cand_count), p(cache.k_int4), p(layer.sel_pages),
-                p(layer.sel_count), kp, p(cache.kv_page_indices), p(cache.kv_page_indptr),
-                p(cache.kv_last_page_len), B, H, Hkv, kp, sm, stream),
+            "quest_score": (rotating(lambda l, c, q: lambda: L.twl_quest_page_scores(
+                p(q), 0, p(c.meta), p(c.kv_page_indices), p(c.kv_page_indptr), B, H, Hkv,
+                npg, p(l.page_scores), npg, stream)), rows * npg * (512 + 4) + rows * D * 2),
+            "quest_topk": (rotating(lambda l, c, q: lambda: L.twl_quest_topk_pages(
+                p(l.page_scores), npg, p(c.kv_page_indptr), B, H, args.budget, npg,
+                p(l.sel_pages), kp, p(l.sel_count), stream)), rows * (npg * 4 + kp * 4 + 4)),
+            "gemv_int4": (rotating(lambda l, c, q: lambda: L.twl_gemv_int4(
+                p(q), 0, p(l.scores), M, p(l.cand_count), p(c.k_int4), p(l.sel_pages),
+                p(l.sel_count), kp, p(c.kv_page_indices), p(c.kv_page_indptr),
+                p(c.kv_last_page_len), B, H, Hkv, kp, sm, stream)),
                 rows * M * (64 + 16 + 4) + rows * D * 2 + rows * kp * 8),
-            "softmax_top_p": (lambda: L.twl_softmax_top_p_f32(
-                p(layer.scores), M, p(layer.cand_count), rows, M, 0, args.top_p, 1, p(layer.sel_pages),
-                kp, p(layer.idx), M, p(layer.count), 0, 0, stream),
+            "softmax_top_p": (rotating(lambda l, c, q: lambda: L.twl_softmax_top_p_f32(
+                p(l.scores), M, p(l.cand_count), rows, M, 0, args.top_p, 1, p(l.sel_pages),
+                kp, p(l.idx), M, p(l.count), 0, 0, stream)),
                 rows * M * 4 + int(rows * n_bar) * 4 + rows * 4),
-            "sparse_attn": (lambda: L.twl_sparse_attn(
-                p(q), p(layer.out), 0, p(cache.k_cache), p(cache.v_cache), ks[0], ks[1], ks[2],
-                p(layer.idx), M, p(layer.count), p(cache.kv_page_indices), p(cache.kv_page_indptr),
-                B, H, Hkv, sm, 0, p(layer.attn_workspace), layer.attn_workspace.numel(), stream),
+            "sparse_attn": (rotating(lambda l, c, q: lambda: L.twl_sparse_attn(
+                p(q), p(l.out), 0, p(c.k_cache), p(c.v_cache), *c.k_cache.stride()[:3],
+                p(l.idx), M, p(l.count), p(c.kv_page_indices), p(c.kv_page_indptr),
+                B, H, Hkv, sm, 0, p(l.attn_workspace), l.attn_workspace.numel(), stream)),
                 int(rows * n_bar) * (2 * D * 2 + 4) + rows * D * 4),
         }
         for name, (fn, nbytes) in calls.items():
@@ -175,8 +197,6 @@ def main() -> int:
             kernels[name] = {"us": round(us, 2), "bytes": nbytes,
                              "GBps": round(nbytes / us / 1e3, 1),
                              "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
-        layer.forward(q)  # leave the buffers as a whole step leaves them
-        torch.cuda.synchronize()
 
     layer_bytes = sum(kv["bytes"] for kv in kernels.values()) if kernels else None
     dom = kernels.get("quest_score")
@@ -191,10 +211,10 @@ def main() -> int:
     if not args.no_kernels and B == 8 and N == 32768:
         out2 = torch.empty((B, H, N), dtype=torch.float32, device=dev)
         cnt2 = torch.empty((B, H), dtype=torch.int32, device=dev)
-        fn = lambda: L.twl_gemv_int4(p(q), 0, p(out2), N, p(cnt2), p(cache.k_int4), 0, 0, 0,
-                                     p(cache.kv_page_indices), p(cache.kv_page_indptr),
-                                     p(cache.kv_last_page_len), B, H, Hkv, npg, sm, stream)
-        us = _time_calls(fn, 50, 10)
+        fn = rotating(lambda l, c, q: lambda: L.twl_gemv_int4(
+            p(q), 0, p(out2), N, p(cnt2), p(c.k_int4), 0, 0, 0, p(c.kv_page_indices),
+            p(c.kv_page_indptr), p(c.kv_last_page_len), B, H, Hkv, npg, sm, stream))
+        us = _time_calls(fn, 50, 2 * nl)
         nbytes = rows * N * 84 + rows * D * 2
         gemv_cfg2 = {"us": round(us, 2), "bytes": nbytes, "GBps": round(nbytes / us / 1e3, 1),
                      "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
@@ -216,7 +236,8 @@ def main() -> int:
                                f"budget {args.budget}, INT4 K estimate (group 32), top-p "
                                f"{args.top_p}",
                    "batch": B, "context": N, "budget": args.budget, "top_p": args.top_p,
-                   "survivors_mean": round(n_bar, 1), "survivors_max": n_max},
+                   "layers_rotated": nl, "survivors_mean": round(n_bar, 1),
+                   "survivors_max": n_max},
         "layer_bytes": layer_bytes,
         "layer_frac_of_hbm_peak": (round(layer_bytes / wall_us / 1e3 / HBM_PEAK_GBS, 4)
                                    if layer_bytes else None),

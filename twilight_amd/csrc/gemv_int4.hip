@@ -129,8 +129,9 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_int4_kernel(GemvArgs a) {
       const int phys = __builtin_amdgcn_readlane(my_phys, src_lane);
       logical[u] = __builtin_amdgcn_readlane(my_logical, src_lane);
       const uint8_t* rec = base + (size_t)phys * rec_stride;
-      nib[u] = *(const u32x4*)(rec + 16 * lane);
-      sz[u] = *(const uint32_t*)(rec + 1024 + 4 * lane);
+      // read-once stream: keep it out of the way of the data the other kernels reuse
+      nib[u] = __builtin_nontemporal_load((const u32x4*)(rec + 16 * lane));
+      sz[u] = __builtin_nontemporal_load((const uint32_t*)(rec + 1024 + 4 * lane));
     }
 #pragma unroll
     for (int u = 0; u < kGemvUnroll; ++u) {

@@ -79,7 +79,7 @@ __global__ __launch_bounds__(kQsThreads) void quest_score_kernel(QuestScoreArgs 
       const int pa = __builtin_amdgcn_readlane(my_phys, (ia < np) ? ia : 0);
       const int pb = __builtin_amdgcn_readlane(my_phys, (ib < np) ? ib : 0);
       const int phys = half ? pb : pa;
-      mm[u] = *(const u32x4*)(base + (size_t)phys * rec_stride);
+      mm[u] = __builtin_nontemporal_load((const u32x4*)(base + (size_t)phys * rec_stride));
     }
 #pragma unroll
     for (int u = 0; u < kQsUnroll; ++u) {
