@@ -94,6 +94,9 @@ def main() -> int:
     ap.add_argument("--top-p", type=float, default=0.95)
     ap.add_argument("--layers", type=int, default=4,
                     help="independent layer caches visited round-robin (cold-cache steps)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run 4 device copies of 1 GiB (a kernel of known traffic, used to "
+                         "scale the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel breakdown")
     args = ap.parse_args()
@@ -116,6 +119,14 @@ def main() -> int:
     B, H, Hkv, N, D = args.batch, 32, 32, args.context, 128
     npg = N // 16
     dt = torch.float16
+
+    if args.calibrate_copy:
+        src = torch.full((1 << 28,), 1.0, dtype=torch.float32, device=dev)   # 1 GiB
+        dst = torch.empty_like(src)
+        for _ in range(4):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     # ---- inputs, resident in HBM before anything is timed ----------------------------------
     # `--layers` independent caches (different data, same shape) are visited round-robin, as the
