@@ -171,7 +171,7 @@ int twl_sparse_attn(const void* q, void* out, int dtype, const void* k_cache, co
  * k = min(pages of the request, max(1, budget/16) + (budget%16 != 0)) (quest.py:93-98), top-k by
  * score with ties resolved toward the lower page number. Output: sel_pages [rows, sel_stride]
  * ascending logical page numbers, sel_count [rows]. page_scores (nullable) float
- * [rows, score_stride] receives the raw page scores.
+ * [rows, score_stride] receives the raw page scores (required: it is also the staging area).
  * ------------------------------------------------------------------------------------------- */
 int twl_quest_select(const void* q, int q_dtype, const void* meta, const int32_t* kv_page_indices,
                      const int32_t* kv_page_indptr, uint32_t batch, uint32_t num_q_heads,

@@ -87,6 +87,9 @@ def test_c_level_validation_without_gpu(hip_lib):
                              1, 1, 1, 1.0, 0, 0, ws, 0) == -1             # workspace NULL
     assert L.twl_quest_select(fake, 0, fake, fake, fake, 1, 1, 1, 0, 4, fake, 4, fake, fake, 4, 0) == -2
     assert L.twl_quest_select(fake, 0, fake, fake, fake, 1, 1, 1, 64, 4, fake, 2, fake, fake, 4, 0) == -2
+    assert L.twl_quest_select(fake, 0, fake, fake, fake, 1, 1, 1, 64, 4, 0, 4, fake, fake, 4, 0) == -1
+    assert L.twl_quest_topk_pages(fake, 4, fake, 1, 1, 64, 4, fake, 2, fake, 0) == -2
+    assert L.twl_quest_page_scores(fake, 0, fake, fake, fake, 1, 1, 1, 4, 0, 4, 0) == -1
     assert L.twl_kv_shadow_build(fake, 0, 4096, 256, 128, 0, 0, 1, 1, 0, 0, 0) == -1
     assert L.twl_dequant_int4(fake, 0, fake, 0) == -2
     assert L.twl_decode_layer(None, 0) == -1

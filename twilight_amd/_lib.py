@@ -24,7 +24,9 @@ MAX_CANDIDATES = 32768
 EXPORTS = (
     "twl_strerror", "twl_abi_version", "twl_device_count", "twl_top_p_f32", "twl_top_p_f16",
     "twl_softmax_top_p_f32", "twl_gemv_int4", "twl_gemv_int4_nhd", "twl_sparse_attn",
-    "twl_sparse_attn_workspace_bytes", "twl_quest_select", "twl_quest_page_scores", "twl_quest_topk_pages", "twl_kv_shadow_build", "twl_dequant_int4", "twl_decode_layer",
+    "twl_sparse_attn_workspace_bytes", "twl_quest_select",
+    "twl_quest_page_scores", "twl_quest_topk_pages", "twl_kv_shadow_build", "twl_dequant_int4",
+    "twl_decode_layer",
 )
 
 

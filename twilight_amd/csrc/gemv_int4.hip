@@ -8,9 +8,11 @@
 // zero pair). Lane l holds token l/4, quantisation group l%4 — exactly the 32 nibbles that share
 // one scale — so dequantisation factors out of the inner loop:
 //     partial = scale * sum_j q_j * nibble_j + zero * sum_j q_j
-// with sum_j q_j precomputed once per row. Nibbles become exact fp16 integers with one
-// v_and_or (1024 + n) and one packed subtract, products are accumulated in fp32 by v_dot2, and a
-// two-step DPP quad reduction yields the token's score.
+// with sum_j q_j precomputed once per row. Nibbles become exact fp16 values with one shift and one
+// v_and_or, products are accumulated in fp32 by v_dot2, a two-step DPP quad reduction yields the
+// token's score, and the 64 scores of four pages leave in one 256-byte store. The kernel is close
+// to co-limited by VALU issue (about 100 instructions per page fit under the HBM stream at 7 TB/s),
+// which is why the unpack is kept to 11 instructions per 8 nibbles.
 #include "twl_common.h"
 
 namespace twl {
@@ -33,19 +35,31 @@ struct GemvArgs {
   float sm_scale;
 };
 
-constexpr int kGemvThreads = 256;                 // 4 wavefronts
-constexpr int kGemvPagesPerWave = 16;
+#ifndef TWL_GEMV_THREADS
+#define TWL_GEMV_THREADS 256
+#endif
+#ifndef TWL_GEMV_PAGES_PER_WAVE
+#define TWL_GEMV_PAGES_PER_WAVE 16
+#endif
+#ifndef TWL_GEMV_UNROLL
+#define TWL_GEMV_UNROLL 4
+#endif
+constexpr int kGemvThreads = TWL_GEMV_THREADS;    // 4 wavefronts
+constexpr int kGemvPagesPerWave = TWL_GEMV_PAGES_PER_WAVE;  // <= 64: one lane per page id
 constexpr int kGemvPagesPerBlock = kGemvPagesPerWave * (kGemvThreads / kWave);
-constexpr int kGemvUnroll = 4;
+constexpr int kGemvUnroll = TWL_GEMV_UNROLL;      // pages in flight per wavefront
 
-// 8 nibbles of one dword against 8 q values held as 4 half2 pairs (n0,n4),(n1,n5),(n2,n6),(n3,n7)
+// 8 nibbles of one dword against 8 q values held as 4 half2 pairs (n0,n4),(n1,n5),(n2,n6),(n3,n7).
+// A nibble moved to mantissa bits 4..7 of an fp16 with exponent 0 is exactly 1 + n/64, so one
+// shift and one v_and_or turn two nibbles into a half2 and v_dot2 accumulates
+// sum q*(1 + n/64) in fp32; the caller removes the bias with sum q (a number of the same size:
+// the cancellation costs about one fp32 ulp of sum q).
 __device__ __forceinline__ float dot8_nibbles(uint32_t w, const half2_t* qp, float acc) {
-  const half2_t bias = {(_Float16)1024.0f, (_Float16)1024.0f};
-  const uint32_t m = 0x000F000Fu, magic = 0x64006400u;  // fp16 1024 + n
-  half2_t a0 = __builtin_bit_cast(half2_t, (w & m) | magic) - bias;
-  half2_t a1 = __builtin_bit_cast(half2_t, ((w >> 4) & m) | magic) - bias;
-  half2_t a2 = __builtin_bit_cast(half2_t, ((w >> 8) & m) | magic) - bias;
-  half2_t a3 = __builtin_bit_cast(half2_t, ((w >> 12) & m) | magic) - bias;
+  const uint32_t m = 0x00F000F0u, one = 0x3C003C00u;
+  half2_t a0 = __builtin_bit_cast(half2_t, ((w << 4) & m) | one);
+  half2_t a1 = __builtin_bit_cast(half2_t, (w & m) | one);
+  half2_t a2 = __builtin_bit_cast(half2_t, ((w >> 4) & m) | one);
+  half2_t a3 = __builtin_bit_cast(half2_t, ((w >> 8) & m) | one);
   acc = __builtin_amdgcn_fdot2(a0, qp[0], acc, false);
   acc = __builtin_amdgcn_fdot2(a1, qp[1], acc, false);
   acc = __builtin_amdgcn_fdot2(a2, qp[2], acc, false);
@@ -53,38 +67,79 @@ __device__ __forceinline__ float dot8_nibbles(uint32_t w, const half2_t* qp, flo
   return acc;
 }
 
-template <int QDT>
+// score of one page for this lane's token: 32 nibbles of one group against the lane's q slice
+__device__ __forceinline__ float page_partial(const u32x4& nib, uint32_t sz, const half2_t* qp,
+                                              float qsum) {
+  float acc = 0.0f;
+#ifdef TWL_GEMV_NOCOMPUTE
+  acc = as_f32((nib.x ^ nib.y ^ nib.z ^ nib.w) & 0x3F800000u);
+#else
+  acc = dot8_nibbles(nib.x, qp + 0, acc);
+  acc = dot8_nibbles(nib.y, qp + 4, acc);
+  acc = dot8_nibbles(nib.z, qp + 8, acc);
+  acc = dot8_nibbles(nib.w, qp + 12, acc);
+#endif
+  // sum q*nibble = 64 * (acc - sum q);  partial = scale * sum q*nibble + zero * sum q
+  const float scale64 = f16_bits_to_f32(sz & 0xFFFFu) * 64.0f;
+  const float zero = f16_bits_to_f32(sz >> 16);
+  return quad_allreduce<OpSum>(fmaf(scale64, acc - qsum, zero * qsum));
+}
+
+// HAS_SEL: the row has its own page list (sel_pages / sel_count); otherwise every page of the
+// request is a candidate.
+template <int QDT, bool HAS_SEL>
 __global__ __launch_bounds__(kGemvThreads) void gemv_int4_kernel(GemvArgs a) {
+  constexpr int U = kGemvUnroll;
+  constexpr int G = kGemvPagesPerWave / U;  // load groups per wavefront
   const uint32_t row = blockIdx.y;
   const uint32_t b = row / a.num_q_heads;
   const uint32_t h = row - b * a.num_q_heads;
   const uint32_t kvh = h / (a.num_q_heads / a.num_kv_heads);
   const int lane = lane_id();
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int p0 = blockIdx.x * kGemvPagesPerBlock + wave * kGemvPagesPerWave;
 
+  // everything that depends only on the kernel arguments is requested at once
   const int pg_begin = a.kv_page_indptr[b];
-  const int req_pages = a.kv_page_indptr[b + 1] - pg_begin;
-  int n_pages = a.sel_pages ? (a.sel_count ? a.sel_count[row] : (int)a.sel_stride) : req_pages;
+  const int pg_end = a.kv_page_indptr[b + 1];
+  const int last_len = a.kv_last_page_len[b];
+  const int sel_n = HAS_SEL ? (a.sel_count ? a.sel_count[row] : (int)a.sel_stride) : 0;
+  int my_logical = p0 + lane;
+  if (HAS_SEL) {
+    // read ahead of the count: the slot exists whenever it is inside the row's stride
+    my_logical = (lane < kGemvPagesPerWave && (uint32_t)(p0 + lane) < a.sel_stride)
+                     ? a.sel_pages[(size_t)row * a.sel_stride + p0 + lane] : 0;
+  }
+  const int g = lane & 3;
+  const int t = lane >> 2;
+  u32x4 qraw[4];
+  {
+    const uint16_t* qrow = (const uint16_t*)a.q + (size_t)row * TWL_HEAD_DIM + 32 * g;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) qraw[i] = *(const u32x4*)(qrow + 8 * i);
+  }
+
+  const int req_pages = pg_end - pg_begin;
+  int n_pages = HAS_SEL ? sel_n : req_pages;
   n_pages = min(max(n_pages, 0), (int)a.max_pages);
   if (req_pages <= 0) n_pages = 0;
   if (blockIdx.x == 0 && threadIdx.x == 0 && a.out_count) a.out_count[row] = n_pages * TWL_PAGE;
-
-  const int p0 = blockIdx.x * kGemvPagesPerBlock + wave * kGemvPagesPerWave;
   if (p0 >= n_pages) return;
   const int np = min(kGemvPagesPerWave, n_pages - p0);
 
+  // ---- page ids of this wave's run: lane i owns run entry i ---------------------------------
+  my_logical = min(max(my_logical, 0), req_pages - 1);  // a corrupt list must not leave the table
+  int my_phys = 0;
+  if (lane < np) my_phys = a.kv_page_indices[pg_begin + my_logical];
+
   // ---- q: lane (t = l/4, g = l%4) keeps q[32g .. 32g+32) as 16 half2 pairs -------------------
-  const int g = lane & 3;
-  const int t = lane >> 2;
   half2_t qp[16];
   float qsum = 0.0f;
   {
-    const uint16_t* qrow = (const uint16_t*)a.q + (size_t)row * TWL_HEAD_DIM + 32 * g;
     float qf[32];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      u32x4 v = *(const u32x4*)(qrow + 8 * i);
-      const uint32_t ws[4] = {v.x, v.y, v.z, v.w};
+      const uint32_t ws[4] = {qraw[i].x, qraw[i].y, qraw[i].z, qraw[i].w};
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         qf[8 * i + 2 * j] = bits16_to_f32<QDT>(ws[j] & 0xFFFFu);
@@ -102,53 +157,65 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_int4_kernel(GemvArgs a) {
     for (int i = 0; i < 32; ++i) qsum += (float)(_Float16)qf[i];
   }
 
-  // ---- page ids of this wave's run: lane i owns run entry i ---------------------------------
-  int my_logical = -1, my_phys = 0;
-  if (lane < np) {
-    my_logical = a.sel_pages ? a.sel_pages[(size_t)row * a.sel_stride + p0 + lane] : p0 + lane;
-    my_logical = min(max(my_logical, 0), req_pages - 1);  // a corrupt list must not leave the table
-    my_phys = a.kv_page_indices[pg_begin + my_logical];
-  }
-  const int last_len = a.kv_last_page_len[b];
   const size_t rec_stride = (size_t)a.num_kv_heads * TWL_INT4_RECORD_BYTES;
-  const uint8_t* base = a.k_int4 + (size_t)kvh * TWL_INT4_RECORD_BYTES;
+  const uint8_t* base = a.k_int4 + (size_t)kvh * TWL_INT4_RECORD_BYTES + 16 * lane;
   float* orow = a.out + (size_t)row * a.out_stride + (size_t)p0 * TWL_PAGE;
   const float ninf = -__builtin_inff();
 
+  // ---- stream: group k+1 is requested before group k is consumed -----------------------------
+  u32x4 nib[2][U];
+  uint32_t sz[2][U];
+  auto issue = [&](int grp, int buf) {
 #pragma unroll
-  for (int i0 = 0; i0 < kGemvPagesPerWave; i0 += kGemvUnroll) {
-    if (i0 >= np) break;
-    u32x4 nib[kGemvUnroll];
-    uint32_t sz[kGemvUnroll];
-    int logical[kGemvUnroll];
-#pragma unroll
-    for (int u = 0; u < kGemvUnroll; ++u) {
-      const int i = i0 + u;
+    for (int u = 0; u < U; ++u) {
+      const int i = grp * U + u;
       // entries past the run reuse entry 0: a valid address, result discarded
-      const int src_lane = (i < np) ? i : 0;
-      const int phys = __builtin_amdgcn_readlane(my_phys, src_lane);
-      logical[u] = __builtin_amdgcn_readlane(my_logical, src_lane);
+      const int phys = __builtin_amdgcn_readlane(my_phys, (i < np) ? i : 0);
       const uint8_t* rec = base + (size_t)phys * rec_stride;
       // read-once stream: keep it out of the way of the data the other kernels reuse
-      nib[u] = __builtin_nontemporal_load((const u32x4*)(rec + 16 * lane));
-      sz[u] = __builtin_nontemporal_load((const uint32_t*)(rec + 1024 + 4 * lane));
+      nib[buf][u] = __builtin_nontemporal_load((const u32x4*)rec);
+      sz[buf][u] = __builtin_nontemporal_load((const uint32_t*)(rec + 1024 - 12 * lane));
     }
+  };
+#ifndef TWL_GEMV_DBUF
+#define TWL_GEMV_DBUF 0
+#endif
+  static_assert(U == 4, "the output transpose below moves 4 pages x 16 tokens per store");
+  // lane l stores element l of the group's 64 scores (page l/16, token l%16); it takes that value
+  // from the lane that owns token l%16 and whose group index equals the page: lane 4*(l%16)+l/16
+  const int src_lane4 = 4 * (4 * (lane & 15) + (lane >> 4));
+  if (TWL_GEMV_DBUF) issue(0, 0);
 #pragma unroll
-    for (int u = 0; u < kGemvUnroll; ++u) {
-      const int i = i0 + u;
-      float acc = 0.0f;
-      acc = dot8_nibbles(nib[u].x, qp + 0, acc);
-      acc = dot8_nibbles(nib[u].y, qp + 4, acc);
-      acc = dot8_nibbles(nib[u].z, qp + 8, acc);
-      acc = dot8_nibbles(nib[u].w, qp + 12, acc);
-      const float scale = f16_bits_to_f32(sz[u] & 0xFFFFu);
-      const float zero = f16_bits_to_f32(sz[u] >> 16);
-      float part = fmaf(zero, qsum, scale * acc);
-      part = quad_allreduce<OpSum>(part);
-      if (i < np && g == 0) {
-        const int valid = (logical[u] == req_pages - 1) ? last_len : TWL_PAGE;
-        orow[i * TWL_PAGE + t] = (t < valid) ? part * a.sm_scale : ninf;
+  for (int grp = 0; grp < G; ++grp) {
+    const int buf = TWL_GEMV_DBUF ? (grp & 1) : 0;
+    if (TWL_GEMV_DBUF) {
+      if (grp + 1 < G && (grp + 1) * U < np) issue(grp + 1, buf ^ 1);
+    } else if (grp * U < np) {
+      issue(grp, 0);
+    }
+    if (grp * U < np) {
+      float mine = 0.0f;  // the score this lane hands over: page g of the group, token t
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int i = grp * U + u;
+        const float part = page_partial(nib[buf][u], sz[buf][u], qp, qsum);
+        const int logical = __builtin_amdgcn_readlane(my_logical, (i < np) ? i : 0);
+        const int valid = (logical == req_pages - 1) ? last_len : TWL_PAGE;
+        const float val = (t < valid) ? part * a.sm_scale : ninf;
+        mine = (g == u) ? val : mine;
       }
+      const float sc = as_f32(__builtin_amdgcn_ds_bpermute(src_lane4, as_i32(mine)));
+      // one 256-byte store per group; pages past the run are masked off
+#ifdef TWL_GEMV_NOSTORE
+      if (grp * U + (lane >> 4) < np && sc == 12345.0f)
+#else
+      if (grp * U + (lane >> 4) < np)
+#endif
+#ifdef TWL_GEMV_NTSTORE
+        __builtin_nontemporal_store(sc, orow + grp * U * TWL_PAGE + lane);
+#else
+        orow[grp * U * TWL_PAGE + lane] = sc;
+#endif
     }
   }
 }
@@ -222,7 +289,7 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_int4_nhd_kernel(GemvNhdArgs
       acc = dot8_nibbles(nib.y, qp + 4, acc);
       acc = dot8_nibbles(nib.z, qp + 8, acc);
       acc = dot8_nibbles(nib.w, qp + 12, acc);
-      float part = fmaf(zero, qsum, scale * acc);
+      float part = fmaf(scale * 64.0f, acc - qsum, zero * qsum);
       // tokens are aligned to quads, so all four lanes of a quad take this branch together
       part = quad_allreduce<OpSum>(part);
       if (g == 0)
@@ -260,12 +327,15 @@ extern "C" int twl_gemv_int4(const void* q, int q_dtype, float* out, uint32_t ou
   a.num_kv_heads = num_kv_heads; a.max_pages = max_pages_per_row; a.sm_scale = sm_scale;
   const uint32_t gx = (max_pages_per_row + twl::kGemvPagesPerBlock - 1) / twl::kGemvPagesPerBlock;
   dim3 grid(gx, batch * num_q_heads);
-  if (q_dtype == TWL_F16)
-    hipLaunchKernelGGL((twl::gemv_int4_kernel<TWL_F16>), grid, dim3(twl::kGemvThreads), 0,
-                       (hipStream_t)stream, a);
-  else
-    hipLaunchKernelGGL((twl::gemv_int4_kernel<TWL_BF16>), grid, dim3(twl::kGemvThreads), 0,
-                       (hipStream_t)stream, a);
+  const dim3 blk(twl::kGemvThreads);
+  hipStream_t st = (hipStream_t)stream;
+  if (q_dtype == TWL_F16) {
+    if (sel_pages) hipLaunchKernelGGL((twl::gemv_int4_kernel<TWL_F16, true>), grid, blk, 0, st, a);
+    else hipLaunchKernelGGL((twl::gemv_int4_kernel<TWL_F16, false>), grid, blk, 0, st, a);
+  } else {
+    if (sel_pages) hipLaunchKernelGGL((twl::gemv_int4_kernel<TWL_BF16, true>), grid, blk, 0, st, a);
+    else hipLaunchKernelGGL((twl::gemv_int4_kernel<TWL_BF16, false>), grid, blk, 0, st, a);
+  }
   return hipGetLastError() == hipSuccess ? TWL_OK : TWL_ELAUNCH;
 }
 

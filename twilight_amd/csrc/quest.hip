@@ -8,15 +8,17 @@
 // 4 KiB of K). Kernel 1 streams the metadata (the largest HBM term of the decode layer): one
 // 16-byte load per lane covers 4 channels' min and max, so a wavefront scores 2 pages per load
 // instruction; the max/min choice is one bit-select per channel pair because sign(q) is fixed for
-// the row, and products are accumulated in fp32. Kernel 2 selects the k best pages of a row with
-// an MSB-first radix select on order-preserving keys held in registers and emits them in
-// ascending page order (ties at the k-th score go to the lower page number; torch.topk leaves
-// that order unspecified, quest.py:99).
+// the row, and products are accumulated in fp32. The k best pages of a row are then selected with
+// an MSB-first radix select on order-preserving keys held in registers and emitted in ascending
+// page order (ties at the k-th score go to the lower page number; torch.topk leaves that order
+// unspecified, quest.py:99). (Letting the last scoring workgroup of a row do the selection, to
+// save the second launch, was measured and is slower: the device-scope stores and the ticket
+// keep every scoring workgroup alive for a memory round trip longer.)
 #include "twl_common.h"
 
 namespace twl {
 
-struct QuestScoreArgs {
+struct QuestArgs {
   const void* q;
   const uint8_t* meta;
   const int32_t* kv_page_indices;
@@ -25,6 +27,10 @@ struct QuestScoreArgs {
   uint32_t max_pages;  // pages per request the grid and the score row are sized for
   float* page_scores;
   uint32_t score_stride;
+  uint32_t token_budget;
+  int32_t* sel_pages;
+  uint32_t sel_stride;
+  int32_t* sel_count;
 };
 
 constexpr int kQsThreads = 256;
@@ -32,90 +38,10 @@ constexpr int kQsPagesPerWave = 32;
 constexpr int kQsPagesPerBlock = kQsPagesPerWave * (kQsThreads / kWave);  // 128
 constexpr int kQsUnroll = 4;  // load instructions in flight per wave (2 pages each)
 
-template <int DT>
-__global__ __launch_bounds__(kQsThreads) void quest_score_kernel(QuestScoreArgs a) {
-  const uint32_t row = blockIdx.y;
-  const uint32_t b = row / a.num_q_heads;
-  const uint32_t h = row - b * a.num_q_heads;
-  const uint32_t kvh = h / (a.num_q_heads / a.num_kv_heads);
-  const int lane = lane_id();
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-  const int pg_begin = a.kv_page_indptr[b];
-  const int n_pages = min(a.kv_page_indptr[b + 1] - pg_begin, (int)a.max_pages);
-  const int p0 = blockIdx.x * kQsPagesPerBlock + wave * kQsPagesPerWave;
-  if (p0 >= n_pages) return;
-  const int np = min(kQsPagesPerWave, n_pages - p0);
-
-  const int c = lane & 31;   // channel chunk: dims 4c..4c+3
-  const int half = lane >> 5;  // which of the 2 pages of a load
-  // q for dims 4c..4c+3 and the per-half select mask (all ones where q > 0)
-  uint32_t qw[2];
-  {
-    u32x2 v = *(const u32x2*)((const uint16_t*)a.q + (size_t)row * TWL_HEAD_DIM + 4 * c);
-    qw[0] = v.x; qw[1] = v.y;
-  }
-  float qf[4];
-  uint32_t selmask[2];
-#pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    qf[2 * j] = bits16_to_f32<DT>(qw[j] & 0xFFFFu);
-    qf[2 * j + 1] = bits16_to_f32<DT>(qw[j] >> 16);
-    selmask[j] = (qf[2 * j] > 0.0f ? 0x0000FFFFu : 0u) | (qf[2 * j + 1] > 0.0f ? 0xFFFF0000u : 0u);
-  }
-
-  int my_phys = 0;
-  if (lane < np) my_phys = a.kv_page_indices[pg_begin + p0 + lane];
-  const size_t rec_stride = (size_t)a.num_kv_heads * TWL_META_RECORD_BYTES;
-  const uint8_t* base = a.meta + (size_t)kvh * TWL_META_RECORD_BYTES + 16 * c;
-  float* orow = a.page_scores + (size_t)row * a.score_stride + p0;
-
-#pragma unroll
-  for (int i0 = 0; i0 < kQsPagesPerWave; i0 += 2 * kQsUnroll) {
-    if (i0 >= np) break;
-    u32x4 mm[kQsUnroll];
-#pragma unroll
-    for (int u = 0; u < kQsUnroll; ++u) {
-      const int ia = i0 + 2 * u, ib = ia + 1;
-      const int pa = __builtin_amdgcn_readlane(my_phys, (ia < np) ? ia : 0);
-      const int pb = __builtin_amdgcn_readlane(my_phys, (ib < np) ? ib : 0);
-      const int phys = half ? pb : pa;
-      mm[u] = __builtin_nontemporal_load((const u32x4*)(base + (size_t)phys * rec_stride));
-    }
-#pragma unroll
-    for (int u = 0; u < kQsUnroll; ++u) {
-      // words: x,y = min[4c..4c+3], z,w = max[4c..4c+3]
-      const uint32_t s0 = (mm[u].z & selmask[0]) | (mm[u].x & ~selmask[0]);
-      const uint32_t s1 = (mm[u].w & selmask[1]) | (mm[u].y & ~selmask[1]);
-      float acc;
-      if (DT == TWL_F16) {
-        acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, s0),
-                                     __builtin_bit_cast(half2_t, qw[0]), 0.0f, false);
-        acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, s1),
-                                     __builtin_bit_cast(half2_t, qw[1]), acc, false);
-      } else {
-        acc = qf[0] * as_f32(s0 << 16);
-        acc = fmaf(qf[1], as_f32(s0 & 0xFFFF0000u), acc);
-        acc = fmaf(qf[2], as_f32(s1 << 16), acc);
-        acc = fmaf(qf[3], as_f32(s1 & 0xFFFF0000u), acc);
-      }
-      acc = row16_allreduce<OpSum>(acc);
-      acc += dpp<kDppBcast15, 0xA>(0.0f, acc);  // lanes 16..31 / 48..63 now hold a page total
-      const int i = i0 + 2 * u + half;
-      if ((lane & 31) == 31 && i < np) orow[i] = acc;
-    }
-  }
-}
-
-struct QuestSelectArgs {
-  const float* page_scores;
-  uint32_t score_stride;
-  const int32_t* kv_page_indptr;
-  uint32_t num_q_heads;
-  uint32_t max_pages;
-  uint32_t token_budget;
-  int32_t* sel_pages;
-  uint32_t sel_stride;
-  int32_t* sel_count;
+struct SelSmem {
+  int hist[256];
+  int pick[2];       // chosen digit, remaining k
+  int wave_tot[16];
 };
 
 __device__ __forceinline__ uint32_t order_key(float f) {
@@ -123,15 +49,11 @@ __device__ __forceinline__ uint32_t order_key(float f) {
   return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 
-// Thread t holds pages [t*VPT, (t+1)*VPT) of the row.
+// Top-k pages of one row by all THREADS threads of the workgroup; thread t holds pages
+// [t*VPT, (t+1)*VPT).
 template <int THREADS, int VPT>
-__global__ __launch_bounds__(THREADS) void quest_select_kernel(QuestSelectArgs a) {
+__device__ __forceinline__ void quest_select_row(const QuestArgs& a, uint32_t row, SelSmem& sm) {
   constexpr int NWAVES = THREADS / kWave;
-  __shared__ int hist[256];
-  __shared__ int pick[2];       // chosen digit, remaining k
-  __shared__ int wave_tot[16];
-
-  const uint32_t row = blockIdx.x;
   const uint32_t b = row / a.num_q_heads;
   const int tx = threadIdx.x;
   const int lane = lane_id();
@@ -151,10 +73,16 @@ __global__ __launch_bounds__(THREADS) void quest_select_kernel(QuestSelectArgs a
 
   uint32_t key[VPT];
   const float* src = a.page_scores + (size_t)row * a.score_stride;
+  {
+    // all loads are issued before any is consumed (index clamped instead of predicated)
+    float v[VPT];
 #pragma unroll
-  for (int j = 0; j < VPT; ++j) {
-    const int e = tx * VPT + j;
-    key[j] = (e < n_pages) ? order_key(src[e]) : 0u;
+    for (int j = 0; j < VPT; ++j) {
+      const int e = min(tx * VPT + j, n_pages - 1);
+      v[j] = src[e];
+    }
+#pragma unroll
+    for (int j = 0; j < VPT; ++j) key[j] = (tx * VPT + j < n_pages) ? order_key(v[j]) : 0u;
   }
 
   // ---- radix select of the k-th largest key ------------------------------------------------
@@ -162,12 +90,12 @@ __global__ __launch_bounds__(THREADS) void quest_select_kernel(QuestSelectArgs a
   int k_rem = k;
 #pragma unroll
   for (int shift = 24; shift >= 0; shift -= 8) {
-    if (tx < 256) hist[tx] = 0;
+    for (int i = tx; i < 256; i += THREADS) sm.hist[i] = 0;
     __syncthreads();
 #pragma unroll
     for (int j = 0; j < VPT; ++j) {
       if ((key[j] & prefix_mask) == prefix && key[j] != 0u)
-        atomicAdd(&hist[(key[j] >> shift) & 0xFFu], 1);
+        atomicAdd(&sm.hist[(key[j] >> shift) & 0xFFu], 1);
     }
     __syncthreads();
     if (wave == 0) {
@@ -176,7 +104,7 @@ __global__ __launch_bounds__(THREADS) void quest_select_kernel(QuestSelectArgs a
       int mine = 0;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        hcnt[j] = hist[255 - 4 * lane - j];
+        hcnt[j] = sm.hist[255 - 4 * lane - j];
         mine += hcnt[j];
       }
       const int incl = wave_inclusive_scan(mine);
@@ -185,17 +113,17 @@ __global__ __launch_bounds__(THREADS) void quest_select_kernel(QuestSelectArgs a
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           if (run < k_rem && k_rem <= run + hcnt[j]) {
-            pick[0] = 255 - 4 * lane - j;
-            pick[1] = k_rem - run;
+            sm.pick[0] = 255 - 4 * lane - j;
+            sm.pick[1] = k_rem - run;
           }
           run += hcnt[j];
         }
       }
     }
     __syncthreads();
-    prefix |= (uint32_t)pick[0] << shift;
+    prefix |= (uint32_t)sm.pick[0] << shift;
     prefix_mask |= 0xFFu << shift;
-    k_rem = pick[1];
+    k_rem = sm.pick[1];
   }
   const uint32_t T = prefix;  // k-th largest key; k_rem of the keys equal to T are taken
 
@@ -205,11 +133,11 @@ __global__ __launch_bounds__(THREADS) void quest_select_kernel(QuestSelectArgs a
   for (int j = 0; j < VPT; ++j) packed += (key[j] > T ? 0x10000 : 0) + (key[j] == T ? 1 : 0);
   const int incl = wave_inclusive_scan(packed);
   const int wtot = __builtin_amdgcn_readlane(incl, 63);
-  if (lane == 0) wave_tot[wave] = wtot;
+  if (lane == 0) sm.wave_tot[wave] = wtot;
   __syncthreads();
   int before = incl - packed;
 #pragma unroll
-  for (int w = 0; w < NWAVES; ++w) before += (w < wave) ? wave_tot[w] : 0;
+  for (int w = 0; w < NWAVES; ++w) before += (w < wave) ? sm.wave_tot[w] : 0;
   int gt_before = before >> 16, eq_before = before & 0xFFFF;
 #pragma unroll
   for (int j = 0; j < VPT; ++j) {
@@ -222,6 +150,93 @@ __global__ __launch_bounds__(THREADS) void quest_select_kernel(QuestSelectArgs a
       ++eq_before;
     }
   }
+}
+
+template <int THREADS, int VPT>
+__global__ __launch_bounds__(THREADS) void quest_select_kernel(QuestArgs a) {
+  __shared__ SelSmem sm;
+  quest_select_row<THREADS, VPT>(a, blockIdx.x, sm);
+}
+
+template <int DT>
+__global__ __launch_bounds__(kQsThreads) void quest_score_kernel(QuestArgs a) {
+  const uint32_t row = blockIdx.y;
+  const uint32_t b = row / a.num_q_heads;
+  const uint32_t h = row - b * a.num_q_heads;
+  const uint32_t kvh = h / (a.num_q_heads / a.num_kv_heads);
+  const int lane = lane_id();
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int pg_begin = a.kv_page_indptr[b];
+  const int n_pages = min(max(a.kv_page_indptr[b + 1] - pg_begin, 0), (int)a.max_pages);
+  const int p0 = blockIdx.x * kQsPagesPerBlock + wave * kQsPagesPerWave;
+  const int np = min(kQsPagesPerWave, n_pages - p0);  // <= 0: this wave has nothing to stream
+
+  if (np > 0) {
+    const int c = lane & 31;     // channel chunk: dims 4c..4c+3
+    const int half = lane >> 5;  // which of the 2 pages of a load
+    // q for dims 4c..4c+3 and the per-half select mask (all ones where q > 0)
+    uint32_t qw[2];
+    {
+      u32x2 v = *(const u32x2*)((const uint16_t*)a.q + (size_t)row * TWL_HEAD_DIM + 4 * c);
+      qw[0] = v.x; qw[1] = v.y;
+    }
+    int my_phys = 0;
+    if (lane < np) my_phys = a.kv_page_indices[pg_begin + p0 + lane];
+    float qf[4];
+    uint32_t selmask[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      qf[2 * j] = bits16_to_f32<DT>(qw[j] & 0xFFFFu);
+      qf[2 * j + 1] = bits16_to_f32<DT>(qw[j] >> 16);
+      selmask[j] = (qf[2 * j] > 0.0f ? 0x0000FFFFu : 0u) | (qf[2 * j + 1] > 0.0f ? 0xFFFF0000u : 0u);
+    }
+    const size_t rec_stride = (size_t)a.num_kv_heads * TWL_META_RECORD_BYTES;
+    const uint8_t* base = a.meta + (size_t)kvh * TWL_META_RECORD_BYTES + 16 * c;
+    float keep = 0.0f;  // lane i ends up with the score of page p0 + i
+
+#pragma unroll
+    for (int i0 = 0; i0 < kQsPagesPerWave; i0 += 2 * kQsUnroll) {
+      if (i0 >= np) break;
+      u32x4 mm[kQsUnroll];
+#pragma unroll
+      for (int u = 0; u < kQsUnroll; ++u) {
+        const int ia = i0 + 2 * u, ib = ia + 1;
+        const int pa = __builtin_amdgcn_readlane(my_phys, (ia < np) ? ia : 0);
+        const int pb = __builtin_amdgcn_readlane(my_phys, (ib < np) ? ib : 0);
+        const int phys = half ? pb : pa;
+        mm[u] = __builtin_nontemporal_load((const u32x4*)(base + (size_t)phys * rec_stride));
+      }
+#pragma unroll
+      for (int u = 0; u < kQsUnroll; ++u) {
+        // words: x,y = min[4c..4c+3], z,w = max[4c..4c+3]
+        const uint32_t s0 = (mm[u].z & selmask[0]) | (mm[u].x & ~selmask[0]);
+        const uint32_t s1 = (mm[u].w & selmask[1]) | (mm[u].y & ~selmask[1]);
+        float acc;
+        if (DT == TWL_F16) {
+          acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, s0),
+                                       __builtin_bit_cast(half2_t, qw[0]), 0.0f, false);
+          acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, s1),
+                                       __builtin_bit_cast(half2_t, qw[1]), acc, false);
+        } else {
+          acc = qf[0] * as_f32(s0 << 16);
+          acc = fmaf(qf[1], as_f32(s0 & 0xFFFF0000u), acc);
+          acc = fmaf(qf[2], as_f32(s1 << 16), acc);
+          acc = fmaf(qf[3], as_f32(s1 & 0xFFFF0000u), acc);
+        }
+        acc = row16_allreduce<OpSum>(acc);
+        acc += dpp<kDppBcast15, 0xA>(0.0f, acc);  // lanes 16..31 / 48..63 now hold a page total
+        const float sa = as_f32(__builtin_amdgcn_readlane(as_i32(acc), 31));
+        const float sb = as_f32(__builtin_amdgcn_readlane(as_i32(acc), 63));
+        const int ia = i0 + 2 * u;
+        keep = (lane == ia) ? sa : keep;
+        keep = (lane == ia + 1) ? sb : keep;
+      }
+    }
+    // one store per wave: 32 consecutive scores
+    float* orow = a.page_scores + (size_t)row * a.score_stride + p0;
+    if (lane < np) orow[lane] = keep;
+  }
+
 }
 
 }  // namespace twl
@@ -243,6 +258,21 @@ static int check_quest_common(const void* q, int q_dtype, const void* meta,
   return TWL_OK;
 }
 
+static int check_budget(uint32_t token_budget, uint32_t max_pages_per_req, uint32_t sel_stride) {
+  if (token_budget == 0) return TWL_EINVAL;
+  uint64_t k = (token_budget / TWL_PAGE ? token_budget / TWL_PAGE : 1) +
+               (token_budget % TWL_PAGE ? 1 : 0);
+  if (k > max_pages_per_req) k = max_pages_per_req;
+  return sel_stride < k ? TWL_EINVAL : TWL_OK;
+}
+
+static void launch_score(int q_dtype, dim3 grid, hipStream_t s, const twl::QuestArgs& a) {
+  if (q_dtype == TWL_F16)
+    hipLaunchKernelGGL((twl::quest_score_kernel<TWL_F16>), grid, dim3(twl::kQsThreads), 0, s, a);
+  else
+    hipLaunchKernelGGL((twl::quest_score_kernel<TWL_BF16>), grid, dim3(twl::kQsThreads), 0, s, a);
+}
+
 extern "C" int twl_quest_page_scores(const void* q, int q_dtype, const void* meta,
                                      const int32_t* kv_page_indices,
                                      const int32_t* kv_page_indptr, uint32_t batch,
@@ -253,19 +283,13 @@ extern "C" int twl_quest_page_scores(const void* q, int q_dtype, const void* met
                               num_q_heads, num_kv_heads, max_pages_per_req, page_scores,
                               score_stride);
   if (rc != TWL_OK) return rc;
-  twl::QuestScoreArgs sa{};
-  sa.q = q; sa.meta = (const uint8_t*)meta; sa.kv_page_indices = kv_page_indices;
-  sa.kv_page_indptr = kv_page_indptr; sa.num_q_heads = num_q_heads; sa.num_kv_heads = num_kv_heads;
-  sa.max_pages = max_pages_per_req;
-  sa.page_scores = page_scores; sa.score_stride = score_stride;
+  twl::QuestArgs a{};
+  a.q = q; a.meta = (const uint8_t*)meta; a.kv_page_indices = kv_page_indices;
+  a.kv_page_indptr = kv_page_indptr; a.num_q_heads = num_q_heads; a.num_kv_heads = num_kv_heads;
+  a.max_pages = max_pages_per_req; a.page_scores = page_scores; a.score_stride = score_stride;
   dim3 grid((max_pages_per_req + twl::kQsPagesPerBlock - 1) / twl::kQsPagesPerBlock,
             batch * num_q_heads);
-  if (q_dtype == TWL_F16)
-    hipLaunchKernelGGL((twl::quest_score_kernel<TWL_F16>), grid, dim3(twl::kQsThreads), 0,
-                       (hipStream_t)stream, sa);
-  else
-    hipLaunchKernelGGL((twl::quest_score_kernel<TWL_BF16>), grid, dim3(twl::kQsThreads), 0,
-                       (hipStream_t)stream, sa);
+  launch_score(q_dtype, grid, (hipStream_t)stream, a);
   return hipGetLastError() == hipSuccess ? TWL_OK : TWL_ELAUNCH;
 }
 
@@ -278,32 +302,28 @@ extern "C" int twl_quest_topk_pages(const float* page_scores, uint32_t score_str
   if (batch == 0 || num_q_heads == 0) return TWL_EINVAL;
   if (max_pages_per_req == 0 || max_pages_per_req > 16384 || score_stride < max_pages_per_req)
     return TWL_EINVAL;
-  if (token_budget == 0) return TWL_EINVAL;
-  {
-    uint64_t k = (token_budget / TWL_PAGE ? token_budget / TWL_PAGE : 1) +
-                 (token_budget % TWL_PAGE ? 1 : 0);
-    if (k > max_pages_per_req) k = max_pages_per_req;
-    if (sel_stride < k) return TWL_EINVAL;
-  }
+  int rc = check_budget(token_budget, max_pages_per_req, sel_stride);
+  if (rc != TWL_OK) return rc;
   if ((uint64_t)batch * num_q_heads > 65535u) return TWL_EINVAL;
   if (((uintptr_t)page_scores) & 3u) return TWL_EALIGN;
   hipStream_t s = (hipStream_t)stream;
   const uint32_t rows = batch * num_q_heads;
-  twl::QuestSelectArgs ta{};
-  ta.page_scores = page_scores; ta.score_stride = score_stride; ta.kv_page_indptr = kv_page_indptr;
-  ta.num_q_heads = num_q_heads; ta.max_pages = max_pages_per_req; ta.token_budget = token_budget;
-  ta.sel_pages = sel_pages; ta.sel_stride = sel_stride; ta.sel_count = sel_count;
+  twl::QuestArgs a{};
+  a.page_scores = const_cast<float*>(page_scores); a.score_stride = score_stride;
+  a.kv_page_indptr = kv_page_indptr; a.num_q_heads = num_q_heads; a.max_pages = max_pages_per_req;
+  a.token_budget = token_budget; a.sel_pages = sel_pages; a.sel_stride = sel_stride;
+  a.sel_count = sel_count;
   const uint32_t n = max_pages_per_req;
   if (n <= 512)
-    hipLaunchKernelGGL((twl::quest_select_kernel<256, 2>), dim3(rows), dim3(256), 0, s, ta);
+    hipLaunchKernelGGL((twl::quest_select_kernel<256, 2>), dim3(rows), dim3(256), 0, s, a);
   else if (n <= 2048)
-    hipLaunchKernelGGL((twl::quest_select_kernel<1024, 2>), dim3(rows), dim3(1024), 0, s, ta);
+    hipLaunchKernelGGL((twl::quest_select_kernel<1024, 2>), dim3(rows), dim3(1024), 0, s, a);
   else if (n <= 4096)
-    hipLaunchKernelGGL((twl::quest_select_kernel<1024, 4>), dim3(rows), dim3(1024), 0, s, ta);
+    hipLaunchKernelGGL((twl::quest_select_kernel<1024, 4>), dim3(rows), dim3(1024), 0, s, a);
   else if (n <= 8192)
-    hipLaunchKernelGGL((twl::quest_select_kernel<1024, 8>), dim3(rows), dim3(1024), 0, s, ta);
+    hipLaunchKernelGGL((twl::quest_select_kernel<1024, 8>), dim3(rows), dim3(1024), 0, s, a);
   else
-    hipLaunchKernelGGL((twl::quest_select_kernel<1024, 16>), dim3(rows), dim3(1024), 0, s, ta);
+    hipLaunchKernelGGL((twl::quest_select_kernel<1024, 16>), dim3(rows), dim3(1024), 0, s, a);
   return hipGetLastError() == hipSuccess ? TWL_OK : TWL_ELAUNCH;
 }
 
@@ -314,16 +334,11 @@ extern "C" int twl_quest_select(const void* q, int q_dtype, const void* meta,
                                 int32_t* sel_pages, uint32_t sel_stride, int32_t* sel_count,
                                 float* page_scores, uint32_t score_stride, void* stream) {
   if (!sel_pages || !sel_count) return TWL_ENULL;
-  if (token_budget == 0) return TWL_EINVAL;
-  {
-    uint64_t k = (token_budget / TWL_PAGE ? token_budget / TWL_PAGE : 1) +
-                 (token_budget % TWL_PAGE ? 1 : 0);
-    if (k > max_pages_per_req) k = max_pages_per_req;
-    if (sel_stride < k) return TWL_EINVAL;
-  }
-  int rc = twl_quest_page_scores(q, q_dtype, meta, kv_page_indices, kv_page_indptr, batch,
-                                 num_q_heads, num_kv_heads, max_pages_per_req, page_scores,
-                                 score_stride, stream);
+  int rc = check_budget(token_budget, max_pages_per_req, sel_stride);
+  if (rc != TWL_OK) return rc;
+  rc = twl_quest_page_scores(q, q_dtype, meta, kv_page_indices, kv_page_indptr, batch,
+                             num_q_heads, num_kv_heads, max_pages_per_req, page_scores,
+                             score_stride, stream);
   if (rc != TWL_OK) return rc;
   return twl_quest_topk_pages(page_scores, score_stride, kv_page_indptr, batch, num_q_heads,
                               token_budget, max_pages_per_req, sel_pages, sel_stride, sel_count,
