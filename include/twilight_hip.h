@@ -129,16 +129,37 @@ int twl_gemv_int4(const void* q, int q_dtype, float* out, uint32_t out_stride, i
                   uint32_t num_q_heads, uint32_t num_kv_heads, uint32_t max_pages_per_row,
                   float sm_scale, void* stream);
 
-/* Same GEMV in the tensor layout of benchmark/efficiency/bench_gemv.py:390-454: k_u8
- * [max_pages, page_size, num_heads, 64] uint8 (low nibble = even element), scales / zeros fp16
- * [max_pages, page_size, num_heads] (one group per token), q fp16 [batch, num_heads, 128], o fp16
+/* ---------------------------------------------------------------------------------------------
+ * Token-granular paged score GEMVs in the tensor layouts (and call shapes) of the absent
+ * ftka.cuda_ops.gemv module, as used by benchmark/efficiency/bench_gemv.py. K cache
+ * [max_pages, page_size, num_heads, 128 elements]; q fp16 [batch, num_heads, 128]; o fp16
  * [batch, num_heads, o_stride] written in place for n < request length; one page list per request
- * shared by all heads. */
+ * shared by all heads.
+ *   twl_gemv_int4_nhd  batched_sparse_gemv_int4_k, bench_gemv.py:445-454: k_u8 [.., 64] uint8 (low
+ *                      nibble = even element), scales / zeros fp16 [max_pages, page_size, heads],
+ *                      dequant k*scale + zero (:181)
+ *   twl_gemv_int8_nhd  batched_sparse_gemv_int8_k, bench_gemv.py:135-144: k_u8 [.., 128] uint8 =
+ *                      int8 value + 128 (:78,93), same scales / zeros
+ *   twl_gemv_f16_nhd   batched_sparse_gemv, bench_gemv.py:234-241: fp16 K cache
+ *   twl_gemv_f16_single  single_sparse_gemv, bench_gemv.py:33: q [heads,128], k [seq,heads,128],
+ *                      o [heads, seq]
+ * ------------------------------------------------------------------------------------------- */
 int twl_gemv_int4_nhd(const void* q, void* o, uint32_t o_stride, const uint8_t* k_u8,
                       const void* scales, const void* zeros, const int32_t* kv_page_indices,
                       const int32_t* kv_page_indptr, const int32_t* kv_last_page_len,
                       uint32_t batch, uint32_t num_heads, uint32_t page_size,
                       uint32_t max_pages_per_req, float sm_scale, void* stream);
+int twl_gemv_int8_nhd(const void* q, void* o, uint32_t o_stride, const uint8_t* k_u8,
+                      const void* scales, const void* zeros, const int32_t* kv_page_indices,
+                      const int32_t* kv_page_indptr, const int32_t* kv_last_page_len,
+                      uint32_t batch, uint32_t num_heads, uint32_t page_size,
+                      uint32_t max_pages_per_req, float sm_scale, void* stream);
+int twl_gemv_f16_nhd(const void* q, void* o, uint32_t o_stride, const void* k_cache,
+                     const int32_t* kv_page_indices, const int32_t* kv_page_indptr,
+                     const int32_t* kv_last_page_len, uint32_t batch, uint32_t num_heads,
+                     uint32_t page_size, uint32_t max_pages_per_req, float sm_scale, void* stream);
+int twl_gemv_f16_single(const void* q, void* o, const void* k, uint32_t num_heads,
+                        uint32_t seq_len, float sm_scale, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Sparse paged decode attention over survivor lists.

@@ -46,7 +46,7 @@ def assert_scores_close(got, want, rtol=1e-3, atol_frac=1e-4):
     assert np.array_equal(got[~finite], want[~finite])
     w = np.where(finite, want, 0.0)
     rms = np.sqrt((w ** 2).sum(-1, keepdims=True) / np.maximum(finite.sum(-1, keepdims=True), 1))
-    err = np.abs(np.where(finite, got - want, 0.0))
+    err = np.abs(np.where(finite, got, 0.0) - w)
     bound = rtol * np.abs(w) + atol_frac * rms + 1e-30
     bad = err > bound
     assert not bad.any(), f"{bad.sum()} scores off; worst err {err.max()} (bound {bound[bad].min()})"

@@ -208,3 +208,52 @@ def test_gemv_full_size_cfg2_sampled_and_linear(dev, paged):
     o2, _ = K.sparse_gemv_int4(q2.to(dev), rec, ids, indptr, last, max_pages=npg)
     err = (o1 + o2 - out).abs().max().item()
     assert err < 2e-5, err
+
+
+def test_ftka_shaped_fp16_int8_and_single_entries(dev):
+    # call shapes of benchmark/efficiency/bench_gemv.py:33 (single), :135-144 (int8), :234-241 (fp16);
+    # the references there are plain matmuls (:36-42, :181, :259-296)
+    B, H, page_size, pages = 2, 4, 2, 40
+    g = torch.Generator().manual_seed(12)
+    q = torch.randn((B, H, 128), generator=g).half()
+    k16 = torch.randn((pages, page_size, H, 128), generator=g).half()
+    k_i8 = torch.randint(-128, 128, (pages, page_size, H, 128), generator=g, dtype=torch.int16)
+    k_u8 = (k_i8 + 128).to(torch.uint8)                                    # bench_gemv.py:93
+    scales = (torch.rand((pages, page_size, H), generator=g) * 0.02 + 0.001).half()
+    zeros = (torch.randn((pages, page_size, H), generator=g) * 0.1).half()
+    per_req = [13, 20]
+    idx = torch.randperm(pages, generator=g)[:sum(per_req)].to(torch.int32)
+    indptr = torch.tensor([0, 13, 33], dtype=torch.int32)
+    last = torch.tensor([1, 2], dtype=torch.int32)
+    N = 20 * page_size
+    d = lambda t: t.to(dev)
+    o16 = torch.full((B, H, 1, N), 9.0, dtype=torch.float16, device=dev)
+    K.batched_sparse_gemv(d(q), o16, d(k16), d(idx), d(indptr), d(last))
+    o8 = torch.full((B, H, N), 9.0, dtype=torch.float16, device=dev)
+    K.batched_sparse_gemv_int8_k(d(q), o8, d(k_u8), d(scales), d(zeros), d(idx), d(indptr), d(last))
+    deq8 = k_i8.float() * scales.float()[..., None] + zeros.float()[..., None]
+    for b in range(B):
+        n_tok = (per_req[b] - 1) * page_size + int(last[b])
+        phys = idx[indptr[b]:indptr[b + 1]].long()
+        w16 = torch.einsum("hd,nhd->hn", q[b].double(), k16[phys].reshape(-1, H, 128)[:n_tok].double())
+        assert torch.allclose(o16.cpu()[b, :, 0, :n_tok].double(), w16, rtol=2e-3, atol=2e-2)
+        w8 = torch.einsum("hd,nhd->hn", q[b].double(), deq8[phys].reshape(-1, H, 128)[:n_tok].double())
+        assert torch.allclose(o8.cpu()[b, :, :n_tok].double(), w8, rtol=2e-3, atol=2e-2)
+        assert torch.all(o16.cpu()[b, :, 0, n_tok:] == 9.0) and torch.all(o8.cpu()[b, :, n_tok:] == 9.0)
+    # constant case of bench_gemv.py:80-112: int8 value 3, scale 1, zero 0, q = 1 -> 384
+    ones_q = torch.ones((1, 2, 128), dtype=torch.float16, device=dev)
+    k3 = torch.full((8, 1, 2, 128), 131, dtype=torch.uint8, device=dev)
+    o3 = torch.zeros((1, 2, 8), dtype=torch.float16, device=dev)
+    K.batched_sparse_gemv_int8_k(ones_q, o3, k3, torch.ones((8, 1, 2), dtype=torch.float16, device=dev),
+                                 torch.zeros((8, 1, 2), dtype=torch.float16, device=dev),
+                                 torch.arange(8, dtype=torch.int32, device=dev),
+                                 torch.tensor([0, 8], dtype=torch.int32, device=dev),
+                                 torch.ones(1, dtype=torch.int32, device=dev))
+    assert torch.all(o3 == 384.0)
+    # single request (bench_gemv.py:23-42)
+    qs = torch.randn((H, 128), generator=g).half()
+    ks = torch.randn((77, H, 128), generator=g).half()
+    os_ = torch.empty((H, 77), dtype=torch.float16, device=dev)
+    K.single_sparse_gemv(d(qs), os_, d(ks))
+    ref = torch.matmul(qs.double().unsqueeze(1), ks.double().transpose(0, 1).transpose(1, 2)).squeeze(1)
+    assert torch.allclose(os_.cpu().double(), ref, rtol=1e-2, atol=2e-2)      # tolerances of :41-42

@@ -23,7 +23,8 @@ MAX_CANDIDATES = 32768
 # every symbol include/twilight_hip.h declares
 EXPORTS = (
     "twl_strerror", "twl_abi_version", "twl_device_count", "twl_top_p_f32", "twl_top_p_f16",
-    "twl_softmax_top_p_f32", "twl_gemv_int4", "twl_gemv_int4_nhd", "twl_sparse_attn",
+    "twl_softmax_top_p_f32", "twl_gemv_int4", "twl_gemv_int4_nhd",
+    "twl_gemv_int8_nhd", "twl_gemv_f16_nhd", "twl_gemv_f16_single", "twl_sparse_attn",
     "twl_sparse_attn_workspace_bytes", "twl_quest_select",
     "twl_quest_page_scores", "twl_quest_topk_pages", "twl_kv_shadow_build", "twl_dequant_int4",
     "twl_decode_layer",
@@ -77,6 +78,9 @@ def lib() -> ctypes.CDLL:
     L.twl_gemv_int4.argtypes = [vp, i32, vp, u32, vp, vp, vp, vp, u32, vp, vp, vp, u32, u32, u32,
                                 u32, f32, vp]
     L.twl_gemv_int4_nhd.argtypes = [vp, vp, u32, vp, vp, vp, vp, vp, vp, u32, u32, u32, u32, f32, vp]
+    L.twl_gemv_int8_nhd.argtypes = L.twl_gemv_int4_nhd.argtypes
+    L.twl_gemv_f16_nhd.argtypes = [vp, vp, u32, vp, vp, vp, vp, u32, u32, u32, u32, f32, vp]
+    L.twl_gemv_f16_single.argtypes = [vp, vp, vp, u32, u32, f32, vp]
     L.twl_sparse_attn.argtypes = [vp, vp, i32, vp, vp, u64, u64, u64, vp, u32, vp, vp, vp, u32, u32,
                                   u32, f32, vp, vp, u64, vp]
     L.twl_sparse_attn_workspace_bytes.argtypes = [u32, u32]

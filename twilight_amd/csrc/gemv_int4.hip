@@ -220,84 +220,6 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_int4_kernel(GemvArgs a) {
   }
 }
 
-// ---- the same arithmetic over the tensor layout of benchmark/efficiency/bench_gemv.py:390-454 ---
-struct GemvNhdArgs {
-  const uint16_t* q;
-  uint16_t* o;
-  uint32_t o_stride;
-  const uint8_t* k_u8;
-  const uint16_t* scales;
-  const uint16_t* zeros;
-  const int32_t* kv_page_indices;
-  const int32_t* kv_page_indptr;
-  const int32_t* kv_last_page_len;
-  uint32_t num_heads;
-  uint32_t page_size;
-  uint32_t max_tok;  // tokens per request the grid and the output row are sized for
-  float sm_scale;
-};
-
-// One wavefront scores 16 tokens per step: lane l -> token l/4 of the step, 32-element slice l%4.
-// A token's 64 nibble bytes are contiguous; scale / zero are per token.
-__global__ __launch_bounds__(kGemvThreads) void gemv_int4_nhd_kernel(GemvNhdArgs a) {
-  const uint32_t row = blockIdx.y;
-  const uint32_t b = row / a.num_heads;
-  const uint32_t h = row - b * a.num_heads;
-  const int lane = lane_id();
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-  const int g = lane & 3;
-  const int t = lane >> 2;
-
-  const int pg_begin = a.kv_page_indptr[b];
-  const int req_pages = a.kv_page_indptr[b + 1] - pg_begin;
-  if (req_pages <= 0) return;
-  const int n_tok = min((req_pages - 1) * (int)a.page_size + a.kv_last_page_len[b], (int)a.max_tok);
-
-  half2_t qp[16];
-  float qsum = 0.0f;
-  {
-    const uint16_t* qrow = a.q + (size_t)row * TWL_HEAD_DIM + 32 * g;
-    float qf[32];
-#pragma unroll
-    for (int i = 0; i < 32; ++i) qf[i] = f16_bits_to_f32(qrow[i]);
-#pragma unroll
-    for (int w = 0; w < 4; ++w)
-#pragma unroll
-      for (int s = 0; s < 4; ++s) {
-        half2_t pr = {(_Float16)qf[8 * w + s], (_Float16)qf[8 * w + s + 4]};
-        qp[4 * w + s] = pr;
-      }
-#pragma unroll
-    for (int i = 0; i < 32; ++i) qsum += qf[i];
-  }
-
-  constexpr int kTokPerBlock = 16 * 4 * 4;  // 4 waves x 4 steps x 16 tokens
-  const int n0 = blockIdx.x * kTokPerBlock + wave * 64;
-#pragma unroll
-  for (int s = 0; s < 4; ++s) {
-    const int n = n0 + 16 * s + t;
-    if (n < n_tok) {
-      const int lp = n / (int)a.page_size;
-      const int slot = n - lp * (int)a.page_size;
-      const size_t tok = ((size_t)a.kv_page_indices[pg_begin + lp] * a.page_size + slot) *
-                             a.num_heads + h;
-      u32x4 nib = *(const u32x4*)(a.k_u8 + tok * 64 + 16 * g);
-      const float scale = f16_bits_to_f32(a.scales[tok]);
-      const float zero = f16_bits_to_f32(a.zeros[tok]);
-      float acc = 0.0f;
-      acc = dot8_nibbles(nib.x, qp + 0, acc);
-      acc = dot8_nibbles(nib.y, qp + 4, acc);
-      acc = dot8_nibbles(nib.z, qp + 8, acc);
-      acc = dot8_nibbles(nib.w, qp + 12, acc);
-      float part = fmaf(scale * 64.0f, acc - qsum, zero * qsum);
-      // tokens are aligned to quads, so all four lanes of a quad take this branch together
-      part = quad_allreduce<OpSum>(part);
-      if (g == 0)
-        a.o[(size_t)row * a.o_stride + n] = (uint16_t)f32_to_f16_bits(part * a.sm_scale);
-    }
-  }
-}
-
 }  // namespace twl
 
 extern "C" int twl_gemv_int4(const void* q, int q_dtype, float* out, uint32_t out_stride,
@@ -339,31 +261,3 @@ extern "C" int twl_gemv_int4(const void* q, int q_dtype, float* out, uint32_t ou
   return hipGetLastError() == hipSuccess ? TWL_OK : TWL_ELAUNCH;
 }
 
-extern "C" int twl_gemv_int4_nhd(const void* q, void* o, uint32_t o_stride, const uint8_t* k_u8,
-                                 const void* scales, const void* zeros,
-                                 const int32_t* kv_page_indices, const int32_t* kv_page_indptr,
-                                 const int32_t* kv_last_page_len, uint32_t batch,
-                                 uint32_t num_heads, uint32_t page_size,
-                                 uint32_t max_pages_per_req, float sm_scale, void* stream) {
-  if (!q || !o || !k_u8 || !scales || !zeros || !kv_page_indices || !kv_page_indptr ||
-      !kv_last_page_len)
-    return TWL_ENULL;
-  if (batch == 0 || num_heads == 0 || page_size == 0 || max_pages_per_req == 0) return TWL_EINVAL;
-  if ((uint64_t)max_pages_per_req * page_size > o_stride) return TWL_EINVAL;
-  if ((uint64_t)batch * num_heads > 65535u) return TWL_EINVAL;
-  if ((((uintptr_t)k_u8) & 15u) || (((uintptr_t)q) & 1u) || (((uintptr_t)o) & 1u))
-    return TWL_EALIGN;
-  twl::GemvNhdArgs a{};
-  a.q = (const uint16_t*)q; a.o = (uint16_t*)o; a.o_stride = o_stride; a.k_u8 = k_u8;
-  a.scales = (const uint16_t*)scales; a.zeros = (const uint16_t*)zeros;
-  a.kv_page_indices = kv_page_indices; a.kv_page_indptr = kv_page_indptr;
-  a.kv_last_page_len = kv_last_page_len; a.num_heads = num_heads; a.page_size = page_size;
-  a.sm_scale = sm_scale;
-  const uint64_t max_tok = (uint64_t)max_pages_per_req * page_size;
-  if (max_tok > 0x7FFFFFFFull) return TWL_EINVAL;
-  a.max_tok = (uint32_t)max_tok;
-  dim3 grid((uint32_t)((max_tok + 255) / 256), batch * num_heads);
-  hipLaunchKernelGGL(twl::gemv_int4_nhd_kernel, grid, dim3(twl::kGemvThreads), 0,
-                     (hipStream_t)stream, a);
-  return hipGetLastError() == hipSuccess ? TWL_OK : TWL_ELAUNCH;
-}

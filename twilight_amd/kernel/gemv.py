@@ -129,3 +129,93 @@ def batched_sparse_gemv_int4_k(q: torch.Tensor, o: torch.Tensor, k_u8: torch.Ten
             ptr(kv_page_indices), ptr(kv_page_indptr), ptr(kv_last_page_len), B, H, page_size,
             max_pages_per_req, float(sm_scale), stream_of(q))
     _lib.check(rc, "BatchedSparseGemvInt4K")
+
+
+def _check_nhd_common(q, o, k_cache, last_dim, kv_page_indices, kv_page_indptr, kv_last_page_len,
+                      o_dims):
+    check_input(q, "q"); check_dim(3, q, "q"); check_dtype(q, torch.float16, "q")
+    check_input(o, "o"); check_dim(o_dims, o, "o"); check_dtype(o, torch.float16, "o")
+    check_input(k_cache, "k_cache"); check_dim(4, k_cache, "k_cache")
+    B, H, D = q.shape
+    if D != _lib.HEAD_DIM or k_cache.size(3) != last_dim or k_cache.size(2) != H:
+        raise RuntimeError(f"k_cache must be [max_pages, page_size, num_heads, {last_dim}]")
+    for name, t in (("kv_page_indices", kv_page_indices), ("kv_page_indptr", kv_page_indptr),
+                    ("kv_last_page_len", kv_last_page_len)):
+        check_input(t, name); check_dtype(t, torch.int32, name)
+    if o.size(0) != B or o.size(1) != H:
+        raise RuntimeError("o must be fp16 [B, H, (1,) N]")
+    if kv_page_indptr.numel() != B + 1 or kv_last_page_len.numel() != B:
+        raise RuntimeError("kv_page_indptr must have B+1 and kv_last_page_len B elements")
+    check_same_device(q, ("o", o), ("k_cache", k_cache), ("kv_page_indices", kv_page_indices),
+                      ("kv_page_indptr", kv_page_indptr), ("kv_last_page_len", kv_last_page_len))
+    page_size = k_cache.size(1)
+    n_out = o.size(-1)
+    if n_out // page_size == 0:
+        raise RuntimeError("o is shorter than one page")
+    return B, H, page_size, n_out
+
+
+def batched_sparse_gemv(q: torch.Tensor, o: torch.Tensor, k_cache: torch.Tensor,
+                        kv_page_indices: torch.Tensor, kv_page_indptr: torch.Tensor,
+                        kv_last_page_len: torch.Tensor, sm_scale: float = 1.0) -> None:
+    """Call shape of ``ftka.cuda_ops.gemv.batched_sparse_gemv`` at
+    benchmark/efficiency/bench_gemv.py:234-241: ``o[b,h,0,n] = q[b,h,:] . k_cache[token n of b]``.
+
+    ``q`` fp16 [B,H,128]; ``o`` fp16 [B,H,1,N] written in place; ``k_cache`` fp16
+    [max_pages, page_size, H, 128]; CSR page list per request.
+    """
+    B, H, page_size, n_out = _check_nhd_common(q, o, k_cache, _lib.HEAD_DIM, kv_page_indices,
+                                               kv_page_indptr, kv_last_page_len, 4)
+    check_dtype(k_cache, torch.float16, "k_cache")
+    if o.size(2) != 1:
+        raise RuntimeError("o must be fp16 [B, H, 1, N]")
+    with torch.cuda.device(q.device):
+        rc = _lib.lib().twl_gemv_f16_nhd(ptr(q), ptr(o), n_out, ptr(k_cache), ptr(kv_page_indices),
+                                         ptr(kv_page_indptr), ptr(kv_last_page_len), B, H,
+                                         page_size, n_out // page_size, float(sm_scale),
+                                         stream_of(q))
+    _lib.check(rc, "BatchedSparseGemv")
+
+
+def batched_sparse_gemv_int8_k(q: torch.Tensor, o: torch.Tensor, k_u8: torch.Tensor,
+                               quant_scales: torch.Tensor, quant_zeros: torch.Tensor,
+                               kv_page_indices: torch.Tensor, kv_page_indptr: torch.Tensor,
+                               kv_last_page_len: torch.Tensor, sm_scale: float = 1.0) -> None:
+    """Call shape of ``ftka.cuda_ops.gemv.batched_sparse_gemv_int8_k`` at
+    benchmark/efficiency/bench_gemv.py:135-144: ``k_u8`` uint8 [max_pages, page_size, H, 128] holds
+    ``int8 value + 128`` (:78,93); dequant ``(k_u8 - 128) * scale + zero`` with per-token fp16
+    ``quant_scales`` / ``quant_zeros`` [max_pages, page_size, H] (:181); ``o`` fp16 [B,H,N]."""
+    B, H, page_size, n_out = _check_nhd_common(q, o, k_u8, _lib.HEAD_DIM, kv_page_indices,
+                                               kv_page_indptr, kv_last_page_len, 3)
+    check_dtype(k_u8, torch.uint8, "k_cache")
+    for name, t in (("quant_scales", quant_scales), ("quant_zeros", quant_zeros)):
+        check_input(t, name); check_dtype(t, torch.float16, name)
+        if tuple(t.shape) != tuple(k_u8.shape[:3]):
+            raise RuntimeError(f"{name} must be fp16 [max_pages, page_size, num_heads]")
+    check_same_device(q, ("quant_scales", quant_scales), ("quant_zeros", quant_zeros))
+    with torch.cuda.device(q.device):
+        rc = _lib.lib().twl_gemv_int8_nhd(ptr(q), ptr(o), n_out, ptr(k_u8), ptr(quant_scales),
+                                          ptr(quant_zeros), ptr(kv_page_indices),
+                                          ptr(kv_page_indptr), ptr(kv_last_page_len), B, H,
+                                          page_size, n_out // page_size, float(sm_scale),
+                                          stream_of(q))
+    _lib.check(rc, "BatchedSparseGemvInt8K")
+
+
+def single_sparse_gemv(q: torch.Tensor, o: torch.Tensor, k: torch.Tensor,
+                       sm_scale: float = 1.0) -> None:
+    """Call shape of ``ftka.cuda_ops.gemv.single_sparse_gemv`` at
+    benchmark/efficiency/bench_gemv.py:33: ``o[h,n] = q[h,:] . k[n,h,:]`` for one request;
+    ``q`` fp16 [H,128], ``k`` fp16 [N,H,128], ``o`` fp16 [H,N] written in place."""
+    check_input(q, "q"); check_dim(2, q, "q"); check_dtype(q, torch.float16, "q")
+    check_input(k, "k"); check_dim(3, k, "k"); check_dtype(k, torch.float16, "k")
+    check_input(o, "o"); check_dim(2, o, "o"); check_dtype(o, torch.float16, "o")
+    H, D = q.shape
+    N = k.size(0)
+    if D != _lib.HEAD_DIM or k.size(1) != H or k.size(2) != D or tuple(o.shape) != (H, N) or N == 0:
+        raise RuntimeError("shapes must be q [H,128], k [N,H,128], o [H,N]")
+    check_same_device(q, ("k", k), ("o", o))
+    with torch.cuda.device(q.device):
+        rc = _lib.lib().twl_gemv_f16_single(ptr(q), ptr(o), ptr(k), H, N, float(sm_scale),
+                                            stream_of(q))
+    _lib.check(rc, "SingleSparseGemv")
