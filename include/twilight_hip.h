@@ -230,6 +230,23 @@ int twl_kv_shadow_build(const void* k_cache, int kv_dtype, uint64_t page_stride,
 int twl_dequant_int4(const void* k_int4, uint32_t num_records, float* out, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
+ * Double-Sparse label ops (strides are in elements).
+ * twl_get_label_tensor replaces get_label_tensor, twilight/kernel/triton/channel.py:11-79:
+ *   out[l,h,c] = x[l,h,channel[h,c]], elements of elem_bytes (2 or 4) bytes, channel int64.
+ * twl_bgemv_int8 replaces bgemv_int8, twilight/kernel/triton/bgemv_int8.py:12-75:
+ *   out[b,h,n] = (sum_c q[b,h,c] * k[b*n_ctx+n,h,c]) * scale[b*n_ctx+n,h]; q / scale / out fp16,
+ *   k int8, fp32 accumulation.
+ * ------------------------------------------------------------------------------------------- */
+int twl_get_label_tensor(const void* x, const int64_t* channel, void* out, uint32_t elem_bytes,
+                         uint32_t L, uint32_t H, uint32_t r, int64_t sx_l, int64_t sx_h,
+                         int64_t sx_d, int64_t sc_h, int64_t sc_c, int64_t so_l, int64_t so_h,
+                         int64_t so_c, void* stream);
+int twl_bgemv_int8(const void* q_label, const int8_t* k_label, const void* k_scales, void* out,
+                   uint32_t B, uint32_t H, uint32_t r, uint32_t n_ctx, int64_t sq_b, int64_t sq_h,
+                   int64_t sq_d, int64_t sk_t, int64_t sk_h, int64_t sk_d, int64_t ss_t,
+                   int64_t ss_h, int64_t so_b, int64_t so_h, int64_t so_n, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
  * The whole decode layer on one stream: quest select -> INT4 GEMV -> softmax + top-p -> sparse
  * attention (twilight/pyimpl/attention.py:188-306 for q_len == 1). Every intermediate is a
  * caller-provided buffer (see the field comments); no host synchronisation happens inside.

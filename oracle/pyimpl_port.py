@@ -287,3 +287,25 @@ def mask_to_lists(mask: torch.Tensor) -> Tuple[np.ndarray, np.ndarray]:
         nz = np.nonzero(m[r])[0]
         idx[r, :nz.size] = nz
     return idx, count
+
+
+# --------------------------------------------------------------------------------------------
+# Double-Sparse label ops (the reference's own torch references)
+# --------------------------------------------------------------------------------------------
+def get_label_tensor_ref(x: torch.Tensor, channel: torch.Tensor, r: int) -> torch.Tensor:
+    """The indexing twilight/kernel/triton/channel.py:98-101 checks against: X[i, j, channel[j]]."""
+    L, H, _ = x.shape
+    out = torch.empty((L, H, r), dtype=x.dtype)
+    for h in range(H):
+        out[:, h] = x[:, h, channel[h, :r]]
+    return out
+
+
+def bgemv_int8_ref(q_label: torch.Tensor, k_label: torch.Tensor, k_scales: torch.Tensor):
+    """torch_bgemv_int8, twilight/kernel/triton/bgemv_int8.py:78-93, evaluated in fp32."""
+    B, H, r = q_label.shape
+    n_ctx = k_label.shape[0] // B
+    k = k_label.float() * k_scales.float()[:, :, None]                       # bgemv_int8.py:83
+    q = q_label.float().view(B, H, 1, r)                                      # :86
+    k = k.view(B, n_ctx, H, r).transpose(1, 2).transpose(2, 3)                # :87
+    return torch.matmul(q, k).squeeze(-2)                                     # :89

@@ -1,0 +1,58 @@
+"""GPU parity of the Double-Sparse label ops against the reference's own torch checks
+(twilight/kernel/triton/channel.py:82-106, twilight/kernel/triton/bgemv_int8.py:78-134)."""
+import pytest
+import torch
+
+from oracle import pyimpl_port as P
+import twilight_amd.kernel as K
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dt", [torch.float32, torch.float16, torch.bfloat16])
+def test_get_label_tensor(dev, dt):
+    # shapes of the reference's self-test (channel.py:84-93) and a larger strided case
+    g = torch.Generator().manual_seed(0)
+    for (L, H, D, r) in ((10, 3, 8, 4), (257, 32, 128, 16)):
+        x = torch.randn((L, H, D), generator=g).to(dt)
+        channel = torch.stack([torch.randperm(D, generator=g)[:r] for _ in range(H)]).to(torch.int64)
+        out = torch.empty((L, H, r), dtype=dt, device=dev)
+        K.get_label_tensor(x.to(dev), channel.to(dev), out, r)
+        assert torch.equal(out.cpu(), P.get_label_tensor_ref(x, channel, r))     # a gather: exact
+    # non-contiguous input view, as double_sparse.py:72-77 produces before .contiguous()
+    xs = torch.randn((4, 50, 6, 128), generator=g).to(dt)                        # [B,N,H,D]
+    xv = xs.to(dev).transpose(1, 2)[1].transpose(0, 1)                           # [N,H,D] strided
+    out = torch.empty((50, 6, 8), dtype=dt, device=dev)
+    ch = torch.stack([torch.randperm(128, generator=g)[:8] for _ in range(6)]).to(torch.int64)
+    K.get_label_tensor(xv, ch.to(dev), out, 8)
+    assert torch.equal(out.cpu(), P.get_label_tensor_ref(xs[1], ch, 8))
+
+
+def test_bgemv_int8_reference_selftest_shape(dev):
+    # the reference's own check: B = H = 32, N_CTX = 2048, r = 8, normal(0.1, 0.2), atol 1e-3 rtol 0
+    # (bgemv_int8.py:98-134)
+    B, H, N, r = 32, 32, 2048, 8
+    g = torch.Generator().manual_seed(0)
+    q = (torch.randn((B, H, r), generator=g) * 0.2 + 0.1).half()
+    kf = (torch.randn((B * N, H, r), generator=g) * 0.2 + 0.1).half()
+    scales = (kf.float().abs().max(-1)[0] / 127.0).half()                       # :107
+    k8 = (kf.float() / scales.float()[:, :, None]).to(torch.int8)               # :108
+    out = torch.empty((B, H, N), dtype=torch.float16, device=dev)
+    ret = K.bgemv_int8(q.to(dev), k8.to(dev), scales.to(dev), out)
+    assert ret is out
+    ref = P.bgemv_int8_ref(q, k8, scales)
+    assert torch.allclose(out.cpu().float(), ref, atol=1e-3, rtol=0)
+
+
+def test_bgemv_int8_ragged(dev):
+    B, H, N, r = 3, 5, 131, 16
+    g = torch.Generator().manual_seed(1)
+    q = torch.randn((B, H, r), generator=g).half()
+    k8 = torch.randint(-128, 128, (B * N, H, r), generator=g, dtype=torch.int16).to(torch.int8)
+    scales = (torch.rand((B * N, H), generator=g) * 0.01).half()
+    out = torch.empty((B, H, N), dtype=torch.float16, device=dev)
+    K.bgemv_int8(q.to(dev), k8.to(dev), scales.to(dev), out)
+    ref = P.bgemv_int8_ref(q, k8, scales)
+    assert torch.allclose(out.cpu().float(), ref, atol=2e-3, rtol=2e-3)
+    with pytest.raises(RuntimeError):
+        K.bgemv_int8(q.to(dev), k8.to(dev), scales.to(dev), out[:, :, :-1])

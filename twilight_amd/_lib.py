@@ -7,7 +7,8 @@ from __future__ import annotations
 
 import ctypes
 import os
-from ctypes import POINTER, c_char_p, c_float, c_int, c_int32, c_uint8, c_uint32, c_uint64, c_void_p
+from ctypes import (POINTER, c_char_p, c_float, c_int, c_int32, c_int64, c_uint8, c_uint32,
+                    c_uint64, c_void_p)
 
 from .build import LIB_PATH
 
@@ -27,7 +28,7 @@ EXPORTS = (
     "twl_gemv_int8_nhd", "twl_gemv_f16_nhd", "twl_gemv_f16_single", "twl_sparse_attn",
     "twl_sparse_attn_workspace_bytes", "twl_quest_select",
     "twl_quest_page_scores", "twl_quest_topk_pages", "twl_kv_shadow_build", "twl_dequant_int4",
-    "twl_decode_layer",
+    "twl_decode_layer", "twl_get_label_tensor", "twl_bgemv_int8",
 )
 
 
@@ -91,6 +92,8 @@ def lib() -> ctypes.CDLL:
     L.twl_kv_shadow_build.argtypes = [vp, i32, u64, u64, u64, vp, vp, u32, u32, vp, vp, vp]
     L.twl_dequant_int4.argtypes = [vp, u32, vp, vp]
     L.twl_decode_layer.argtypes = [POINTER(LayerArgs), vp]
+    L.twl_get_label_tensor.argtypes = [vp, vp, vp, u32, u32, u32, u32] + [c_int64] * 8 + [vp]
+    L.twl_bgemv_int8.argtypes = [vp, vp, vp, vp, u32, u32, u32, u32] + [c_int64] * 11 + [vp]
     for name in EXPORTS:
         if name not in ("twl_strerror", "twl_sparse_attn_workspace_bytes"):
             getattr(L, name).restype = c_int
