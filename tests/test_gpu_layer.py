@@ -112,3 +112,73 @@ def test_decode_append_keeps_shadow_fresh(dev):
     oa, ob = a(q).clone(), b(q).clone()
     assert torch.equal(a.sel_pages, b.sel_pages) and torch.equal(a.count, b.count)
     assert torch.equal(oa, ob)
+
+
+def test_full_size_cfg4_layer_sampled_rows_and_properties(dev):
+    # BASELINE config 4 at its full size: B=16, 32 MHA heads, ctx 32768, fp16 paged KV (shuffled
+    # pages), Quest budget 8192, p = 0.95. The oracle (dense, CPU) checks a sample of (batch, head)
+    # rows end to end; size-independent properties check every row.
+    B, H, N, budget, p = 16, 32, 32768, 8192, 0.95
+    npg = N // 16
+    q, k, v, (ids, indptr, last) = synth.layer_inputs_device(B, H, H, N, torch.float16, dev, seed=3)
+    cache = PagedKVCache(B * npg, H, torch.float16, dev)
+    cache.k_cache, cache.v_cache = k, v
+    cache.set_page_table(ids, indptr, last)
+    cache.rebuild_shadow()
+    layer = TwilightDecodeLayer(cache, H, token_budget=budget, top_p=p, high="max")
+    out = layer(q).clone()
+    torch.cuda.synchronize()
+    rows = B * H
+    cnt = layer.count.reshape(rows).cpu().numpy()
+    selc = layer.sel_count.reshape(rows).cpu().numpy()
+    assert np.all(selc == 512) and np.all(cnt >= 1) and np.all(cnt <= 8192)
+    assert torch.isfinite(out.float()).all()
+    # every row: survivors ascending, inside the selected pages, and they carry >= p of the
+    # softmax of the row's own candidate scores
+    sel = layer.sel_pages.reshape(rows, -1)
+    idx = layer.idx.reshape(rows, -1)
+    scores = layer.scores.reshape(rows, -1)
+    probs = torch.softmax(scores, dim=-1)
+    pos = torch.arange(idx.shape[1], device=dev)[None, :]
+    valid = pos < layer.count.reshape(rows, 1)
+    tok = torch.where(valid, idx, torch.full_like(idx, -1))
+    assert bool(((tok[:, 1:] > tok[:, :-1]) | ~valid[:, 1:]).all())
+    page_of = (idx // 16).long()
+    slot = torch.searchsorted(sel.long().contiguous(), page_of.clamp(min=0).contiguous())
+    slot = slot.clamp(max=sel.shape[1] - 1)
+    assert bool(((torch.gather(sel.long(), 1, slot) == page_of) | ~valid).all())
+    cand = slot * 16 + (idx % 16).long()
+    kept = torch.where(valid, torch.gather(probs, 1, cand.clamp(0, probs.shape[1] - 1)), torch.zeros_like(probs[:, :1]).expand_as(cand))
+    assert float(kept.sum(-1).min()) >= p - 1e-5
+    # sampled rows against the dense oracle
+    ids_c = ids.cpu().long()
+    rng = np.random.default_rng(0)
+    long_row = int(np.argmax(cnt))
+    picks = sorted(set([long_row] + [int(r) for r in rng.integers(0, rows, 5)]))
+    tol = 1e-3
+    compared = 0
+    for r in picks:
+        b, h = divmod(r, H)
+        phys = ids_c[b * npg:(b + 1) * npg].to(dev)
+        kd = k[phys, :, h].reshape(N, 128).float().cpu()[None, None]
+        vd = v[phys, :, h].reshape(N, 128).float().cpu()[None, None]
+        qd = q[b, h].float().cpu()[None, None, None]
+        ref = P.decode_layer_dense(qd, kd, vd, top_p=p, token_budget=budget,
+                                   high_mode=native.HIGH_MAX, quant="storage",
+                                   prob_dtype=torch.float16)
+        m0 = np.zeros(N, dtype=bool)
+        for pg in sel[r, :selc[r]].cpu().numpy():
+            m0[pg * 16:(pg + 1) * 16] = True
+        if not np.array_equal(m0, ref["mask0"].reshape(N).numpy()):
+            continue  # a page tied with the 512th score within rounding: rows are incomparable
+        gm = np.zeros((1, N), dtype=bool)
+        gm[0, idx[r, :cnt[r]].cpu().numpy()] = True
+        pr = ref["probs"].reshape(1, N).numpy()
+        _, _, _, margin = native.top_p_mask_f32(pr, p, native.HIGH_MAX, return_margin=True)
+        assert_top_p_parity(pr, p, gm, ref["mask"].reshape(1, N).numpy(), ref["low"], margin,
+                            margin_tol=5e-6)
+        own = P.masked_attention(qd, kd, vd, torch.from_numpy(gm).reshape(1, 1, 1, N),
+                                 prob_dtype=torch.float16 if cnt[r] <= 128 else torch.float32)
+        assert torch.allclose(out[b, h].float().cpu(), own[0, 0, 0], rtol=tol, atol=tol), r
+        compared += 1
+    assert compared >= len(picks) - 1, (compared, len(picks))
