@@ -14,10 +14,12 @@ import twilight_amd.kernel as K
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("dt,N,budget", [(torch.float16, 1000, 256), (torch.float16, 4096, 1000),
-                                         (torch.bfloat16, 777, 64), (torch.float16, 40, 4096)])
-def test_quest_select_vs_dense_reference(dev, dt, N, budget):
-    B, H, Hkv = 2, 4, 2
+@pytest.mark.parametrize("dt,N,budget,H,Hkv", [
+    (torch.float16, 1000, 256, 4, 2), (torch.float16, 4096, 1000, 4, 4),
+    (torch.bfloat16, 777, 64, 8, 2), (torch.float16, 40, 4096, 4, 2),
+    (torch.float16, 600, 100, 8, 1), (torch.bfloat16, 333, 48, 6, 2)])
+def test_quest_select_vs_dense_reference(dev, dt, N, budget, H, Hkv):
+    B = 2
     g = torch.Generator().manual_seed(N)
     q = torch.randn((B, H, 1, 128), generator=g).to(dt)
     k = torch.randn((B, Hkv, N, 128), generator=g).to(dt)

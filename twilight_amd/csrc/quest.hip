@@ -86,16 +86,58 @@ __device__ __forceinline__ void quest_select_row(const QuestArgs& a, uint32_t ro
   }
 
   // ---- radix select of the k-th largest key ------------------------------------------------
-  uint32_t prefix = 0, prefix_mask = 0;
-  int k_rem = k;
+  // Page scores of a row share their sign and most of their exponent, so a pass over the top
+  // byte would pile every key into one or two LDS bins (serialised atomics). The bits that are
+  // common to the row's largest and smallest key are skipped: the first digit starts at the
+  // highest bit in which two keys differ.
+  uint32_t kmax = 0u, kmin = 0xFFFFFFFFu;
 #pragma unroll
-  for (int shift = 24; shift >= 0; shift -= 8) {
+  for (int j = 0; j < VPT; ++j) {
+    kmax = max(kmax, key[j]);
+    kmin = min(kmin, key[j] ? key[j] : 0xFFFFFFFFu);
+  }
+#pragma unroll
+  for (int ctrl_step = 0; ctrl_step < 1; ++ctrl_step) {
+    kmax = max(kmax, (uint32_t)dpp<kDppXor1>(0, (int)kmax));
+    kmin = min(kmin, (uint32_t)dpp<kDppXor1>((int)0xFFFFFFFF, (int)kmin));
+    kmax = max(kmax, (uint32_t)dpp<kDppXor2>(0, (int)kmax));
+    kmin = min(kmin, (uint32_t)dpp<kDppXor2>((int)0xFFFFFFFF, (int)kmin));
+    kmax = max(kmax, (uint32_t)dpp<kDppHalfMirror>(0, (int)kmax));
+    kmin = min(kmin, (uint32_t)dpp<kDppHalfMirror>((int)0xFFFFFFFF, (int)kmin));
+    kmax = max(kmax, (uint32_t)dpp<kDppMirror>(0, (int)kmax));
+    kmin = min(kmin, (uint32_t)dpp<kDppMirror>((int)0xFFFFFFFF, (int)kmin));
+    kmax = max(kmax, (uint32_t)dpp<kDppBcast15, 0xA>(0, (int)kmax));
+    kmin = min(kmin, (uint32_t)dpp<kDppBcast15, 0xA>((int)0xFFFFFFFF, (int)kmin));
+    kmax = max(kmax, (uint32_t)dpp<kDppBcast31, 0xC>(0, (int)kmax));
+    kmin = min(kmin, (uint32_t)dpp<kDppBcast31, 0xC>((int)0xFFFFFFFF, (int)kmin));
+  }
+  if (lane == kWave - 1) {
+    sm.hist[wave] = (int)kmax;
+    sm.hist[16 + wave] = (int)kmin;
+  }
+  __syncthreads();
+  kmax = 0u; kmin = 0xFFFFFFFFu;
+#pragma unroll
+  for (int w = 0; w < NWAVES; ++w) {
+    kmax = max(kmax, (uint32_t)sm.hist[w]);
+    kmin = min(kmin, (uint32_t)sm.hist[16 + w]);
+  }
+  __syncthreads();  // hist is reused below
+  const uint32_t diff = kmax ^ kmin;
+  int top = diff ? 32 - __builtin_clz(diff) : 0;  // low bits in which keys of the row may differ
+  uint32_t prefix_mask = top >= 32 ? 0u : ~((1u << top) - 1u);
+  uint32_t prefix = kmax & prefix_mask;
+  int k_rem = k;
+  while (top > 0) {
+    const int bits = min(8, top);
+    const int shift = top - bits;
+    const uint32_t dmask = (1u << bits) - 1u;
     for (int i = tx; i < 256; i += THREADS) sm.hist[i] = 0;
     __syncthreads();
 #pragma unroll
     for (int j = 0; j < VPT; ++j) {
       if ((key[j] & prefix_mask) == prefix && key[j] != 0u)
-        atomicAdd(&sm.hist[(key[j] >> shift) & 0xFFu], 1);
+        atomicAdd(&sm.hist[(key[j] >> shift) & dmask], 1);
     }
     __syncthreads();
     if (wave == 0) {
@@ -122,8 +164,9 @@ __device__ __forceinline__ void quest_select_row(const QuestArgs& a, uint32_t ro
     }
     __syncthreads();
     prefix |= (uint32_t)sm.pick[0] << shift;
-    prefix_mask |= 0xFFu << shift;
+    prefix_mask |= dmask << shift;
     k_rem = sm.pick[1];
+    top = shift;
   }
   const uint32_t T = prefix;  // k-th largest key; k_rem of the keys equal to T are taken
 
@@ -158,85 +201,99 @@ __global__ __launch_bounds__(THREADS) void quest_select_kernel(QuestArgs a) {
   quest_select_row<THREADS, VPT>(a, blockIdx.x, sm);
 }
 
-template <int DT>
+// GROUP q heads share one kv head (GQA): a workgroup row is one (batch, kv head) and every metadata
+// record is loaded once and scored against the GROUP queries. GROUP == 1 also serves group sizes
+// without a specialisation: then a row is one (batch, q head) and records are re-read per q head.
+template <int DT, int GROUP>
 __global__ __launch_bounds__(kQsThreads) void quest_score_kernel(QuestArgs a) {
-  const uint32_t row = blockIdx.y;
-  const uint32_t b = row / a.num_q_heads;
-  const uint32_t h = row - b * a.num_q_heads;
-  const uint32_t kvh = h / (a.num_q_heads / a.num_kv_heads);
+  const uint32_t rows_per_batch = GROUP == 1 ? a.num_q_heads : a.num_kv_heads;
+  const uint32_t b = blockIdx.y / rows_per_batch;
+  const uint32_t r = blockIdx.y - b * rows_per_batch;
+  const uint32_t kvh = GROUP == 1 ? r / (a.num_q_heads / a.num_kv_heads) : r;
+  const uint32_t row0 = b * a.num_q_heads + (GROUP == 1 ? r : r * GROUP);  // first q-head row
   const int lane = lane_id();
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int pg_begin = a.kv_page_indptr[b];
   const int n_pages = min(max(a.kv_page_indptr[b + 1] - pg_begin, 0), (int)a.max_pages);
   const int p0 = blockIdx.x * kQsPagesPerBlock + wave * kQsPagesPerWave;
   const int np = min(kQsPagesPerWave, n_pages - p0);  // <= 0: this wave has nothing to stream
+  if (np <= 0) return;
 
-  if (np > 0) {
-    const int c = lane & 31;     // channel chunk: dims 4c..4c+3
-    const int half = lane >> 5;  // which of the 2 pages of a load
-    // q for dims 4c..4c+3 and the per-half select mask (all ones where q > 0)
-    uint32_t qw[2];
-    {
-      u32x2 v = *(const u32x2*)((const uint16_t*)a.q + (size_t)row * TWL_HEAD_DIM + 4 * c);
-      qw[0] = v.x; qw[1] = v.y;
-    }
-    int my_phys = 0;
-    if (lane < np) my_phys = a.kv_page_indices[pg_begin + p0 + lane];
-    float qf[4];
-    uint32_t selmask[2];
+  const int c = lane & 31;     // channel chunk: dims 4c..4c+3
+  const int half = lane >> 5;  // which of the 2 pages of a load
+  // q for dims 4c..4c+3 and the per-half select mask (all ones where q > 0), per q head
+  uint32_t qw[GROUP][2];
+#pragma unroll
+  for (int g = 0; g < GROUP; ++g) {
+    u32x2 v = *(const u32x2*)((const uint16_t*)a.q + (size_t)(row0 + g) * TWL_HEAD_DIM + 4 * c);
+    qw[g][0] = v.x; qw[g][1] = v.y;
+  }
+  int my_phys = 0;
+  if (lane < np) my_phys = a.kv_page_indices[pg_begin + p0 + lane];
+  float qf[GROUP][4];
+  uint32_t selmask[GROUP][2];
+#pragma unroll
+  for (int g = 0; g < GROUP; ++g)
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      qf[2 * j] = bits16_to_f32<DT>(qw[j] & 0xFFFFu);
-      qf[2 * j + 1] = bits16_to_f32<DT>(qw[j] >> 16);
-      selmask[j] = (qf[2 * j] > 0.0f ? 0x0000FFFFu : 0u) | (qf[2 * j + 1] > 0.0f ? 0xFFFF0000u : 0u);
+      qf[g][2 * j] = bits16_to_f32<DT>(qw[g][j] & 0xFFFFu);
+      qf[g][2 * j + 1] = bits16_to_f32<DT>(qw[g][j] >> 16);
+      selmask[g][j] = (qf[g][2 * j] > 0.0f ? 0x0000FFFFu : 0u) |
+                      (qf[g][2 * j + 1] > 0.0f ? 0xFFFF0000u : 0u);
     }
-    const size_t rec_stride = (size_t)a.num_kv_heads * TWL_META_RECORD_BYTES;
-    const uint8_t* base = a.meta + (size_t)kvh * TWL_META_RECORD_BYTES + 16 * c;
-    float keep = 0.0f;  // lane i ends up with the score of page p0 + i
+  const size_t rec_stride = (size_t)a.num_kv_heads * TWL_META_RECORD_BYTES;
+  const uint8_t* base = a.meta + (size_t)kvh * TWL_META_RECORD_BYTES + 16 * c;
+  float keep[GROUP];  // lane i ends up with the score of page p0 + i
+#pragma unroll
+  for (int g = 0; g < GROUP; ++g) keep[g] = 0.0f;
 
 #pragma unroll
-    for (int i0 = 0; i0 < kQsPagesPerWave; i0 += 2 * kQsUnroll) {
-      if (i0 >= np) break;
-      u32x4 mm[kQsUnroll];
+  for (int i0 = 0; i0 < kQsPagesPerWave; i0 += 2 * kQsUnroll) {
+    if (i0 >= np) break;
+    u32x4 mm[kQsUnroll];
 #pragma unroll
-      for (int u = 0; u < kQsUnroll; ++u) {
-        const int ia = i0 + 2 * u, ib = ia + 1;
-        const int pa = __builtin_amdgcn_readlane(my_phys, (ia < np) ? ia : 0);
-        const int pb = __builtin_amdgcn_readlane(my_phys, (ib < np) ? ib : 0);
-        const int phys = half ? pb : pa;
-        mm[u] = __builtin_nontemporal_load((const u32x4*)(base + (size_t)phys * rec_stride));
-      }
+    for (int u = 0; u < kQsUnroll; ++u) {
+      const int ia = i0 + 2 * u, ib = ia + 1;
+      const int pa = __builtin_amdgcn_readlane(my_phys, (ia < np) ? ia : 0);
+      const int pb = __builtin_amdgcn_readlane(my_phys, (ib < np) ? ib : 0);
+      const int phys = half ? pb : pa;
+      mm[u] = __builtin_nontemporal_load((const u32x4*)(base + (size_t)phys * rec_stride));
+    }
 #pragma unroll
-      for (int u = 0; u < kQsUnroll; ++u) {
+    for (int u = 0; u < kQsUnroll; ++u) {
+      const int ia = i0 + 2 * u;
+#pragma unroll
+      for (int g = 0; g < GROUP; ++g) {
         // words: x,y = min[4c..4c+3], z,w = max[4c..4c+3]
-        const uint32_t s0 = (mm[u].z & selmask[0]) | (mm[u].x & ~selmask[0]);
-        const uint32_t s1 = (mm[u].w & selmask[1]) | (mm[u].y & ~selmask[1]);
+        const uint32_t s0 = (mm[u].z & selmask[g][0]) | (mm[u].x & ~selmask[g][0]);
+        const uint32_t s1 = (mm[u].w & selmask[g][1]) | (mm[u].y & ~selmask[g][1]);
         float acc;
         if (DT == TWL_F16) {
           acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, s0),
-                                       __builtin_bit_cast(half2_t, qw[0]), 0.0f, false);
+                                       __builtin_bit_cast(half2_t, qw[g][0]), 0.0f, false);
           acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, s1),
-                                       __builtin_bit_cast(half2_t, qw[1]), acc, false);
+                                       __builtin_bit_cast(half2_t, qw[g][1]), acc, false);
         } else {
-          acc = qf[0] * as_f32(s0 << 16);
-          acc = fmaf(qf[1], as_f32(s0 & 0xFFFF0000u), acc);
-          acc = fmaf(qf[2], as_f32(s1 << 16), acc);
-          acc = fmaf(qf[3], as_f32(s1 & 0xFFFF0000u), acc);
+          acc = qf[g][0] * as_f32(s0 << 16);
+          acc = fmaf(qf[g][1], as_f32(s0 & 0xFFFF0000u), acc);
+          acc = fmaf(qf[g][2], as_f32(s1 << 16), acc);
+          acc = fmaf(qf[g][3], as_f32(s1 & 0xFFFF0000u), acc);
         }
         acc = row16_allreduce<OpSum>(acc);
         acc += dpp<kDppBcast15, 0xA>(0.0f, acc);  // lanes 16..31 / 48..63 now hold a page total
         const float sa = as_f32(__builtin_amdgcn_readlane(as_i32(acc), 31));
         const float sb = as_f32(__builtin_amdgcn_readlane(as_i32(acc), 63));
-        const int ia = i0 + 2 * u;
-        keep = (lane == ia) ? sa : keep;
-        keep = (lane == ia + 1) ? sb : keep;
+        keep[g] = (lane == ia) ? sa : keep[g];
+        keep[g] = (lane == ia + 1) ? sb : keep[g];
       }
     }
-    // one store per wave: 32 consecutive scores
-    float* orow = a.page_scores + (size_t)row * a.score_stride + p0;
-    if (lane < np) orow[lane] = keep;
   }
-
+  // one store per wave and q head: 32 consecutive scores
+  if (lane < np) {
+#pragma unroll
+    for (int g = 0; g < GROUP; ++g)
+      a.page_scores[(size_t)(row0 + g) * a.score_stride + p0 + lane] = keep[g];
+  }
 }
 
 }  // namespace twl
@@ -266,11 +323,23 @@ static int check_budget(uint32_t token_budget, uint32_t max_pages_per_req, uint3
   return sel_stride < k ? TWL_EINVAL : TWL_OK;
 }
 
-static void launch_score(int q_dtype, dim3 grid, hipStream_t s, const twl::QuestArgs& a) {
+template <int GROUP>
+static void launch_score_g(int q_dtype, dim3 grid, hipStream_t s, const twl::QuestArgs& a) {
   if (q_dtype == TWL_F16)
-    hipLaunchKernelGGL((twl::quest_score_kernel<TWL_F16>), grid, dim3(twl::kQsThreads), 0, s, a);
+    hipLaunchKernelGGL((twl::quest_score_kernel<TWL_F16, GROUP>), grid, dim3(twl::kQsThreads), 0,
+                       s, a);
   else
-    hipLaunchKernelGGL((twl::quest_score_kernel<TWL_BF16>), grid, dim3(twl::kQsThreads), 0, s, a);
+    hipLaunchKernelGGL((twl::quest_score_kernel<TWL_BF16, GROUP>), grid, dim3(twl::kQsThreads), 0,
+                       s, a);
+}
+
+static void launch_score(int q_dtype, uint32_t batch, hipStream_t s, const twl::QuestArgs& a) {
+  const uint32_t gx = (a.max_pages + twl::kQsPagesPerBlock - 1) / twl::kQsPagesPerBlock;
+  const uint32_t group = a.num_q_heads / a.num_kv_heads;
+  if (group == 2) launch_score_g<2>(q_dtype, dim3(gx, batch * a.num_kv_heads), s, a);
+  else if (group == 4) launch_score_g<4>(q_dtype, dim3(gx, batch * a.num_kv_heads), s, a);
+  else if (group == 8) launch_score_g<8>(q_dtype, dim3(gx, batch * a.num_kv_heads), s, a);
+  else launch_score_g<1>(q_dtype, dim3(gx, batch * a.num_q_heads), s, a);
 }
 
 extern "C" int twl_quest_page_scores(const void* q, int q_dtype, const void* meta,
@@ -287,9 +356,7 @@ extern "C" int twl_quest_page_scores(const void* q, int q_dtype, const void* met
   a.q = q; a.meta = (const uint8_t*)meta; a.kv_page_indices = kv_page_indices;
   a.kv_page_indptr = kv_page_indptr; a.num_q_heads = num_q_heads; a.num_kv_heads = num_kv_heads;
   a.max_pages = max_pages_per_req; a.page_scores = page_scores; a.score_stride = score_stride;
-  dim3 grid((max_pages_per_req + twl::kQsPagesPerBlock - 1) / twl::kQsPagesPerBlock,
-            batch * num_q_heads);
-  launch_score(q_dtype, grid, (hipStream_t)stream, a);
+  launch_score(q_dtype, batch, (hipStream_t)stream, a);
   return hipGetLastError() == hipSuccess ? TWL_OK : TWL_ELAUNCH;
 }
 

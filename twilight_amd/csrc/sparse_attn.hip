@@ -68,9 +68,10 @@ struct AttnSmem {
 
 // One chunk (survivors [128*split, 128*split+128) of `row`, which has n > 128*split survivors).
 // Called by all threads of the workgroup.
-template <int DT>
+// `tok_pre` (chunk 0 only, HAVE_TOK): the chunk's survivor index of this thread, already loaded.
+template <int DT, bool HAVE_TOK>
 __device__ __forceinline__ void attn_chunk(const AttnArgs& a, AttnSmem& sm, uint32_t row,
-                                           int split, int n) {
+                                           int split, int n, int tok_pre) {
   int (&slot_id)[kAttnChunk] = sm.slot_id;
   float (&w)[kAttnChunk] = sm.w;
   float (&red)[2][16] = sm.red;
@@ -94,7 +95,7 @@ __device__ __forceinline__ void attn_chunk(const AttnArgs& a, AttnSmem& sm, uint
   if (tx < kAttnChunk) {
     int sid = 0;
     if (tx < cn) {
-      const int tok = a.idx[(size_t)row * a.idx_stride + j0 + tx];
+      const int tok = HAVE_TOK ? tok_pre : a.idx[(size_t)row * a.idx_stride + j0 + tx];
       sid = a.kv_page_indices[a.kv_page_indptr[b] + (tok >> 4)] * TWL_PAGE + (tok & 15);
     }
     slot_id[tx] = sid;
@@ -231,10 +232,20 @@ __device__ __forceinline__ void attn_chunk(const AttnArgs& a, AttnSmem& sm, uint
   const float gl = block_allreduce<OpSum, kAttnWaves>(lsum, red[1]);  // barrier: factors visible
   const int d = tx & (TWL_HEAD_DIM - 1), half = tx >> 7;
   float go = 0.0f;
-#pragma unroll 4
-  for (int s = half; s < n_splits; s += 2)
-    go = fmaf(__hip_atomic_load(prow + (size_t)s * kAttnPartial + 2 + d, __ATOMIC_RELAXED,
-                                __HIP_MEMORY_SCOPE_AGENT), fm[s], go);
+  for (int s0 = half; s0 < n_splits; s0 += 32) {  // 16 loads in flight per thread
+    float pv[16];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+      const int s = min(s0 + 2 * u, n_splits - 1);
+      pv[u] = __hip_atomic_load(prow + (size_t)s * kAttnPartial + 2 + d, __ATOMIC_RELAXED,
+                                __HIP_MEMORY_SCOPE_AGENT);
+    }
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+      const int s = s0 + 2 * u;
+      go = fmaf(pv[u], (s < n_splits) ? fm[s] : 0.0f, go);
+    }
+  }
   if (half == 1) oacc[8][d] = go;
   __syncthreads();
   if (half == 0) go += oacc[8][d];
@@ -259,13 +270,16 @@ __global__ __launch_bounds__(kAttnThreads) void sparse_attn_kernel(AttnArgs a) {
   const int tx = threadIdx.x;
   if (blockIdx.x < a.rows) {
     const uint32_t row = blockIdx.x;
+    // the first survivors are requested together with the count they depend on
+    const int tok_pre = ((uint32_t)tx < min((uint32_t)kAttnChunk, a.idx_stride))
+                            ? a.idx[(size_t)row * a.idx_stride + tx] : 0;
     const int n = min(max(a.count[row], 0), (int)a.idx_stride);
     if (n == 0) {
       if (tx < TWL_HEAD_DIM) ((uint16_t*)a.out)[(size_t)row * TWL_HEAD_DIM + tx] = 0;
       if (tx == 0 && a.lse_out) a.lse_out[row] = -__builtin_inff();
       return;
     }
-    attn_chunk<DT>(a, sm, row, 0, n);
+    attn_chunk<DT, true>(a, sm, row, 0, n, tok_pre);
     return;
   }
   const int lane = lane_id();
@@ -298,7 +312,7 @@ __global__ __launch_bounds__(kAttnThreads) void sparse_attn_kernel(AttnArgs a) {
       __syncthreads();
     }
     if (!hit) return;  // j is past the last overflow chunk: nothing left for this workgroup
-    attn_chunk<DT>(a, sm, (uint32_t)found[0], found[1], found[2]);
+    attn_chunk<DT, false>(a, sm, (uint32_t)found[0], found[1], found[2], 0);
     __syncthreads();
   }
 }
