@@ -92,6 +92,10 @@ def main() -> int:
     ap.add_argument("--context", type=int, default=32768)
     ap.add_argument("--budget", type=int, default=8192)
     ap.add_argument("--top-p", type=float, default=0.95)
+    ap.add_argument("--workload", choices=["longchat", "llama3"], default="longchat",
+                    help="longchat: 32 MHA heads fp16 (the headline workload); llama3: GQA 32/8 "
+                         "bf16, with a dense-decode baseline (the same attention kernel over "
+                         "every token)")
     ap.add_argument("--layers", type=int, default=4,
                     help="independent layer caches visited round-robin (cold-cache steps)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -116,9 +120,11 @@ def main() -> int:
     L = _lib.lib()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    B, H, Hkv, N, D = args.batch, 32, 32, args.context, 128
+    llama = args.workload == "llama3"
+    B, H, Hkv, N, D = args.batch, 32, (8 if llama else 32), args.context, 128
     npg = N // 16
-    dt = torch.float16
+    dt = torch.bfloat16 if llama else torch.float16
+    qcode = 1 if llama else 0   # twl_dtype of q / K / V
 
     if args.calibrate_copy:
         src = torch.full((1 << 28,), 1.0, dtype=torch.float32, device=dev)   # 1 GiB
@@ -183,13 +189,14 @@ def main() -> int:
         it, wu = max(args.steps, 50), 2 * nl
         calls = {
             "quest_score": (rotating(lambda l, c, q: lambda: L.twl_quest_page_scores(
-                p(q), 0, p(c.meta), p(c.kv_page_indices), p(c.kv_page_indptr), B, H, Hkv,
-                npg, p(l.page_scores), npg, stream)), rows * npg * (512 + 4) + rows * D * 2),
+                p(q), qcode, p(c.meta), p(c.kv_page_indices), p(c.kv_page_indptr), B, H, Hkv,
+                npg, p(l.page_scores), npg, stream)),
+                B * Hkv * npg * 512 + rows * npg * 4 + rows * D * 2),
             "quest_topk": (rotating(lambda l, c, q: lambda: L.twl_quest_topk_pages(
                 p(l.page_scores), npg, p(c.kv_page_indptr), B, H, args.budget, npg,
                 p(l.sel_pages), kp, p(l.sel_count), stream)), rows * (npg * 4 + kp * 4 + 4)),
             "gemv_int4": (rotating(lambda l, c, q: lambda: L.twl_gemv_int4(
-                p(q), 0, p(l.scores), M, p(l.cand_count), p(c.k_int4), p(l.sel_pages),
+                p(q), qcode, p(l.scores), M, p(l.cand_count), p(c.k_int4), p(l.sel_pages),
                 p(l.sel_count), kp, p(c.kv_page_indices), p(c.kv_page_indptr),
                 p(c.kv_last_page_len), B, H, Hkv, kp, sm, stream)),
                 rows * M * (64 + 16 + 4) + rows * D * 2 + rows * kp * 8),
@@ -198,7 +205,7 @@ def main() -> int:
                 kp, p(l.idx), M, p(l.count), 0, 0, stream)),
                 rows * M * 4 + int(rows * n_bar) * 4 + rows * 4),
             "sparse_attn": (rotating(lambda l, c, q: lambda: L.twl_sparse_attn(
-                p(q), p(l.out), 0, p(c.k_cache), p(c.v_cache), *c.k_cache.stride()[:3],
+                p(q), p(l.out), qcode, p(c.k_cache), p(c.v_cache), *c.k_cache.stride()[:3],
                 p(l.idx), M, p(l.count), p(c.kv_page_indices), p(c.kv_page_indptr),
                 B, H, Hkv, sm, 0, p(l.attn_workspace), l.attn_workspace.numel(), stream)),
                 int(rows * n_bar) * (2 * D * 2 + 4) + rows * D * 4),
@@ -219,11 +226,11 @@ def main() -> int:
 
     # ---- stand-alone INT4 GEMV at 8 x 32 x 32768 candidates (all pages of every request) ----
     gemv_cfg2 = None
-    if not args.no_kernels and B == 8 and N == 32768:
+    if not args.no_kernels and B == 8 and N == 32768 and not llama:
         out2 = torch.empty((B, H, N), dtype=torch.float32, device=dev)
         cnt2 = torch.empty((B, H), dtype=torch.int32, device=dev)
         fn = rotating(lambda l, c, q: lambda: L.twl_gemv_int4(
-            p(q), 0, p(out2), N, p(cnt2), p(c.k_int4), 0, 0, 0, p(c.kv_page_indices),
+            p(q), qcode, p(out2), N, p(cnt2), p(c.k_int4), 0, 0, 0, p(c.kv_page_indices),
             p(c.kv_page_indptr), p(c.kv_last_page_len), B, H, Hkv, npg, sm, stream))
         us = _time_calls(fn, 50, 2 * nl)
         nbytes = rows * N * 84 + rows * D * 2
@@ -233,19 +240,57 @@ def main() -> int:
                                  "shuffled pages"}
         del out2
 
+    # ---- dense-decode baseline on the same GPU: the same attention kernel over every token ----
+    dense = None
+    if llama and not args.no_kernels:
+        full_idx = torch.arange(N, dtype=torch.int32, device=dev).repeat(B, H, 1).contiguous()
+        full_cnt = torch.full((B, H), N, dtype=torch.int32, device=dev)
+        ws = torch.zeros(int(L.twl_sparse_attn_workspace_bytes(rows, N)), dtype=torch.uint8, device=dev)
+        outd = torch.empty_like(qs[0])
+        fn = rotating(lambda l, c, q: lambda: L.twl_sparse_attn(
+            p(q), p(outd), qcode, p(c.k_cache), p(c.v_cache), *c.k_cache.stride()[:3], p(full_idx), N,
+            p(full_cnt), p(c.kv_page_indices), p(c.kv_page_indptr), B, H, Hkv, sm, 0, p(ws),
+            ws.numel(), stream))
+        us = _time_calls(fn, 20, nl)
+        nbytes = B * Hkv * N * 2 * D * 2
+        dense = {"us": round(us, 2), "bytes": nbytes, "GBps": round(nbytes / us / 1e3, 1),
+                 "what": "twl_sparse_attn over all 32768 tokens of every row (the sparse kernel "
+                         "used densely: K/V are fetched per q head, 4x the bytes counted here, "
+                         "which count K/V once per kv head)"}
+        del full_idx, ws
+        # torch's own dense decode attention over contiguous K/V of one layer (GQA-aware)
+        try:
+            c0 = layers[0].cache
+            phys = c0.kv_page_indices.long().reshape(B, npg)
+            kd = c0.k_cache[phys].reshape(B, N, Hkv, D).permute(0, 2, 1, 3).contiguous()
+            vd = c0.v_cache[phys].reshape(B, N, Hkv, D).permute(0, 2, 1, 3).contiguous()
+            q4 = qs[0].reshape(B, H, 1, D)
+            sdpa = lambda: torch.nn.functional.scaled_dot_product_attention(
+                q4, kd, vd, is_causal=False, enable_gqa=True)
+            dense["torch_sdpa_us"] = round(_time_calls(sdpa, 20, 3), 2)
+            dense["torch_sdpa_what"] = ("torch.nn.functional.scaled_dot_product_attention, q "
+                                        "[B,32,1,128], contiguous bf16 K/V [B,8,32768,128], "
+                                        "enable_gqa=True, same data every call (warm caches)")
+            del kd, vd
+        except Exception as e:  # a missing SDPA backend must not fail the benchmark
+            dense["torch_sdpa_us"] = None
+            dense["torch_sdpa_what"] = f"not available: {type(e).__name__}: {e}"
+
     cpu = None
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and not llama:
         cpu = cpu_baseline(N, H, args.budget, args.top_p, B)
 
     line = {
         "metric": "us/decode-layer at 32k ctx (select+prune+attn)",
         "value": round(wall_us, 2), "unit": "us", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(wall_us / 1e3, 5), "higher_is_better": False,
-        "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
-        "config": {"workload": f"Select-then-Prune decode layer, Longchat-7B shape: B={B}, 32 MHA "
-                               f"heads, head_dim 128, fp16 paged KV (page 16), context {N}, Quest "
-                               f"budget {args.budget}, INT4 K estimate (group 32), top-p "
-                               f"{args.top_p}",
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if llama else "f16",
+        "data": "synthetic",
+        "config": {"workload": (f"Select-then-Prune decode layer, "
+                                f"{'Llama-3-8B shape: GQA 32/8' if llama else 'Longchat-7B shape: 32 MHA'}"
+                                f" heads, B={B}, head_dim 128, {'bf16' if llama else 'fp16'} paged KV "
+                                f"(page 16), context {N}, Quest budget {args.budget}, INT4 K estimate "
+                                f"(group 32), top-p {args.top_p}"),
                    "batch": B, "context": N, "budget": args.budget, "top_p": args.top_p,
                    "layers_rotated": nl, "survivors_mean": round(n_bar, 1),
                    "survivors_max": n_max},
@@ -254,6 +299,8 @@ def main() -> int:
                                    if layer_bytes else None),
         "roofline": roofline, "kernels": kernels, "gemv_cfg2": gemv_cfg2, "cpu_baseline": cpu,
     }
+    if dense:
+        line["dense_decode_baseline"] = dense
     print(json.dumps(line))
     return 0
 
