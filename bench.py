@@ -31,6 +31,13 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 
+# HBM bytes per launch of quest_score_kernel at the default workload, measured with
+# `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` (131404.9 KiB x 2.000 + 2048.0 KiB x 1.000, the
+# factors being what the same counters read for a 1 GiB device copy; the summary of those runs is
+# kept under profiles/). bench.py cannot read counters itself, so the figure is reported only for
+# the exact configuration it was measured on.
+QUEST_SCORE_TRAFFIC_BYTES_DEFAULT = int((131404.9 * 2.000 + 2048.0 * 1.000) * 1024)
+
 
 def _time_calls(fn, iters: int, warmup: int) -> float:
     """Average microseconds per call of ``fn`` (which enqueues on the current stream), measured
@@ -222,7 +229,9 @@ def main() -> int:
     if dom:
         roofline = {"bound": "hbm", "kernel": "quest_score_kernel", "achieved": dom["GBps"],
                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": dom["frac_of_hbm_peak"],
-                    "bytes_per_launch": dom["bytes"], "us_per_launch": dom["us"], "traffic": None}
+                    "bytes_per_launch": dom["bytes"], "us_per_launch": dom["us"],
+                    "traffic": (QUEST_SCORE_TRAFFIC_BYTES_DEFAULT
+                                if (B, N, args.budget, llama) == (8, 32768, 8192, False) else None)}
 
     # ---- stand-alone INT4 GEMV at 8 x 32 x 32768 candidates (all pages of every request) ----
     gemv_cfg2 = None
