@@ -108,6 +108,8 @@ def main() -> int:
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run 4 device copies of 1 GiB (a kernel of known traffic, used to "
                          "scale the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
+    ap.add_argument("--split-estimator", action="store_true",
+                    help="run the INT4 GEMV and the softmax + top-p as two launches instead of one")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel breakdown")
     args = ap.parse_args()
@@ -153,7 +155,7 @@ def main() -> int:
         cache.set_page_table(ids, indptr, last)
         cache.rebuild_shadow()
         layers.append(TwilightDecodeLayer(cache, H, token_budget=args.budget, top_p=args.top_p,
-                                          high="max"))
+                                          high="max", fused_estimator=not args.split_estimator))
         qs.append(q)
     torch.cuda.synchronize()
     nl = len(layers)
@@ -207,6 +209,12 @@ def main() -> int:
                 p(l.sel_count), kp, p(c.kv_page_indices), p(c.kv_page_indptr),
                 p(c.kv_last_page_len), B, H, Hkv, kp, sm, stream)),
                 rows * M * (64 + 16 + 4) + rows * D * 2 + rows * kp * 8),
+            "gemv_top_p": (rotating(lambda l, c, q: lambda: L.twl_gemv_top_p(
+                p(q), qcode, p(c.k_int4), p(l.sel_pages), p(l.sel_count), kp,
+                p(c.kv_page_indices), p(c.kv_page_indptr), p(c.kv_last_page_len), B, H, Hkv, kp,
+                sm, 0, args.top_p, 1, p(l.idx), M, p(l.count), 0, M, p(l.cand_count), 0, stream)),
+                rows * M * (64 + 16) + rows * D * 2 + rows * kp * 8 + int(rows * n_bar) * 4
+                + rows * 8),
             "softmax_top_p": (rotating(lambda l, c, q: lambda: L.twl_softmax_top_p_f32(
                 p(l.scores), M, p(l.cand_count), rows, M, 0, args.top_p, 1, p(l.sel_pages),
                 kp, p(l.idx), M, p(l.count), 0, 0, stream)),
@@ -223,7 +231,12 @@ def main() -> int:
                              "GBps": round(nbytes / us / 1e3, 1),
                              "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
 
-    layer_bytes = sum(kv["bytes"] for kv in kernels.values()) if kernels else None
+    # the kernels one layer step launches: the fused estimator + pruner unless --split-estimator
+    used = (("quest_score", "quest_topk", "gemv_int4", "softmax_top_p", "sparse_attn")
+            if args.split_estimator else ("quest_score", "quest_topk", "gemv_top_p", "sparse_attn"))
+    for name in kernels:
+        kernels[name]["in_layer_step"] = name in used
+    layer_bytes = sum(kernels[n]["bytes"] for n in used) if kernels else None
     dom = kernels.get("quest_score")
     roofline = None
     if dom:

@@ -113,6 +113,27 @@ int twl_softmax_top_p_f32(const float* scores, uint32_t score_stride, const int3
                           void* stream);
 
 /* ---------------------------------------------------------------------------------------------
+ * Estimator and pruner in one launch: twl_gemv_int4 over a row's page list followed by
+ * twl_softmax_top_p_f32 on those scores, the scores staying in registers.
+ * Replaces: twilight/pyimpl/attention.py:252-255 (estimate) + twilight/pyimpl/top_p.py:10-15
+ * (softmax, mask kernel) + attention.py:280-281 (combine), in index-list form.
+ * Arguments as in twl_gemv_int4 and twl_softmax_top_p_f32; sel_pages is required and
+ * max_pages_per_row * 16 <= TWL_MAX_CANDIDATES. scores_out (nullable) float [rows, score_stride]
+ * receives the raw scaled scores (candidate order, -inf past the last page's length) for
+ * inspection; cand_count (nullable) int32 [rows] the candidate count; low_out (nullable) the final
+ * lower pivot. The survivor list idx / count is identical to the two-call sequence: the same
+ * arithmetic runs on the same values, only the summation order of the softmax denominator and of
+ * the bisection sums differs (fp32, the order inside a sum is unspecified in both).
+ * ------------------------------------------------------------------------------------------- */
+int twl_gemv_top_p(const void* q, int q_dtype, const void* k_int4, const int32_t* sel_pages,
+                   const int32_t* sel_count, uint32_t sel_stride, const int32_t* kv_page_indices,
+                   const int32_t* kv_page_indptr, const int32_t* kv_last_page_len, uint32_t batch,
+                   uint32_t num_q_heads, uint32_t num_kv_heads, uint32_t max_pages_per_row,
+                   float sm_scale, const float* p_arr, float p, int high_mode, int32_t* idx,
+                   uint32_t idx_stride, int32_t* count, float* scores_out, uint32_t score_stride,
+                   int32_t* cand_count, float* low_out, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
  * INT4-K score GEMV over candidate pages: out[r, c] = sm_scale * sum_d q[r,d] * dequant(K[c,d]).
  * Replaces: the estimator matmul twilight/pyimpl/attention.py:252-255 and the absent
  * ftka.cuda_ops.gemv.batched_sparse_gemv_int4_k whose call site is
@@ -282,6 +303,10 @@ typedef struct twl_layer_args {
   void* attn_workspace; uint64_t attn_workspace_bytes; /* see twl_sparse_attn */
   /* output */
   void* out;                /* [batch, num_q_heads, 128], dtype */
+  /* estimator + pruner: 0 = one fused launch (twl_gemv_top_p), 1 = twl_gemv_int4 then
+   * twl_softmax_top_p_f32. In fused mode `scores` is filled only when keep_scores != 0. */
+  int split_estimator;
+  int keep_scores;
 } twl_layer_args;
 
 int twl_decode_layer(const twl_layer_args* args, void* stream);

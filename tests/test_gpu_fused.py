@@ -1,0 +1,155 @@
+"""GPU parity of the one-launch estimator + pruner (INT4 score GEMV, softmax, top-p, compaction)
+against the oracle's restatement of twilight/pyimpl/attention.py:252-255 and
+twilight/pyimpl/top_p.py:10-15 (csrc/include/sampling.cuh:156-231), and against the two-launch
+sequence of the same library."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import native
+from oracle import pyimpl_port as P
+from twilight_amd import synth
+import twilight_amd.kernel as K
+from _checks import assert_scores_close, assert_top_p_parity
+
+pytestmark = pytest.mark.gpu
+
+
+def _peaky_q(B, H, rec, ids, indptr, seed):
+    """q aligned with a few random tokens of each request so that the softmax has heavy hitters."""
+    g = torch.Generator().manual_seed(seed)
+    codes, scale, zero = P.unpack_int4_records(rec.numpy())
+    deq = torch.from_numpy(native.int4_dequant(codes, scale, zero))       # [P,Hkv,16,128]
+    Hkv = deq.shape[1]
+    q = torch.randn((B, H, 128), generator=g) * 0.5
+    for b in range(B):
+        npg = int(indptr[b + 1] - indptr[b])
+        for h in range(H):
+            for _ in range(int(torch.randint(1, 6, (1,), generator=g))):
+                pg = int(ids[int(indptr[b]) + int(torch.randint(0, npg, (1,), generator=g))])
+                tok = int(torch.randint(0, 16, (1,), generator=g))
+                q[b, h] += deq[pg, h // (H // Hkv), tok] * float(torch.rand(1, generator=g) * 12 + 4)
+    return q, deq
+
+
+def _case(dev, B, H, Hkv, npg, S, last_len, p, high, qdt, seed, ragged=True, per_row_p=False):
+    rec = synth.int4_records_random(B * npg, Hkv, seed=seed)
+    ids, indptr, last = synth.identity_page_table(B, npg, last_len=last_len, shuffle_seed=seed + 1)
+    q, deq = _peaky_q(B, H, rec, ids, indptr, seed + 2)
+    q = q.to(qdt)
+    g = torch.Generator().manual_seed(seed + 3)
+    sel = torch.stack([torch.sort(torch.randperm(npg, generator=g)[:S]).values
+                       for _ in range(B * H)]).reshape(B, H, S).to(torch.int32)
+    if ragged:
+        cnt_in = torch.randint(1, S + 1, (B, H), generator=g).to(torch.int32)
+        cnt_in[0, 0] = S
+        cnt_in[-1, -1] = 1
+        if B * H > 2:
+            cnt_in[0, 1] = 0                                           # a row without candidates
+    else:
+        cnt_in = torch.full((B, H), S, dtype=torch.int32)
+    rows = B * H
+    top_p = (torch.rand(rows, generator=g) * 0.5 + 0.45) if per_row_p else p
+    d = lambda t: t.to(dev)
+    args = (d(q), d(rec), d(ids), d(indptr), d(last))
+    idx, count, cand, scores, low = K.sparse_gemv_int4_top_p(
+        *args, d(sel), d(cnt_in), d(top_p) if per_row_p else top_p, high=high,
+        sm_scale=1 / math.sqrt(128), return_scores=True, return_low=True)
+    M = S * 16
+    assert torch.equal(cand.cpu(), cnt_in * 16)
+    sc = scores.cpu().numpy().reshape(rows, M)
+    ix = idx.cpu().numpy().reshape(rows, M)
+    cn = count.cpu().numpy().reshape(rows)
+    # 1. scores: oracle GEMV over the dequantised records (1e-3 relative), -inf past last_len
+    want = np.full((rows, M), -np.inf)
+    qf = q.float()
+    for b in range(B):
+        for h in range(H):
+            r = b * H + h
+            n = int(cnt_in[b, h])
+            phys = ids[indptr[b] + sel[b, h, :n].long()].long()
+            w = (deq[phys, h // (H // Hkv)].reshape(-1, 128).double() @ qf[b, h].double()) / math.sqrt(128)
+            w = w.numpy()
+            tok = (sel[b, h, :n, None].long() * 16 + torch.arange(16)[None]).reshape(-1).numpy()
+            w[tok >= (npg - 1) * 16 + last_len] = -np.inf
+            want[r, :n * 16] = w
+    assert_scores_close(sc, want)
+    # 2. the pruned lists against the oracle run on the GPU's own scores
+    x = torch.from_numpy(sc).masked_fill(torch.from_numpy(np.isinf(sc)), torch.finfo(torch.float32).min)
+    hm = native.HIGH_MAX if high == "max" else native.HIGH_FIRST
+    p_np = top_p.numpy().astype(np.float32) if per_row_p else p
+    live = np.nonzero(cnt_in.reshape(-1).numpy() > 0)[0]
+    om, oprobs, ol, _ = P.top_p_unnormalized(x.reshape(rows, 1, 1, M)[live], p_np[live] if per_row_p else p_np, hm)
+    pn = oprobs.reshape(len(live), M).numpy()
+    _, _, _, og = native.top_p_mask_f32(pn, p_np[live] if per_row_p else p_np, hm, return_margin=True)
+    selr = sel.reshape(rows, S).numpy()
+    gm = np.zeros((rows, M), dtype=bool)
+    for r in range(rows):
+        toks = ix[r, :cn[r]]
+        assert np.all(np.diff(toks) > 0)
+        pos = np.searchsorted(selr[r], toks // 16) * 16 + toks % 16
+        assert np.array_equal(selr[r][pos // 16] * 16 + pos % 16, toks)
+        gm[r, pos] = True
+    for r in range(rows):
+        if r not in live:
+            assert cn[r] == 0
+    n_exact = assert_top_p_parity(pn, p_np[live] if per_row_p else p_np, gm[live],
+                                  om.reshape(len(live), M).numpy(), ol, og, margin_tol=5e-6)
+    assert n_exact >= 0.9 * len(live)
+    # 3. the two-launch sequence of the same library: same scores bit for bit, same lists
+    s2, c2 = K.sparse_gemv_int4(*args, sel_pages=d(sel), sel_count=d(cnt_in))
+    assert torch.equal(c2.cpu(), cand.cpu())
+    s2n = s2.cpu().numpy().reshape(rows, M)
+    for r in range(rows):
+        n = int(cnt_in.reshape(-1)[r]) * 16
+        assert np.array_equal(s2n[r, :n].view(np.uint32), sc[r, :n].view(np.uint32))
+    i2, n2, l2 = K.softmax_top_p(s2, d(top_p) if per_row_p else top_p, lens=c2, sel_pages=d(sel),
+                                 high=high, return_low=True)
+    n2 = n2.cpu().numpy().reshape(rows)
+    i2 = i2.cpu().numpy().reshape(rows, M)
+    margin = np.full(rows, np.inf, dtype=np.float32)
+    margin[live] = og
+    same = [bool(n2[r] == cn[r] and np.array_equal(i2[r, :n2[r]], ix[r, :cn[r]])) for r in range(rows)]
+    assert sum(same) >= 0.9 * rows
+    for r in range(rows):
+        assert same[r] or margin[r] < 5e-6, r
+
+
+@pytest.mark.parametrize("S", [5, 16, 29, 64, 100, 256, 400, 1000, 2048])
+def test_every_kernel_shape(dev, S):
+    # one case per instantiated (threads, values per thread) shape; full lists, MHA, fp16
+    B, H = (2, 4) if S <= 400 else (1, 4)
+    npg = max(S + 3, int(S * 1.3))
+    _case(dev, B, H, H, npg, S, 16, 0.9, "max", torch.float16, seed=S, ragged=False)
+
+
+@pytest.mark.parametrize("S,Hkv,qdt,high,last_len,per_row_p", [
+    (70, 8, torch.float16, "max", 16, False),
+    (70, 2, torch.bfloat16, "max", 7, False),      # GQA 4:1, bf16 q, partial last page
+    (130, 8, torch.float16, "first", 16, False),   # the reference's initial upper bound
+    (300, 1, torch.float16, "max", 1, True),       # MQA, per-row p (top_p_arr)
+    (513, 4, torch.bfloat16, "first", 3, True),
+])
+def test_ragged_lists(dev, S, Hkv, qdt, high, last_len, per_row_p):
+    _case(dev, 2, 8, Hkv, S + 40, S, last_len, 0.85, high, qdt, seed=7 * S, per_row_p=per_row_p)
+
+
+def test_errors(dev):
+    rec = synth.int4_records_random(8, 2, seed=0).to(dev)
+    ids, indptr, last = [t.to(dev) for t in synth.identity_page_table(1, 8)]
+    q = torch.randn((1, 4, 128), device=dev).half()
+    sel = torch.arange(4, dtype=torch.int32, device=dev).repeat(1, 4, 1).contiguous()
+    cnt = torch.full((1, 4), 4, dtype=torch.int32, device=dev)
+    K.sparse_gemv_int4_top_p(q, rec, ids, indptr, last, sel, cnt, 0.9)
+    with pytest.raises(RuntimeError):
+        K.sparse_gemv_int4_top_p(q, rec, ids, indptr, last, sel, cnt, 1.5)
+    with pytest.raises(RuntimeError):
+        K.sparse_gemv_int4_top_p(q.float(), rec, ids, indptr, last, sel, cnt, 0.9)
+    with pytest.raises(RuntimeError):
+        K.sparse_gemv_int4_top_p(q, rec, ids, indptr, last, sel.long(), cnt, 0.9)
+    with pytest.raises(RuntimeError):
+        K.sparse_gemv_int4_top_p(q, rec, ids, indptr, last, sel, cnt, 0.9, max_pages=4096)
+    with pytest.raises(RuntimeError):
+        K.sparse_gemv_int4_top_p(q[:, :3], rec, ids, indptr, last, sel, cnt, 0.9)

@@ -22,14 +22,15 @@ def _lists_to_mask(idx, count, N):
     return m
 
 
-def _run_case(dev, B, H, Hkv, N, budget, p, dt, seed, shuffle=True, n_heavy=16):
+def _run_case(dev, B, H, Hkv, N, budget, p, dt, seed, shuffle=True, n_heavy=16, fused=True):
     q, k, v = synth.heavy_hitter_qkv(B, H, N, n_heavy=n_heavy, mass=0.6, seed=seed, dtype=dt)
     group = H // Hkv
     kk, vv = k[:, ::group].contiguous(), v[:, ::group].contiguous()        # one K/V per kv head
     npg = (N + 15) // 16
     perm = torch.randperm(B * npg, generator=torch.Generator().manual_seed(seed)) if shuffle else None
     cache = PagedKVCache.from_dense(kk.to(dt), vv.to(dt), dev, page_perm=perm)
-    layer = TwilightDecodeLayer(cache, H, token_budget=budget, top_p=p, high="max")
+    layer = TwilightDecodeLayer(cache, H, token_budget=budget, top_p=p, high="max",
+                                fused_estimator=fused, keep_scores=True)
     out = layer(q[:, :, 0].to(dt).to(dev)).cpu().float()
     krep = kk.repeat_interleave(group, dim=1)                               # attention.py:124-126
     vrep = vv.repeat_interleave(group, dim=1)
@@ -76,10 +77,11 @@ def _run_case(dev, B, H, Hkv, N, budget, p, dt, seed, shuffle=True, n_heavy=16):
     return layer, ref
 
 
-def test_cfg1_full_context(dev):
+@pytest.mark.parametrize("fused", [True, False])
+def test_cfg1_full_context(dev, fused):
     # BASELINE config 1: B=1, 32 heads MHA, D=128, N=4096, 16 heavy hitters with ~60 % of the mass,
     # all tokens are candidates, p = 0.95
-    layer, ref = _run_case(dev, 1, 32, 32, 4096, 4096, 0.95, torch.float16, seed=0)
+    layer, ref = _run_case(dev, 1, 32, 32, 4096, 4096, 0.95, torch.float16, seed=0, fused=fused)
     cnt = layer.count.cpu().float()
     assert 16 <= cnt.min() and cnt.mean() < 4096 * 0.8
 
@@ -90,8 +92,9 @@ def test_cfg1_full_context(dev):
     (3, 4, 4, 1000, 250, 0.85, torch.float16),     # ragged: partial last page, budget not /16
     (1, 4, 1, 100, 8192, 0.95, torch.float16),     # budget larger than the context
 ])
-def test_small_layer_configs(dev, B, H, Hkv, N, budget, p, dt):
-    _run_case(dev, B, H, Hkv, N, budget, p, dt, seed=B * 100 + H, n_heavy=8)
+@pytest.mark.parametrize("fused", [True, False])
+def test_small_layer_configs(dev, B, H, Hkv, N, budget, p, dt, fused):
+    _run_case(dev, B, H, Hkv, N, budget, p, dt, seed=B * 100 + H, n_heavy=8, fused=fused)
 
 
 def test_decode_append_keeps_shadow_fresh(dev):
@@ -125,7 +128,8 @@ def test_full_size_cfg4_layer_sampled_rows_and_properties(dev):
     cache.k_cache, cache.v_cache = k, v
     cache.set_page_table(ids, indptr, last)
     cache.rebuild_shadow()
-    layer = TwilightDecodeLayer(cache, H, token_budget=budget, top_p=p, high="max")
+    layer = TwilightDecodeLayer(cache, H, token_budget=budget, top_p=p, high="max",
+                                keep_scores=True)
     out = layer(q).clone()
     torch.cuda.synchronize()
     rows = B * H

@@ -24,7 +24,7 @@ MAX_CANDIDATES = 32768
 # every symbol include/twilight_hip.h declares
 EXPORTS = (
     "twl_strerror", "twl_abi_version", "twl_device_count", "twl_top_p_f32", "twl_top_p_f16",
-    "twl_softmax_top_p_f32", "twl_gemv_int4", "twl_gemv_int4_nhd",
+    "twl_softmax_top_p_f32", "twl_gemv_top_p", "twl_gemv_int4", "twl_gemv_int4_nhd",
     "twl_gemv_int8_nhd", "twl_gemv_f16_nhd", "twl_gemv_f16_single", "twl_sparse_attn",
     "twl_sparse_attn_workspace_bytes", "twl_quest_select",
     "twl_quest_page_scores", "twl_quest_topk_pages", "twl_kv_shadow_build", "twl_dequant_int4",
@@ -51,6 +51,7 @@ class LayerArgs(ctypes.Structure):
         ("count", c_void_p),
         ("attn_workspace", c_void_p), ("attn_workspace_bytes", c_uint64),
         ("out", c_void_p),
+        ("split_estimator", c_int), ("keep_scores", c_int),
     ]
 
 
@@ -76,6 +77,8 @@ def lib() -> ctypes.CDLL:
     L.twl_top_p_f16.argtypes = [vp, i32, vp, vp, vp, vp, f32, u32, u32, u32, i32, vp, vp, vp]
     L.twl_softmax_top_p_f32.argtypes = [vp, u32, vp, u32, u32, vp, f32, i32, vp, u32, vp, u32, vp,
                                         vp, vp, vp]
+    L.twl_gemv_top_p.argtypes = [vp, i32, vp, vp, vp, u32, vp, vp, vp, u32, u32, u32, u32, f32, vp,
+                                 f32, i32, vp, u32, vp, vp, u32, vp, vp, vp]
     L.twl_gemv_int4.argtypes = [vp, i32, vp, u32, vp, vp, vp, vp, u32, vp, vp, vp, u32, u32, u32,
                                 u32, f32, vp]
     L.twl_gemv_int4_nhd.argtypes = [vp, vp, u32, vp, vp, vp, vp, vp, vp, u32, u32, u32, u32, f32, vp]

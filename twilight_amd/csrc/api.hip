@@ -17,7 +17,7 @@ extern "C" const char* twl_strerror(int status) {
   }
 }
 
-extern "C" int twl_abi_version(void) { return 1; }
+extern "C" int twl_abi_version(void) { return 2; }
 
 extern "C" int twl_device_count(void) {
   int n = 0;
@@ -53,17 +53,28 @@ extern "C" int twl_decode_layer(const twl_layer_args* a, void* stream) {
                             a->max_pages_per_req, a->sel_pages, a->sel_stride, a->sel_count,
                             page_scores, ps_stride, stream);
   if (rc != TWL_OK) return rc;
-  // 2. INT4 estimate over the selected pages
-  rc = twl_gemv_int4(a->q, a->dtype, a->scores, a->score_stride, a->cand_count, a->k_int4,
-                     a->sel_pages, a->sel_count, a->sel_stride, a->kv_page_indices,
-                     a->kv_page_indptr, a->kv_last_page_len, a->batch, a->num_q_heads,
-                     a->num_kv_heads, k, a->sm_scale, stream);
-  if (rc != TWL_OK) return rc;
-  // 3. softmax + top-p + compaction to token positions
-  rc = twl_softmax_top_p_f32(a->scores, a->score_stride, a->cand_count, rows, k * TWL_PAGE,
-                             nullptr, a->top_p, a->high_mode, a->sel_pages, a->sel_stride, a->idx,
-                             a->idx_stride, a->count, nullptr, nullptr, stream);
-  if (rc != TWL_OK) return rc;
+  if (!a->split_estimator) {
+    // 2+3. INT4 estimate, softmax, top-p and compaction in one launch
+    rc = twl_gemv_top_p(a->q, a->dtype, a->k_int4, a->sel_pages, a->sel_count, a->sel_stride,
+                        a->kv_page_indices, a->kv_page_indptr, a->kv_last_page_len, a->batch,
+                        a->num_q_heads, a->num_kv_heads, k, a->sm_scale, nullptr, a->top_p,
+                        a->high_mode, a->idx, a->idx_stride, a->count,
+                        a->keep_scores ? a->scores : nullptr, a->score_stride, a->cand_count,
+                        nullptr, stream);
+    if (rc != TWL_OK) return rc;
+  } else {
+    // 2. INT4 estimate over the selected pages
+    rc = twl_gemv_int4(a->q, a->dtype, a->scores, a->score_stride, a->cand_count, a->k_int4,
+                       a->sel_pages, a->sel_count, a->sel_stride, a->kv_page_indices,
+                       a->kv_page_indptr, a->kv_last_page_len, a->batch, a->num_q_heads,
+                       a->num_kv_heads, k, a->sm_scale, stream);
+    if (rc != TWL_OK) return rc;
+    // 3. softmax + top-p + compaction to token positions
+    rc = twl_softmax_top_p_f32(a->scores, a->score_stride, a->cand_count, rows, k * TWL_PAGE,
+                               nullptr, a->top_p, a->high_mode, a->sel_pages, a->sel_stride,
+                               a->idx, a->idx_stride, a->count, nullptr, nullptr, stream);
+    if (rc != TWL_OK) return rc;
+  }
   // 4. exact attention over the survivors
   return twl_sparse_attn(a->q, a->out, a->dtype, a->k_cache, a->v_cache, a->page_stride,
                          a->token_stride, a->head_stride, a->idx, a->idx_stride, a->count,

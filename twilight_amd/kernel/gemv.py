@@ -85,6 +85,80 @@ def sparse_gemv_int4(q: torch.Tensor, k_int4: torch.Tensor, kv_page_indices: tor
     return out, out_count
 
 
+def sparse_gemv_int4_top_p(q: torch.Tensor, k_int4: torch.Tensor, kv_page_indices: torch.Tensor,
+                           kv_page_indptr: torch.Tensor, kv_last_page_len: torch.Tensor,
+                           sel_pages: torch.Tensor, sel_count: Optional[torch.Tensor],
+                           top_p, high: str = "max", max_pages: Optional[int] = None,
+                           sm_scale: Optional[float] = None, return_scores: bool = False,
+                           return_low: bool = False):
+    """Estimator + pruner in one launch: :func:`sparse_gemv_int4` over the rows' page lists, then
+    fp32 softmax, top-p bisection and compaction (twilight/pyimpl/attention.py:252-255,
+    twilight/pyimpl/top_p.py:10-15, attention.py:280-281) without materialising the scores.
+
+    Arguments as :func:`sparse_gemv_int4` (``sel_pages`` is required) and
+    :func:`twilight_amd.kernel.softmax_top_p`. Returns ``(idx int32 [B,H,16*max_pages], count
+    int32 [B,H], cand_count int32 [B,H])`` plus the raw scores and / or the final pivot when asked.
+    """
+    from .sampling import _check_p, _high_mode
+    check_input(q, "q")
+    check_dim(3, q, "q")
+    B, H, D = q.shape
+    if D != _lib.HEAD_DIM:
+        raise RuntimeError(f"head_dim must be {_lib.HEAD_DIM}, got {D}")
+    check_input(k_int4, "k_int4")
+    check_dtype(k_int4, torch.uint8, "k_int4")
+    if k_int4.dim() != 3 or k_int4.size(2) != _lib.INT4_RECORD_BYTES:
+        raise RuntimeError("k_int4 must be uint8 [pages, kv_heads, 1280]")
+    Hkv = k_int4.size(1)
+    if H % Hkv != 0:
+        raise RuntimeError(f"num_q_heads {H} must be a multiple of num_kv_heads {Hkv}")
+    for name, t in (("kv_page_indices", kv_page_indices), ("kv_page_indptr", kv_page_indptr),
+                    ("kv_last_page_len", kv_last_page_len), ("sel_pages", sel_pages)):
+        check_input(t, name)
+        check_dtype(t, torch.int32, name)
+    if kv_page_indptr.numel() != B + 1 or kv_last_page_len.numel() != B:
+        raise RuntimeError("kv_page_indptr must have B+1 and kv_last_page_len B elements")
+    if sel_pages.dim() != 3 or sel_pages.size(0) != B or sel_pages.size(1) != H:
+        raise RuntimeError("sel_pages must be int32 [B, H, S]")
+    sel_stride = sel_pages.size(2)
+    if max_pages is None:
+        max_pages = sel_stride
+    if max_pages * _lib.PAGE > _lib.MAX_CANDIDATES:
+        raise RuntimeError(f"{max_pages * _lib.PAGE} candidates exceed the supported maximum "
+                           f"{_lib.MAX_CANDIDATES}")
+    if sel_count is not None:
+        check_input(sel_count, "sel_count")
+        check_dtype(sel_count, torch.int32, "sel_count")
+        if sel_count.numel() != B * H:
+            raise RuntimeError("sel_count must have B*H elements")
+    p_arr, p_val = _check_p(top_p, B * H, q)
+    check_same_device(q, ("k_int4", k_int4), ("kv_page_indices", kv_page_indices),
+                      ("kv_page_indptr", kv_page_indptr), ("kv_last_page_len", kv_last_page_len),
+                      ("sel_pages", sel_pages), ("sel_count", sel_count))
+    dev = q.device
+    M = max_pages * _lib.PAGE
+    with torch.cuda.device(dev):
+        idx = torch.empty((B, H, M), dtype=torch.int32, device=dev)
+        count = torch.empty((B, H), dtype=torch.int32, device=dev)
+        cand = torch.empty((B, H), dtype=torch.int32, device=dev)
+        scores = (torch.full((B, H, M), float("-inf"), dtype=torch.float32, device=dev)
+                  if return_scores else None)
+        low = torch.empty((B, H), dtype=torch.float32, device=dev) if return_low else None
+        scale = 1.0 / math.sqrt(D) if sm_scale is None else float(sm_scale)
+        rc = _lib.lib().twl_gemv_top_p(
+            ptr(q), dtype_code(q.dtype, "q"), ptr(k_int4), ptr(sel_pages), ptr(sel_count),
+            sel_stride, ptr(kv_page_indices), ptr(kv_page_indptr), ptr(kv_last_page_len), B, H,
+            Hkv, max_pages, scale, ptr(p_arr), p_val, _high_mode(high), ptr(idx), M, ptr(count),
+            ptr(scores), M, ptr(cand), ptr(low), stream_of(q))
+    _lib.check(rc, "SparseGemvInt4TopP")
+    out = [idx, count, cand]
+    if return_scores:
+        out.append(scores)
+    if return_low:
+        out.append(low)
+    return tuple(out)
+
+
 def batched_sparse_gemv_int4_k(q: torch.Tensor, o: torch.Tensor, k_u8: torch.Tensor,
                                quant_scales: torch.Tensor, quant_zeros: torch.Tensor,
                                kv_page_indices: torch.Tensor, kv_page_indptr: torch.Tensor,

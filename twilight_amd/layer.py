@@ -44,7 +44,8 @@ class TwilightDecodeLayer:
     """One attention layer's decode step over a :class:`PagedKVCache`."""
 
     def __init__(self, cache: PagedKVCache, num_q_heads: int, token_budget: int = 8192,
-                 top_p: float = 0.85, high: str = "max", sm_scale: Optional[float] = None):
+                 top_p: float = 0.85, high: str = "max", sm_scale: Optional[float] = None,
+                 fused_estimator: bool = True, keep_scores: bool = False):
         if num_q_heads % cache.num_kv_heads != 0:
             raise RuntimeError("num_q_heads must be a multiple of the cache's kv heads")
         if not (0.0 < top_p <= 1.0):
@@ -55,6 +56,9 @@ class TwilightDecodeLayer:
         self.token_budget, self.top_p = int(token_budget), float(top_p)
         self.high_mode = _lib.TWL_HIGH_FIRST if high == "first" else _lib.TWL_HIGH_MAX
         self.sm_scale = 1.0 / math.sqrt(_lib.HEAD_DIM) if sm_scale is None else float(sm_scale)
+        # fused_estimator: estimate + prune in one launch; the estimator scores are then written
+        # to ``self.scores`` only when keep_scores is set (the split path always writes them)
+        self.fused_estimator, self.keep_scores = bool(fused_estimator), bool(keep_scores)
         self._alloc()
 
     @classmethod
@@ -104,11 +108,14 @@ class TwilightDecodeLayer:
         a.count = ptr(self.count)
         a.attn_workspace, a.attn_workspace_bytes = ptr(self.attn_workspace), self.attn_workspace.numel()
         a.out = ptr(self.out)
+        a.split_estimator = 0 if self.fused_estimator else 1
+        a.keep_scores = 1 if self.keep_scores else 0
         return a
 
     def forward(self, q: torch.Tensor) -> torch.Tensor:
         """``q`` [B, H, 128] in the cache dtype -> attention output [B, H, 128] (same buffer every
-        call). Intermediates stay readable as ``sel_pages/sel_count/scores/idx/count``."""
+        call). Intermediates stay readable as ``sel_pages/sel_count/idx/count`` (and ``scores``
+        with ``keep_scores`` or the split estimator)."""
         c = self.cache
         check_input(q, "q")
         check_dim(3, q, "q")
