@@ -54,19 +54,18 @@ def _time_calls(fn, iters: int, warmup: int) -> float:
     return e0.elapsed_time(e1) * 1000.0 / iters
 
 
-def cpu_baseline(N: int, H: int, budget: int, top_p: float, batch_scale: int, seed: int = 0):
-    """Times the CPU oracle (torch fp32 + the C top-p restatement) on one batch element."""
+def cpu_baseline(N: int, H: int, budget: int, top_p: float, batch_scale: int, dev, seed: int = 0):
+    """Times the CPU oracle (torch fp32 + the C top-p restatement) on one batch element drawn by
+    the generator the GPU workload uses (same planted heavy hitters), un-paged to dense K / V."""
     from oracle import native, pyimpl_port as P
     from twilight_amd import synth
     threads = torch.get_num_threads()
-    g = torch.Generator().manual_seed(seed)
-    q = torch.randn((1, H, 1, 128), generator=g).half().float()
-    k = torch.randn((1, H, N, 128), generator=g).half().float()
-    v = torch.randn((1, H, N, 128), generator=g).half().float()
-    pos = torch.randint(0, N, (H, 24), generator=g)
-    for h in range(H):
-        k[0, h, pos[h]] += 0.9 * q[0, h, 0]
-    k = k.half().float()
+    qd, kd, vd, (ids, _, _) = synth.layer_inputs_device(1, H, H, N, torch.float16, dev, seed=seed)
+    order = ids.long()
+    q = qd.float().cpu().reshape(1, H, 1, 128)
+    k = kd[order].reshape(N, H, 128).permute(1, 0, 2).float().cpu().reshape(1, H, N, 128).contiguous()
+    v = vd[order].reshape(N, H, 128).permute(1, 0, 2).float().cpu().reshape(1, H, N, 128).contiguous()
+    del qd, kd, vd
     # (A) as the reference does it: K is re-quantised inside every decode step
     t0 = time.perf_counter()
     ra = P.decode_layer_dense(q, k, v, top_p=top_p, token_budget=budget, high_mode=native.HIGH_MAX,
@@ -82,7 +81,7 @@ def cpu_baseline(N: int, H: int, budget: int, top_p: float, batch_scale: int, se
         "value": ta * 1e6 * batch_scale, "unit": "us/layer", "cores": threads, "kind": "port",
         "value_k_prequantised": tb * 1e6 * batch_scale,
         "sample": (f"1 of {batch_scale} batch elements (32 heads x {N} tokens, budget {budget}, "
-                   f"p {top_p}) through oracle.pyimpl_port.decode_layer_dense, one run each, "
+                   f"p {top_p}; same generator as the GPU workload) through oracle.pyimpl_port.decode_layer_dense, one run each, "
                    f"time x {batch_scale}; `value` re-quantises K every step like "
                    "twilight/pyimpl/attention.py:247-251, `value_k_prequantised` does not; torch "
                    f"uses {threads} threads, the C quantiser / top-p one"),
@@ -300,7 +299,7 @@ def main() -> int:
 
     cpu = None
     if not args.no_cpu_baseline and not llama:
-        cpu = cpu_baseline(N, H, args.budget, args.top_p, B)
+        cpu = cpu_baseline(N, H, args.budget, args.top_p, B, dev)
 
     line = {
         "metric": "us/decode-layer at 32k ctx (select+prune+attn)",

@@ -247,7 +247,7 @@ static void launch_fused(const FusedArgs& a, uint32_t rows, hipStream_t s) {
   else if (k <= 64) TWL_FUSED_CASE(256, 4);
   else if (k <= 128) TWL_FUSED_CASE(256, 8);
   else if (k <= 256) TWL_FUSED_CASE(256, 16);
-  else if (k <= 512) TWL_FUSED_CASE(1024, 8);
+  else if (k <= 512) TWL_FUSED_CASE(512, 16);  // measured faster than 1024 x 8
   else if (k <= 1024) TWL_FUSED_CASE(1024, 16);
   else TWL_FUSED_CASE(1024, 32);
 #undef TWL_FUSED_CASE
