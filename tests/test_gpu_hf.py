@@ -1,0 +1,84 @@
+"""GPU test of the Hugging Face integration: a random-initialised Llama decodes through the
+patched attention modules (twilight/pyimpl/attention.py:351-418, 481-493 is what is mirrored)."""
+import json
+
+import pytest
+import torch
+
+from twilight_amd import hf
+from test_hf_host import CFG, _tiny_llama
+
+pytestmark = pytest.mark.gpu
+
+
+def _decode(model, ids, steps):
+    """Greedy decode; returns the logits of every decode step [steps, B, vocab] and the tokens."""
+    logits, toks = [], []
+    with torch.no_grad():
+        out = model(ids, use_cache=True)
+        past = out.past_key_values
+        nxt = out.logits[:, -1].argmax(-1, keepdim=True)
+        for _ in range(steps):
+            out = model(nxt, past_key_values=past, use_cache=True)
+            past = out.past_key_values
+            logits.append(out.logits[:, -1].float())
+            toks.append(nxt)
+            nxt = out.logits[:, -1].argmax(-1, keepdim=True)
+    return torch.stack(logits), torch.cat(toks, dim=1)
+
+
+def _forced_decode(model, ids, forced):
+    """Decode feeding the given tokens (so two models see identical inputs at every step)."""
+    logits = []
+    with torch.no_grad():
+        out = model(ids, use_cache=True)
+        past = out.past_key_values
+        for s in range(forced.shape[1]):
+            out = model(forced[:, s:s + 1], past_key_values=past, use_cache=True)
+            past = out.past_key_values
+            logits.append(out.logits[:, -1].float())
+    return torch.stack(logits)
+
+
+@pytest.mark.parametrize("kv_heads", [4, 2])
+def test_decode_with_p_one_equals_dense_decode(dev, kv_heads):
+    # p = 1 and a budget beyond the context keep every token with non-zero estimated probability:
+    # the patched model must reproduce dense decoding up to fp16 rounding of the attention output
+    model = _tiny_llama(layers=4, heads=4, kv_heads=kv_heads, dtype=torch.float16).to(dev)
+    ids = torch.randint(0, 97, (2, 200), generator=torch.Generator().manual_seed(2)).to(dev)
+    ref_logits, toks = _decode(model, ids, 12)           # crosses a page boundary at step 8
+    cfg = json.loads(json.dumps(CFG))
+    cfg["selector"]["token_budget"] = 4096
+    cfg["weight_pruner"]["threshold"] = 1.0
+    info, _ = hf.enable_sparse_attention(model, cfg, enable_budget_info=True, reserve_tokens=64)
+    got = _forced_decode(model, ids, toks)
+    assert torch.isfinite(got).all()
+    assert torch.allclose(got, ref_logits, rtol=2e-2, atol=2e-2), (got - ref_logits).abs().max()
+    # budget statistics: one query per decode step, layers 2 and 3 report, everything is kept
+    assert len(info._budget_num) == 12 and sorted(info._budget_num[0]) == [2, 3]
+    first = info._budget_num[0][2].cpu()
+    assert first.numel() == 2 * 4 and int(first.min()) >= 195 and int(first.max()) <= 201
+    hf.disable_sparse_attention(model)
+    again = _forced_decode(model, ids, toks)
+    assert torch.allclose(again, ref_logits, rtol=1e-3, atol=1e-3)
+
+
+def test_decode_prunes_and_reports_budgets(dev):
+    model = _tiny_llama(layers=4, heads=4, kv_heads=2, dtype=torch.float16).to(dev)
+    ids = torch.randint(0, 97, (3, 333), generator=torch.Generator().manual_seed(3)).to(dev)
+    ref_logits, toks = _decode(model, ids, 6)
+    info, _ = hf.enable_sparse_attention(model, CFG, enable_budget_info=True, reserve_tokens=32)
+    got = _forced_decode(model, ids, toks)                # budget 64 tokens, p = 0.9
+    assert torch.isfinite(got).all()
+    per_query = info.get_avg_budget_per_query()
+    assert len(per_query) == 6 and all(1 <= b <= 64 for b in per_query)
+    assert info.get_total_avg_budget_B0() == 64.0
+    # a random-initialised model attends diffusely, so pruning to <= 64 of 333 tokens moves the
+    # logits, but not arbitrarily: the same tokens stay likely
+    cos = torch.nn.functional.cosine_similarity(got.flatten(1), ref_logits.flatten(1), dim=1)
+    assert float(cos.min()) > 0.5
+    # a second prompt through the same patched model starts from a fresh paged cache
+    ids2 = ids[:, :100].contiguous()
+    got2 = _forced_decode(model, ids2, toks[:, :3])
+    assert torch.isfinite(got2).all()
+    assert model.model.layers[2].self_attn._twilight_state.seq_len == 103

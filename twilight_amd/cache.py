@@ -47,6 +47,11 @@ class PagedKVCache:
         npg = ip[1:] - ip[:-1]
         self.max_pages_per_req = int(npg.max().item())
         self._seq_lens = ((npg - 1) * PAGE + kv_last_page_len.cpu().long()).tolist()
+        # host mirrors of the table: append() never reads the device copies back
+        ids = kv_page_indices.cpu().tolist()
+        ipl = ip.tolist()
+        self._per_req = [ids[ipl[b]:ipl[b + 1]] for b in range(len(ipl) - 1)]
+        self._last = kv_last_page_len.cpu().tolist()
 
     @property
     def batch(self) -> int:
@@ -98,31 +103,35 @@ class PagedKVCache:
         token, extends the page table when a request's last page is full (taking ids from
         ``free_pages``), and refreshes the shadow records of the touched pages."""
         B = self.batch
-        ip = self.kv_page_indptr.cpu().tolist()
-        idx = self.kv_page_indices.cpu().tolist()
-        last = self.kv_last_page_len.cpu().tolist()
-        per_req = [idx[ip[b]:ip[b + 1]] for b in range(B)]
+        per_req, last = self._per_req, self._last
         touched, valid, slots = [], [], []
+        grew = False
         for b in range(B):
             if last[b] == PAGE:
                 if not free_pages:
                     raise RuntimeError("PagedKVCache.append: no free page left")
                 per_req[b].append(int(free_pages.pop(0)))
                 last[b] = 0
+                grew = True
             page = per_req[b][-1]
             slots.append((page, last[b]))
             last[b] += 1
+            self._seq_lens[b] += 1
             touched.append(page)
             valid.append(last[b])
         pg = torch.tensor([s[0] for s in slots], device=self.device)
         sl = torch.tensor([s[1] for s in slots], device=self.device)
         self.k_cache[pg, sl] = k_new.to(self.device, self.dtype)
         self.v_cache[pg, sl] = v_new.to(self.device, self.dtype)
-        flat = [p for r in per_req for p in r]
-        ptr = [0]
-        for r in per_req:
-            ptr.append(ptr[-1] + len(r))
-        self.set_page_table(torch.tensor(flat, dtype=torch.int32), torch.tensor(ptr, dtype=torch.int32),
-                            torch.tensor(last, dtype=torch.int32))
+        if grew:  # a request took a new page: the CSR arrays change shape
+            flat = [p for r in per_req for p in r]
+            ptr = [0]
+            for r in per_req:
+                ptr.append(ptr[-1] + len(r))
+            self.kv_page_indices = torch.tensor(flat, dtype=torch.int32, device=self.device)
+            self.kv_page_indptr = torch.tensor(ptr, dtype=torch.int32, device=self.device)
+            self.max_pages_per_req = max(len(r) for r in per_req)
+        # same tensor object every step, so cached argument blocks of the layer stay valid
+        self.kv_last_page_len.copy_(torch.tensor(last, dtype=torch.int32))
         self.rebuild_shadow(torch.tensor(touched, dtype=torch.int32, device=self.device),
                             torch.tensor(valid, dtype=torch.int32, device=self.device))

@@ -1,0 +1,198 @@
+"""Hugging Face Llama / Mistral integration of the Select-then-Prune decode path.
+
+Mirrors ``enable_sparse_attention(model, sparse_config, enable_budget_info, enable_score_info)``
+of twilight/pyimpl/attention.py:351-418 (config template :360-377, module patching :481-493) and
+the budget statistics of twilight/pyimpl/state.py:158-234. Prefill (q_len > 1) runs the model's
+own attention, as the reference runs flash attention there (attention.py:158-183); a decode step
+(q_len == 1) of a patched layer appends the new token to a :class:`PagedKVCache` (K / V pages,
+INT4 K shadow, Quest metadata) and calls :class:`TwilightDecodeLayer` instead of attending over the
+whole context. The first two layers stay dense when ``skip_first_two_layers`` is set
+(attention.py:199-201, config default :413).
+
+Only the configuration the decode path implements is accepted: selector ``quest`` (chunk size 16),
+weight estimator ``min_max_quant`` with 4 bits, weight pruner ``top_p``; anything else raises.
+"""
+from __future__ import annotations
+
+import types
+from typing import Dict, List, Optional, Tuple
+
+import torch
+
+from . import _lib
+from .cache import PagedKVCache
+from .layer import TwilightDecodeLayer, parse_sparse_config
+
+PAGE = _lib.PAGE
+
+
+class HistoryBudgetInfo:
+    """Per query (= one decode step through the model), per layer: survivors per head after
+    pruning (the reference's "B1") and the selector's token budget ("B0"). Same accounting as
+    twilight/pyimpl/state.py:158-234: a new query starts whenever the layer id does not follow the
+    previous one, and averages skip layers 0 and 1."""
+
+    def __init__(self) -> None:
+        self.reset()
+
+    def reset(self) -> None:
+        self._budget_num: List[Dict[int, torch.Tensor]] = []
+        self._B0: List[Dict[int, int]] = []
+        self._last_layer_id = -999
+
+    def update(self, layer_id: int, head_budgets: torch.Tensor) -> None:
+        """``head_budgets``: survivors per (batch, head), any shape; stored flattened."""
+        if layer_id != self._last_layer_id + 1:
+            self._budget_num.append({})
+            self._B0.append({})
+        self._budget_num[-1][layer_id] = head_budgets.detach().flatten().clone()
+        self._last_layer_id = layer_id
+
+    def update_B0(self, layer_id: int, token_budget: int) -> None:
+        if not self._B0:
+            self._B0.append({})
+        self._B0[-1][layer_id] = int(token_budget)
+
+    def get_avg_budget_per_layer_single_query(self, query_index: int) -> List[float]:
+        return [float(v.float().mean()) for v in self._budget_num[query_index].values()]
+
+    def get_avg_budget_cur_query(self) -> List[float]:
+        return self.get_avg_budget_per_layer_single_query(-1)
+
+    def get_avg_budget_per_query(self) -> List[float]:
+        out = []
+        for q in self._budget_num:
+            vals = [float(v.float().mean()) for lid, v in q.items() if lid > 1]
+            out.append(sum(vals) / len(vals) if vals else float("nan"))
+        return out
+
+    def get_avg_budget_per_query_B0(self) -> List[float]:
+        out = []
+        for q in self._B0:
+            vals = [b for lid, b in q.items() if lid > 1]
+            out.append(sum(vals) / len(vals) if vals else float("nan"))
+        return out
+
+    def get_total_avg_budget(self) -> float:
+        v = self.get_avg_budget_per_query()
+        return sum(v) / len(v) if v else float("nan")
+
+    def get_total_avg_budget_B0(self) -> float:
+        v = self.get_avg_budget_per_query_B0()
+        return sum(v) / len(v) if v else float("nan")
+
+    def print_budget_info_single_query(self, query_index: int = -1) -> None:
+        for lid, v in self._budget_num[query_index].items():
+            print(f"Layer {lid}: {v.tolist()} Head Average: {float(v.float().mean()):.2f}")
+
+
+class _LayerState:
+    """What a patched attention module carries between calls."""
+
+    def __init__(self, cfg: dict, reserve_tokens: int, budget_info: Optional[HistoryBudgetInfo]):
+        self.cfg, self.reserve_tokens, self.budget_info = cfg, reserve_tokens, budget_info
+        self.cache: Optional[PagedKVCache] = None
+        self.layer: Optional[TwilightDecodeLayer] = None
+        self.free: List[int] = []
+        self.seq_len = 0
+
+    def reset(self) -> None:
+        self.cache, self.layer, self.free, self.seq_len = None, None, [], 0
+
+
+def _fill_from_prefill(st: _LayerState, k: torch.Tensor, v: torch.Tensor, num_q_heads: int) -> None:
+    """Page the prefill K / V [B, Hkv, N, 128] of a layer and size everything for
+    ``reserve_tokens`` more tokens per request."""
+    B, _, N, _ = k.shape
+    npg = (N + PAGE - 1) // PAGE
+    spare_per_req = (st.reserve_tokens + PAGE - 1) // PAGE + 1
+    st.cache = PagedKVCache.from_dense(k, v, k.device, spare_pages=B * spare_per_req)
+    st.free = list(range(B * npg, B * (npg + spare_per_req)))
+    st.layer = TwilightDecodeLayer(st.cache, num_q_heads, reserve_pages=npg + spare_per_req, **st.cfg)
+    st.seq_len = N
+
+
+def _twilight_attention_forward(self, hidden_states, position_embeddings=None, attention_mask=None,
+                                past_key_values=None, **kwargs):
+    """Replacement of ``LlamaAttention.forward``: the module's own forward for prefill, the
+    Select-then-Prune layer for decode (twilight/pyimpl/attention.py:59-306 split the same way)."""
+    from transformers.models.llama.modeling_llama import apply_rotary_pos_emb
+    st: _LayerState = self._twilight_state
+    q_len = hidden_states.shape[1]
+    if q_len > 1 or past_key_values is None:
+        out = self._twilight_orig_forward(hidden_states, position_embeddings=position_embeddings,
+                                          attention_mask=attention_mask,
+                                          past_key_values=past_key_values, **kwargs)
+        st.reset()
+        if past_key_values is not None:
+            lay = past_key_values.layers[self.layer_idx]
+            if lay.keys.is_cuda:  # the paged cache and its kernels exist on the GPU only
+                _fill_from_prefill(st, lay.keys, lay.values, self.config.num_attention_heads)
+        return out
+    if st.cache is None:
+        raise RuntimeError("decode step without a paged cache: no prefill ran through this layer "
+                           "with use_cache=True on a GPU (there is no CPU path)")
+    B = hidden_states.shape[0]
+    hidden_shape = (B, 1, -1, self.head_dim)
+    q = self.q_proj(hidden_states).view(hidden_shape).transpose(1, 2)
+    k = self.k_proj(hidden_states).view(hidden_shape).transpose(1, 2)
+    v = self.v_proj(hidden_states).view(hidden_shape).transpose(1, 2)
+    cos, sin = position_embeddings
+    q, k = apply_rotary_pos_emb(q, k, cos, sin)
+    past_key_values.update(k, v, self.layer_idx)      # keeps the model's own cache consistent
+    st.cache.append(k[:, :, 0], v[:, :, 0], st.free)
+    st.seq_len += 1
+    out = st.layer(q[:, :, 0].contiguous())           # [B, H, 128]
+    if st.budget_info is not None:
+        st.budget_info.update(self.layer_idx, st.layer.count)
+        st.budget_info.update_B0(self.layer_idx, min(st.layer.token_budget, st.seq_len))
+    attn_output = self.o_proj(out.reshape(B, 1, -1))
+    return attn_output, None
+
+
+def enable_sparse_attention(model, sparse_config: Dict, enable_budget_info: bool = False,
+                            enable_score_info: bool = False, reserve_tokens: int = 4096,
+                            high: str = "max") -> Tuple[Optional[HistoryBudgetInfo], None]:
+    """Patch every Llama / Mistral attention module of ``model`` (twilight/pyimpl/attention.py:
+    351-418, 481-493). ``sparse_config`` is the reference's JSON template
+    (benchmark/configs/config_quest_twi.json). ``reserve_tokens``: decode tokens per request the
+    paged caches are sized for. Returns ``(budget_info, None)``; the accumulated-score statistic
+    of the reference needs the dense attention weights, which this path never forms."""
+    if enable_score_info:
+        raise RuntimeError("enable_score_info needs dense attention weights; not available here")
+    for part in ("compressor",):
+        t = sparse_config.get(part, {}).get("type", "none")
+        if str(t).lower() not in ("none", ""):
+            raise RuntimeError(f"{part} type {t!r} is not supported")
+    if sparse_config.get("use_estimated_weights_in_attn", False):
+        raise RuntimeError("use_estimated_weights_in_attn is not supported")
+    cfg = parse_sparse_config(sparse_config)
+    cfg["high"] = high
+    skip = 2 if sparse_config.get("skip_first_two_layers", True) else 0
+    budget_info = HistoryBudgetInfo() if enable_budget_info else None
+    patched = 0
+    for name, module in model.named_modules():
+        if not all(hasattr(module, a) for a in ("q_proj", "k_proj", "v_proj", "o_proj", "layer_idx")):
+            continue
+        if getattr(module, "head_dim", None) != _lib.HEAD_DIM:
+            raise RuntimeError(f"{name}: head_dim must be {_lib.HEAD_DIM}")
+        if hasattr(module, "_twilight_state"):
+            raise RuntimeError("enable_sparse_attention was already called on this model")
+        if module.layer_idx < skip:
+            continue
+        module._twilight_state = _LayerState(dict(cfg), reserve_tokens, budget_info)
+        module._twilight_orig_forward = module.forward
+        module.forward = types.MethodType(_twilight_attention_forward, module)
+        patched += 1
+    if patched == 0:
+        raise RuntimeError("no attention module was patched")
+    return budget_info, None
+
+
+def disable_sparse_attention(model) -> None:
+    """Undo :func:`enable_sparse_attention` (the reference's ``reset_sparse_config``,
+    attention.py:496-499, only clears its global flag)."""
+    for _, module in model.named_modules():
+        if hasattr(module, "_twilight_state"):
+            module.forward = module._twilight_orig_forward
+            del module._twilight_state, module._twilight_orig_forward

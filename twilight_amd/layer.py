@@ -45,7 +45,8 @@ class TwilightDecodeLayer:
 
     def __init__(self, cache: PagedKVCache, num_q_heads: int, token_budget: int = 8192,
                  top_p: float = 0.85, high: str = "max", sm_scale: Optional[float] = None,
-                 fused_estimator: bool = True, keep_scores: bool = False):
+                 fused_estimator: bool = True, keep_scores: bool = False,
+                 reserve_pages: int = 0):
         if num_q_heads % cache.num_kv_heads != 0:
             raise RuntimeError("num_q_heads must be a multiple of the cache's kv heads")
         if not (0.0 < top_p <= 1.0):
@@ -59,6 +60,9 @@ class TwilightDecodeLayer:
         # fused_estimator: estimate + prune in one launch; the estimator scores are then written
         # to ``self.scores`` only when keep_scores is set (the split path always writes them)
         self.fused_estimator, self.keep_scores = bool(fused_estimator), bool(keep_scores)
+        # work buffers are sized for requests of up to reserve_pages pages, so a context that grows
+        # during decode does not reallocate them every time a request takes a new page
+        self.reserve_pages = int(reserve_pages)
         self._alloc()
 
     @classmethod
@@ -68,14 +72,15 @@ class TwilightDecodeLayer:
     def _alloc(self) -> None:
         c = self.cache
         B, H, dev = c.batch, self.H, c.device
-        self.k_pages = quest_num_pages(self.token_budget, c.max_pages_per_req)
+        cap = max(c.max_pages_per_req, self.reserve_pages)
+        self.k_pages = quest_num_pages(self.token_budget, cap)
         M = self.k_pages * _lib.PAGE
         if M > _lib.MAX_CANDIDATES:
             raise RuntimeError(f"token budget {M} exceeds the supported maximum {_lib.MAX_CANDIDATES}")
         i32, f32 = torch.int32, torch.float32
         self.sel_pages = torch.zeros((B, H, self.k_pages), dtype=i32, device=dev)
         self.sel_count = torch.zeros((B, H), dtype=i32, device=dev)
-        self.page_scores = torch.zeros((B, H, c.max_pages_per_req), dtype=f32, device=dev)
+        self.page_scores = torch.zeros((B, H, cap), dtype=f32, device=dev)
         self.scores = torch.zeros((B, H, M), dtype=f32, device=dev)
         self.cand_count = torch.zeros((B, H), dtype=i32, device=dev)
         self.idx = torch.zeros((B, H, M), dtype=i32, device=dev)
@@ -83,7 +88,7 @@ class TwilightDecodeLayer:
         self.out = torch.zeros((B, H, _lib.HEAD_DIM), dtype=c.dtype, device=dev)
         ws = int(_lib.lib().twl_sparse_attn_workspace_bytes(B * H, M))
         self.attn_workspace = torch.zeros(ws, dtype=torch.uint8, device=dev)
-        self._shape = (B, c.max_pages_per_req)
+        self._shape = (B, cap)
         self._args, self._args_key = None, None
 
     def _build_args(self, q: torch.Tensor) -> "_lib.LayerArgs":
@@ -119,7 +124,7 @@ class TwilightDecodeLayer:
         c = self.cache
         check_input(q, "q")
         check_dim(3, q, "q")
-        if (c.batch, c.max_pages_per_req) != self._shape:
+        if c.batch != self._shape[0] or c.max_pages_per_req > self._shape[1]:
             self._alloc()
         if tuple(q.shape) != (c.batch, self.H, _lib.HEAD_DIM) or q.dtype != c.dtype:
             raise RuntimeError(f"q must be [{c.batch}, {self.H}, {_lib.HEAD_DIM}] of {c.dtype}")
@@ -127,7 +132,7 @@ class TwilightDecodeLayer:
             raise RuntimeError(f"q must be on {c.device}")
         key = (q.data_ptr(), c.k_cache.data_ptr(), c.v_cache.data_ptr(), c.k_int4.data_ptr(),
                c.meta.data_ptr(), c.kv_page_indices.data_ptr(), c.kv_page_indptr.data_ptr(),
-               c.kv_last_page_len.data_ptr())
+               c.kv_last_page_len.data_ptr(), c.max_pages_per_req)
         if self._args_key != key:
             self._args, self._args_key = self._build_args(q), key
         a = self._args
