@@ -268,6 +268,24 @@ int twl_bgemv_int8(const void* q_label, const int8_t* k_label, const void* k_sca
                    int64_t ss_h, int64_t so_b, int64_t so_h, int64_t so_n, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
+ * Base-2 log-sum-exp of per-block-quantised int8 Q.K^T (int8 matrix cores).
+ * Replaces: qk_int8_per_block, twilight/kernel/triton/qk_int8_per_block.py:22-143 (its `lse`
+ * output, :105-109; its first output is identically zero because V is never accumulated).
+ *   lse[b,h,m] = log2 sum_n 2^( float(q[b,h,m,:] . k[b,h/group,n,:]) * q_scale[b,h,m/128]
+ *                                                                  * k_scale[b,h/group,n/64] )
+ * over n < 64*ceil(kv_len/64); keys in [kv_len, 64*ceil(kv_len/64)) count as all-zero rows, as the
+ * reference's masked loads make them (:36-37). q / k int8 with byte strides (batch, head, row) and
+ * contiguous head_dim (64 or 128); pointers and strides must be multiples of 16. q_scale fp32
+ * [batch, num_q_heads, ceil(qo_len/128)], k_scale fp32 [batch, num_kv_heads, ceil(kv_len/64)],
+ * lse fp32 [batch, num_q_heads, qo_len].
+ * ------------------------------------------------------------------------------------------- */
+int twl_qk_int8_lse(const int8_t* q, const int8_t* k, const float* q_scale, const float* k_scale,
+                    float* lse, uint32_t batch, uint32_t num_q_heads, uint32_t num_kv_heads,
+                    uint32_t qo_len, uint32_t kv_len, uint32_t head_dim, int64_t sq_b,
+                    int64_t sq_h, int64_t sq_n, int64_t sk_b, int64_t sk_h, int64_t sk_n,
+                    void* stream);
+
+/* ---------------------------------------------------------------------------------------------
  * The whole decode layer on one stream: quest select -> INT4 GEMV -> softmax + top-p -> sparse
  * attention (twilight/pyimpl/attention.py:188-306 for q_len == 1). Every intermediate is a
  * caller-provided buffer (see the field comments); no host synchronisation happens inside.

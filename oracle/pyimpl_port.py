@@ -309,3 +309,37 @@ def bgemv_int8_ref(q_label: torch.Tensor, k_label: torch.Tensor, k_scales: torch
     q = q_label.float().view(B, H, 1, r)                                      # :86
     k = k.view(B, n_ctx, H, r).transpose(1, 2).transpose(2, 3)                # :87
     return torch.matmul(q, k).squeeze(-2)                                     # :89
+
+
+def qk_int8_lse_ref(q: torch.Tensor, k: torch.Tensor, q_scale: torch.Tensor, k_scale: torch.Tensor):
+    """The `lse` output of qk_int8_per_block, twilight/kernel/triton/qk_int8_per_block.py:22-109,
+    block by block in the kernel's own order and arithmetic (fp32; exp2 / log2).
+
+    ``q`` int8 [b,h_qo,qo_len,d], ``k`` int8 [b,h_kv,kv_len,d] (HND), ``q_scale`` fp32
+    [b,h_qo,ceil(qo_len/128)], ``k_scale`` fp32 [b,h_kv,ceil(kv_len/64)]. Keys past kv_len in the
+    last 64-block are zero rows (masked load, :36-37) and take part with score 0.
+    Returns fp32 [b,h_qo,qo_len].
+    """
+    b, h_qo, qo_len, d = q.shape
+    _, h_kv, kv_len, _ = k.shape
+    group = h_qo // h_kv
+    BM, BN = 128, 64                                                           # :112-113
+    nb = (kv_len + BN - 1) // BN
+    kp = torch.zeros((b, h_kv, nb * BN, d), dtype=torch.int64)
+    kp[:, :, :kv_len] = k.long()
+    kp = kp.repeat_interleave(group, dim=1)                                    # :74,80 (off_h // groups)
+    ks = k_scale.float().reshape(b, h_kv, nb).repeat_interleave(group, dim=1)
+    qs = q_scale.float().reshape(b, h_qo, -1)
+    rows = torch.arange(qo_len)
+    qsr = qs[:, :, rows // BM]                                                 # [b,h,qo_len]
+    m_i = torch.full((b, h_qo, qo_len), float("-inf"))                         # :79
+    l_i = torch.ones((b, h_qo, qo_len))                                        # :80
+    ql = q.long()
+    for j in range(nb):                                                        # :33
+        dot = torch.matmul(ql, kp[:, :, j * BN:(j + 1) * BN].transpose(2, 3))  # exact in int64
+        qk = dot.float() * qsr[..., None] * ks[:, :, j, None, None]            # :39
+        m_ij = torch.maximum(m_i, qk.max(-1).values)                           # :40
+        p = torch.exp2(qk - m_ij[..., None])                                   # :41-42
+        l_i = l_i * torch.exp2(m_i - m_ij) + p.sum(-1)                         # :45-46
+        m_i = m_ij                                                             # :48
+    return torch.log2(l_i) + m_i                                               # :107-108

@@ -56,3 +56,43 @@ def test_bgemv_int8_ragged(dev):
     assert torch.allclose(out.cpu().float(), ref, atol=2e-3, rtol=2e-3)
     with pytest.raises(RuntimeError):
         K.bgemv_int8(q.to(dev), k8.to(dev), scales.to(dev), out[:, :, :-1])
+
+
+@pytest.mark.parametrize("layout", ["HND", "NHD"])
+@pytest.mark.parametrize("b,h_qo,h_kv,qo_len,kv_len,d", [
+    (2, 4, 2, 150, 100, 128),     # partial query block, partial key block (zero-padded tail), GQA
+    (1, 2, 2, 1, 1000, 128),      # decode: one query row
+    (1, 8, 1, 300, 257, 64),      # head_dim 64, MQA
+    (1, 1, 1, 128, 64, 128),      # exactly one block each way
+])
+def test_qk_int8_per_block_lse(dev, layout, b, h_qo, h_kv, qo_len, kv_len, d):
+    # twilight/kernel/triton/qk_int8_per_block.py:111-143: lse in base 2, first output all zeros
+    g = torch.Generator().manual_seed(qo_len + kv_len)
+    q = torch.randint(-127, 128, (b, h_qo, qo_len, d), generator=g, dtype=torch.int8)
+    k = torch.randint(-127, 128, (b, h_kv, kv_len, d), generator=g, dtype=torch.int8)
+    qs = torch.rand((b, h_qo, (qo_len + 127) // 128), generator=g) * 2e-3 + 5e-4
+    ks = torch.rand((b, h_kv, (kv_len + 63) // 64), generator=g) * 2e-3 + 5e-4
+    want = P.qk_int8_lse_ref(q, k, qs, ks)
+    qd, kd = q.to(dev), k.to(dev)
+    if layout == "NHD":
+        qd, kd = qd.transpose(1, 2).contiguous(), kd.transpose(1, 2).contiguous()
+    o, lse = K.qk_int8_per_block(qd, kd, qs.to(dev), ks.to(dev), tensor_layout=layout,
+                                 output_dtype=torch.float16, return_lse=True)
+    assert o.shape == qd.shape and o.dtype == torch.float16 and not o.any()
+    # integer products are exact; exp2 / log2 and the summation order differ by a few ulps
+    assert torch.allclose(lse.cpu(), want, rtol=1e-5, atol=2e-5), (lse.cpu() - want).abs().max()
+    o2, lse2 = K.qk_int8_per_block(qd, kd, qs.to(dev), ks.to(dev), tensor_layout=layout)
+    assert lse2.numel() == 0 and lse2.device.type == "cpu"
+
+
+def test_qk_int8_per_block_errors(dev):
+    q = torch.zeros((1, 2, 8, 128), dtype=torch.int8, device=dev)
+    s = torch.ones((1, 2, 1), device=dev)
+    with pytest.raises(ValueError):
+        K.qk_int8_per_block(q, q, s, s, tensor_layout="XYZ")
+    with pytest.raises(RuntimeError):
+        K.qk_int8_per_block(q.float(), q, s, s, return_lse=True)
+    with pytest.raises(RuntimeError):
+        K.qk_int8_per_block(q[..., :96], q[..., :96], s, s, return_lse=True)   # head_dim 96
+    with pytest.raises(RuntimeError):
+        K.qk_int8_per_block(q, q, s[:, :1], s, return_lse=True)               # q_scale too short

@@ -119,3 +119,26 @@ def test_decode_layer_dense_consistency():
     w = torch.softmax((q @ k.transpose(2, 3)) / math.sqrt(128), -1)
     top8 = w.topk(8, dim=-1).values.sum(-1)
     assert torch.all((top8 > 0.55) & (top8 < 0.66))
+
+
+def test_qk_int8_lse_oracle_is_a_base2_logsumexp():
+    # closed form: lse = log2( sum_n 2^s[m][n] + (#padded keys) * 2^0 ), evaluated in float64 from
+    # the dequantised product; pins scale indexing (q block 128, k block 64, GQA head mapping) and
+    # the zero-padded tail of the last key block
+    g = torch.Generator().manual_seed(0)
+    b, h_qo, h_kv, qo_len, kv_len, d = 2, 4, 2, 150, 100, 64
+    q = torch.randint(-127, 128, (b, h_qo, qo_len, d), generator=g, dtype=torch.int8)
+    k = torch.randint(-127, 128, (b, h_kv, kv_len, d), generator=g, dtype=torch.int8)
+    qs = torch.rand((b, h_qo, 2), generator=g) * 2e-3 + 1e-3
+    ks = torch.rand((b, h_kv, 2), generator=g) * 2e-3 + 1e-3
+    got = P.qk_int8_lse_ref(q, k, qs, ks).double()
+    krep = k.double().repeat_interleave(2, dim=1)
+    s = torch.matmul(q.double(), krep.transpose(2, 3))
+    s = s * qs.double()[:, :, torch.arange(qo_len) // 128][..., None]
+    s = s * ks.double().repeat_interleave(2, dim=1)[:, :, torch.arange(kv_len) // 64][:, :, None, :]
+    want = torch.log2(torch.exp2(s).sum(-1) + (128 - kv_len))
+    assert torch.allclose(got, want, rtol=1e-5, atol=1e-5)
+    # no padding when kv_len is a multiple of 64: a plain logsumexp (in base 2)
+    got2 = P.qk_int8_lse_ref(q, k[:, :, :64], qs, ks[:, :, :1]).double()
+    want2 = torch.logsumexp(s[..., :64] * math.log(2.0), dim=-1) / math.log(2.0)
+    assert torch.allclose(got2, want2, rtol=1e-5, atol=1e-5)

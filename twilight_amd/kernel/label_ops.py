@@ -59,3 +59,49 @@ def bgemv_int8(Q_Label: torch.Tensor, K_Label: torch.Tensor, K_Scales: torch.Ten
                                        *Out.stride(), stream_of(Q_Label))
     _lib.check(rc, "BgemvInt8")
     return Out
+
+
+def qk_int8_per_block(q: torch.Tensor, k: torch.Tensor, q_scale: torch.Tensor, k_scale: torch.Tensor,
+                      tensor_layout: str = "HND", output_dtype: torch.dtype = torch.float16,
+                      return_lse: bool = False):
+    """Same call as twilight/kernel/triton/qk_int8_per_block.py:111-143: ``q`` / ``k`` int8
+    [b,h,n,d] ("HND") or [b,n,h,d] ("NHD") quantised per 128 query rows / 64 key rows with fp32
+    ``q_scale`` [b,h_qo,ceil(qo_len/128)] and ``k_scale`` [b,h_kv,ceil(kv_len/64)]. Returns
+    ``(o, lse)``: ``o`` is the reference's first output, all zeros of ``q``'s shape (it never
+    accumulates V, :30-49,101-102); ``lse`` fp32 [b,h_qo,qo_len] is the base-2 log-sum-exp of the
+    scaled scores, or an empty CPU tensor when ``return_lse`` is False (:127-130)."""
+    for name, t in (("q", q), ("k", k), ("q_scale", q_scale), ("k_scale", k_scale)):
+        check_cuda(t, name)
+    check_dim(4, q, "q"); check_dim(4, k, "k")
+    check_dtype(q, torch.int8, "q"); check_dtype(k, torch.int8, "k")
+    if tensor_layout == "HND":
+        b, h_qo, qo_len, d = q.shape
+        _, h_kv, kv_len, _ = k.shape
+        sq, sk = (q.stride(0), q.stride(1), q.stride(2)), (k.stride(0), k.stride(1), k.stride(2))
+    elif tensor_layout == "NHD":
+        b, qo_len, h_qo, d = q.shape
+        _, kv_len, h_kv, _ = k.shape
+        sq, sk = (q.stride(0), q.stride(2), q.stride(1)), (k.stride(0), k.stride(2), k.stride(1))
+    else:
+        raise ValueError(f"tensor_layout {tensor_layout} not supported")
+    if k.size(0) != b or k.size(3) != d or q.stride(3) != 1 or k.stride(3) != 1:
+        raise RuntimeError("q and k must share batch and head_dim, with contiguous head_dim")
+    if d not in (64, 128) or h_kv == 0 or h_qo % h_kv != 0:
+        raise RuntimeError("head_dim must be 64 or 128 and h_qo a multiple of h_kv")
+    o = torch.zeros(q.shape, dtype=output_dtype, device=q.device)
+    if not return_lse:
+        return o, torch.empty([0], dtype=torch.float32, device="cpu")
+    mb, nb = (qo_len + 127) // 128, (kv_len + 63) // 64
+    qs = q_scale.to(torch.float32).contiguous()
+    ks = k_scale.to(torch.float32).contiguous()
+    if qs.numel() != b * h_qo * mb or ks.numel() != b * h_kv * nb:
+        raise RuntimeError("q_scale must have b*h_qo*ceil(qo_len/128) and k_scale "
+                           "b*h_kv*ceil(kv_len/64) elements")
+    check_same_device(q, ("k", k), ("q_scale", q_scale), ("k_scale", k_scale))
+    with torch.cuda.device(q.device):
+        lse = torch.empty([b, h_qo, qo_len], dtype=torch.float32, device=q.device)
+        if qo_len and kv_len:
+            rc = _lib.lib().twl_qk_int8_lse(ptr(q), ptr(k), ptr(qs), ptr(ks), ptr(lse), b, h_qo,
+                                            h_kv, qo_len, kv_len, d, *sq, *sk, stream_of(q))
+            _lib.check(rc, "QkInt8PerBlock")
+    return o, lse
