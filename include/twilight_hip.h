@@ -246,6 +246,21 @@ int twl_kv_shadow_build(const void* k_cache, int kv_dtype, uint64_t page_stride,
                         const int32_t* valid_len, uint32_t num_pages, uint32_t num_kv_heads,
                         void* k_int4, void* meta, void* stream);
 
+/* Decode append of one token per request in one launch (the per-step form of the row above;
+ * twilight/pyimpl/attention.py:138-141 appends to the HF cache and :247-251 re-quantises all of K
+ * instead). k_new / v_new are [batch, num_kv_heads, 128] with element strides (batch, head). For
+ * request b the token goes to slot s = kv_last_page_len[b] (0..15) of its LAST listed page; the
+ * caller has appended a fresh page to the table and set the length to 0 when the previous page was
+ * full. Writes the K / V rows, the token's INT4 codes and (scale, zero) pairs (a fresh page's
+ * other tokens are zeroed), folds the row into the page's min / max metadata, and stores s + 1
+ * to kv_last_page_len[b]. k_int4 / meta may be NULL. Records are identical to what
+ * twl_kv_shadow_build gives for the same page contents. */
+int twl_kv_append(const void* k_new, const void* v_new, int kv_dtype, uint64_t new_batch_stride,
+                  uint64_t new_head_stride, void* k_cache, void* v_cache, uint64_t page_stride,
+                  uint64_t token_stride, uint64_t head_stride, const int32_t* kv_page_indices,
+                  const int32_t* kv_page_indptr, int32_t* kv_last_page_len, uint32_t batch,
+                  uint32_t num_kv_heads, void* k_int4, void* meta, void* stream);
+
 /* Unpack INT4 shadow records to fp32: out [num_pages, num_kv_heads, 16, 128] (record order).
  * Exists so that tests can compare dequantised values bit for bit. */
 int twl_dequant_int4(const void* k_int4, uint32_t num_records, float* out, void* stream);

@@ -117,6 +117,28 @@ def test_decode_append_keeps_shadow_fresh(dev):
     assert torch.equal(oa, ob)
 
 
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
+def test_append_kernel_records_equal_bulk_build(dev, dt):
+    # token-by-token append (one launch per step) must leave K, V, INT4 records and Quest metadata
+    # bit-identical to paging the final tensors at once; ragged: 3 requests of different phase
+    g = torch.Generator().manual_seed(5)
+    B, Hkv, N0, steps = 3, 5, 47, 40                     # crosses two page boundaries
+    k = (torch.randn((B, Hkv, N0 + steps, 128), generator=g) * 2).to(dt)
+    v = torch.randn((B, Hkv, N0 + steps, 128), generator=g).to(dt)
+    cache = PagedKVCache.from_dense(k[:, :, :N0].contiguous(), v[:, :, :N0].contiguous(), dev,
+                                    spare_pages=12)
+    free = list(range(9, 21))
+    for s in range(steps):
+        # a strided view (the layout a projection + transpose hands over)
+        cache.append(k[:, :, N0 + s].to(dev), v[:, :, N0 + s].to(dev), free)
+    full = PagedKVCache.from_dense(k, v, dev)
+    assert torch.equal(cache.kv_last_page_len.cpu(), full.kv_last_page_len.cpu())
+    ia, ib = cache.kv_page_indices.long(), full.kv_page_indices.long()
+    assert ia.numel() == ib.numel()
+    for name in ("k_cache", "v_cache", "k_int4", "meta"):
+        assert torch.equal(getattr(cache, name)[ia], getattr(full, name)[ib]), name
+
+
 def test_full_size_cfg4_layer_sampled_rows_and_properties(dev):
     # BASELINE config 4 at its full size: B=16, 32 MHA heads, ctx 32768, fp16 paged KV (shuffled
     # pages), Quest budget 8192, p = 0.95. The oracle (dense, CPU) checks a sample of (batch, head)

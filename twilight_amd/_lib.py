@@ -27,7 +27,7 @@ EXPORTS = (
     "twl_softmax_top_p_f32", "twl_gemv_top_p", "twl_gemv_int4", "twl_gemv_int4_nhd",
     "twl_gemv_int8_nhd", "twl_gemv_f16_nhd", "twl_gemv_f16_single", "twl_sparse_attn",
     "twl_sparse_attn_workspace_bytes", "twl_quest_select",
-    "twl_quest_page_scores", "twl_quest_topk_pages", "twl_kv_shadow_build", "twl_dequant_int4",
+    "twl_quest_page_scores", "twl_quest_topk_pages", "twl_kv_shadow_build", "twl_kv_append", "twl_dequant_int4",
     "twl_decode_layer", "twl_get_label_tensor", "twl_bgemv_int8", "twl_qk_int8_lse",
 )
 
@@ -97,6 +97,8 @@ def lib() -> ctypes.CDLL:
     L.twl_decode_layer.argtypes = [POINTER(LayerArgs), vp]
     L.twl_get_label_tensor.argtypes = [vp, vp, vp, u32, u32, u32, u32] + [c_int64] * 8 + [vp]
     L.twl_bgemv_int8.argtypes = [vp, vp, vp, vp, u32, u32, u32, u32] + [c_int64] * 11 + [vp]
+    L.twl_kv_append.argtypes = [vp, vp, i32, u64, u64, vp, vp, u64, u64, u64, vp, vp, vp, u32, u32,
+                                vp, vp, vp]
     i64 = ctypes.c_int64
     L.twl_qk_int8_lse.argtypes = [vp, vp, vp, vp, vp, u32, u32, u32, u32, u32, u32, i64, i64, i64,
                                   i64, i64, i64, vp]

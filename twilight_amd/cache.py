@@ -7,7 +7,7 @@ from typing import Optional
 import torch
 
 from . import _lib
-from .kernel import kv_shadow_build
+from .kernel import kv_append, kv_shadow_build
 
 PAGE = _lib.PAGE
 HEAD_DIM = _lib.HEAD_DIM
@@ -99,12 +99,12 @@ class PagedKVCache:
         return c
 
     def append(self, k_new: torch.Tensor, v_new: torch.Tensor, free_pages: Optional[list] = None) -> None:
-        """Decode append of one token per request: ``k_new`` / ``v_new`` [B, Hkv, 128]. Writes the
-        token, extends the page table when a request's last page is full (taking ids from
-        ``free_pages``), and refreshes the shadow records of the touched pages."""
+        """Decode append of one token per request: ``k_new`` / ``v_new`` [B, Hkv, 128]. Extends the
+        page table when a request's last page is full (taking ids from ``free_pages``; host-side
+        bookkeeping only, nothing is read back from the device), then one kernel writes the token
+        and updates the shadow records and the lengths."""
         B = self.batch
         per_req, last = self._per_req, self._last
-        touched, valid, slots = [], [], []
         grew = False
         for b in range(B):
             if last[b] == PAGE:
@@ -113,17 +113,7 @@ class PagedKVCache:
                 per_req[b].append(int(free_pages.pop(0)))
                 last[b] = 0
                 grew = True
-            page = per_req[b][-1]
-            slots.append((page, last[b]))
-            last[b] += 1
-            self._seq_lens[b] += 1
-            touched.append(page)
-            valid.append(last[b])
-        pg = torch.tensor([s[0] for s in slots], device=self.device)
-        sl = torch.tensor([s[1] for s in slots], device=self.device)
-        self.k_cache[pg, sl] = k_new.to(self.device, self.dtype)
-        self.v_cache[pg, sl] = v_new.to(self.device, self.dtype)
-        if grew:  # a request took a new page: the CSR arrays change shape
+        if grew:  # a request took a new page: the CSR arrays change shape, lengths are re-sent
             flat = [p for r in per_req for p in r]
             ptr = [0]
             for r in per_req:
@@ -131,7 +121,15 @@ class PagedKVCache:
             self.kv_page_indices = torch.tensor(flat, dtype=torch.int32, device=self.device)
             self.kv_page_indptr = torch.tensor(ptr, dtype=torch.int32, device=self.device)
             self.max_pages_per_req = max(len(r) for r in per_req)
-        # same tensor object every step, so cached argument blocks of the layer stay valid
-        self.kv_last_page_len.copy_(torch.tensor(last, dtype=torch.int32))
-        self.rebuild_shadow(torch.tensor(touched, dtype=torch.int32, device=self.device),
-                            torch.tensor(valid, dtype=torch.int32, device=self.device))
+            # same tensor object every step, so cached argument blocks of the layer stay valid
+            self.kv_last_page_len.copy_(torch.tensor(last, dtype=torch.int32))
+        k_new = k_new.to(self.device, self.dtype)
+        v_new = v_new.to(self.device, self.dtype)
+        if k_new.stride(-1) != 1 or v_new.stride() != k_new.stride():
+            k_new, v_new = k_new.contiguous(), v_new.contiguous()
+        # one launch: rows, INT4 codes, min/max metadata, and the device-side lengths + 1
+        kv_append(k_new, v_new, self.k_cache, self.v_cache, self.kv_page_indices,
+                  self.kv_page_indptr, self.kv_last_page_len, self.k_int4, self.meta)
+        for b in range(B):
+            last[b] += 1
+            self._seq_lens[b] += 1

@@ -111,6 +111,109 @@ __global__ __launch_bounds__(kShThreads) void kv_shadow_kernel(ShadowArgs a) {
   }
 }
 
+// Decode append: one new token per request goes into slot kv_last_page_len[b] of the request's
+// last page (the host has made sure that page exists and, when it is a fresh page, has set the
+// length to 0), K and V rows are stored, the token's part of the INT4 record is quantised, the
+// page's min / max metadata is folded with the new row, and the length is advanced. One workgroup
+// per request; its four wavefronts share the kv heads.
+struct AppendArgs {
+  const void* k_new;
+  const void* v_new;
+  uint64_t new_batch_stride, new_head_stride;
+  void* k_cache;
+  void* v_cache;
+  uint64_t page_stride, token_stride, head_stride;
+  const int32_t* kv_page_indices;
+  const int32_t* kv_page_indptr;
+  int32_t* kv_last_page_len;
+  uint32_t num_kv_heads;
+  uint8_t* k_int4;
+  uint8_t* meta;
+};
+
+template <int DT>
+__global__ __launch_bounds__(kShThreads) void kv_append_kernel(AppendArgs a) {
+  const uint32_t b = blockIdx.x;
+  const int lane = lane_id();
+  const int wave = threadIdx.x / kWave;
+  const int pg_end = a.kv_page_indptr[b + 1];
+  const int n_pages = pg_end - a.kv_page_indptr[b];
+  const int slot = a.kv_last_page_len[b];
+  __syncthreads();  // every wave has read the length before it is advanced below
+  if (n_pages <= 0 || slot < 0 || slot >= TWL_PAGE) return;  // nothing sane to do; length untouched
+  const int page = a.kv_page_indices[pg_end - 1];
+  for (uint32_t kvh = wave; kvh < a.num_kv_heads; kvh += kShWaves) {
+    const size_t src_off = (size_t)b * a.new_batch_stride + (size_t)kvh * a.new_head_stride;
+    const size_t dst_off = (size_t)page * a.page_stride + (size_t)slot * a.token_stride +
+                           (size_t)kvh * a.head_stride;
+    // K and V rows: 2 channels per lane
+    const uint32_t kw = *((const uint32_t*)((const uint16_t*)a.k_new + src_off) + lane);
+    const uint32_t vw = *((const uint32_t*)((const uint16_t*)a.v_new + src_off) + lane);
+    *((uint32_t*)((uint16_t*)a.k_cache + dst_off) + lane) = kw;
+    *((uint32_t*)((uint16_t*)a.v_cache + dst_off) + lane) = vw;
+    if (a.k_int4) {
+      uint8_t* rec = a.k_int4 + ((size_t)page * a.num_kv_heads + kvh) * TWL_INT4_RECORD_BYTES;
+      if (slot == 0) {  // a fresh page: the other 15 tokens' parts read as "not written"
+        *(u32x4*)(rec + 16 * lane) = u32x4{0u, 0u, 0u, 0u};
+        *(uint32_t*)(rec + 1024 + 4 * lane) = 0u;
+      }
+      if (lane < 4) {  // lane g quantises group g of the new row (same arithmetic as kv_shadow_kernel)
+        float x[32];
+        const uint16_t* src = (const uint16_t*)a.k_new + src_off + 32 * lane;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          u32x4 v = *(const u32x4*)(src + 8 * i);
+          const uint32_t ws[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            x[8 * i + 2 * j] = bits16_to_f32<DT>(ws[j] & 0xFFFFu);
+            x[8 * i + 2 * j + 1] = bits16_to_f32<DT>(ws[j] >> 16);
+          }
+        }
+        float mn = x[0], mx = x[0];
+#pragma unroll
+        for (int i = 1; i < 32; ++i) {
+          mn = fminf(mn, x[i]);
+          mx = fmaxf(mx, x[i]);
+        }
+        const float range = fmaxf(mx - mn, 1e-9f);
+        float sh = round_to<TWL_F16>(range / 15.0f);
+        sh = fminf(fmaxf(sh, 6.103515625e-05f), 65504.0f);
+        float zh = round_to<TWL_F16>(mn);
+        zh = fminf(fmaxf(zh, -65504.0f), 65504.0f);
+        uint32_t w[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int i = 0; i < 32; ++i) {
+          float c = rintf((x[i] - zh) / sh);
+          c = fminf(fmaxf(c, 0.0f), 15.0f);
+          w[i >> 3] |= (uint32_t)c << (4 * (i & 7));
+        }
+        const int li = 4 * slot + lane;  // the record's (token, group) index
+        *(u32x4*)(rec + 16 * li) = u32x4{w[0], w[1], w[2], w[3]};
+        *(uint32_t*)(rec + 1024 + 4 * li) = f32_to_f16_bits(sh) | (f32_to_f16_bits(zh) << 16);
+      }
+    }
+    if (a.meta) {  // lane l folds channels 2l, 2l+1 into the page's min / max
+      uint8_t* rec = a.meta + ((size_t)page * a.num_kv_heads + kvh) * TWL_META_RECORD_BYTES;
+      const int c = lane >> 1, o = (lane & 1) * 4;
+      uint32_t* pmin = (uint32_t*)(rec + 16 * c + o);
+      uint32_t* pmax = (uint32_t*)(rec + 16 * c + 8 + o);
+      const float k0 = bits16_to_f32<DT>(kw & 0xFFFFu), k1 = bits16_to_f32<DT>(kw >> 16);
+      float mn0 = k0, mn1 = k1, mx0 = k0, mx1 = k1;
+      if (slot > 0) {
+        const uint32_t om = *pmin, ox = *pmax;
+        mn0 = fminf(mn0, bits16_to_f32<DT>(om & 0xFFFFu));
+        mn1 = fminf(mn1, bits16_to_f32<DT>(om >> 16));
+        mx0 = fmaxf(mx0, bits16_to_f32<DT>(ox & 0xFFFFu));
+        mx1 = fmaxf(mx1, bits16_to_f32<DT>(ox >> 16));
+      }
+      *pmin = f32_to_bits16<DT>(mn0) | (f32_to_bits16<DT>(mn1) << 16);
+      *pmax = f32_to_bits16<DT>(mx0) | (f32_to_bits16<DT>(mx1) << 16);
+    }
+  }
+  if (threadIdx.x == 0) a.kv_last_page_len[b] = slot + 1;
+}
+
 // one thread per (record, token, group): 32 outputs
 __global__ __launch_bounds__(256) void dequant_int4_kernel(const uint8_t* k_int4,
                                                            uint32_t num_records, float* out) {
@@ -169,5 +272,38 @@ extern "C" int twl_dequant_int4(const void* k_int4, uint32_t num_records, float*
   const uint64_t threads = (uint64_t)num_records * 64;
   hipLaunchKernelGGL(twl::dequant_int4_kernel, dim3((uint32_t)((threads + 255) / 256)), dim3(256),
                      0, (hipStream_t)stream, (const uint8_t*)k_int4, num_records, out);
+  return hipGetLastError() == hipSuccess ? TWL_OK : TWL_ELAUNCH;
+}
+
+extern "C" int twl_kv_append(const void* k_new, const void* v_new, int kv_dtype,
+                             uint64_t new_batch_stride, uint64_t new_head_stride, void* k_cache,
+                             void* v_cache, uint64_t page_stride, uint64_t token_stride,
+                             uint64_t head_stride, const int32_t* kv_page_indices,
+                             const int32_t* kv_page_indptr, int32_t* kv_last_page_len,
+                             uint32_t batch, uint32_t num_kv_heads, void* k_int4, void* meta,
+                             void* stream) {
+  if (!k_new || !v_new || !k_cache || !v_cache || !kv_page_indices || !kv_page_indptr ||
+      !kv_last_page_len)
+    return TWL_ENULL;
+  if (kv_dtype != TWL_F16 && kv_dtype != TWL_BF16) return TWL_EDTYPE;
+  if (batch == 0 || num_kv_heads == 0) return TWL_EINVAL;
+  if ((page_stride | token_stride | head_stride | new_batch_stride | new_head_stride) & 7u)
+    return TWL_EALIGN;
+  if ((((uintptr_t)k_new) & 15u) || (((uintptr_t)v_new) & 15u) || (((uintptr_t)k_cache) & 15u) ||
+      (((uintptr_t)v_cache) & 15u) || (((uintptr_t)k_int4) & 15u) || (((uintptr_t)meta) & 15u))
+    return TWL_EALIGN;
+  twl::AppendArgs a{};
+  a.k_new = k_new; a.v_new = v_new; a.new_batch_stride = new_batch_stride;
+  a.new_head_stride = new_head_stride; a.k_cache = k_cache; a.v_cache = v_cache;
+  a.page_stride = page_stride; a.token_stride = token_stride; a.head_stride = head_stride;
+  a.kv_page_indices = kv_page_indices; a.kv_page_indptr = kv_page_indptr;
+  a.kv_last_page_len = kv_last_page_len; a.num_kv_heads = num_kv_heads;
+  a.k_int4 = (uint8_t*)k_int4; a.meta = (uint8_t*)meta;
+  if (kv_dtype == TWL_F16)
+    hipLaunchKernelGGL((twl::kv_append_kernel<TWL_F16>), dim3(batch), dim3(twl::kShThreads), 0,
+                       (hipStream_t)stream, a);
+  else
+    hipLaunchKernelGGL((twl::kv_append_kernel<TWL_BF16>), dim3(batch), dim3(twl::kShThreads), 0,
+                       (hipStream_t)stream, a);
   return hipGetLastError() == hipSuccess ? TWL_OK : TWL_ELAUNCH;
 }

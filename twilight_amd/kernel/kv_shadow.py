@@ -51,6 +51,51 @@ def kv_shadow_build(k_cache: torch.Tensor, k_int4: Optional[torch.Tensor],
     _lib.check(rc, "KvShadowBuild")
 
 
+def kv_append(k_new: torch.Tensor, v_new: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+              kv_page_indices: torch.Tensor, kv_page_indptr: torch.Tensor,
+              kv_last_page_len: torch.Tensor, k_int4: Optional[torch.Tensor] = None,
+              meta: Optional[torch.Tensor] = None) -> None:
+    """Decode append of one token per request in one launch. ``k_new`` / ``v_new`` [B,Hkv,128]
+    (head_dim contiguous) go to slot ``kv_last_page_len[b]`` of each request's last listed page;
+    the token's INT4 codes and the page's min/max metadata are updated and ``kv_last_page_len`` is
+    advanced in place. The caller extends the page table (and sets the length to 0) beforehand
+    when a request's last page is full."""
+    ps, ts, hs = _cache_strides(k_cache, "k_cache")
+    if _cache_strides(v_cache, "v_cache") != (ps, ts, hs) or v_cache.dtype != k_cache.dtype:
+        raise RuntimeError("k_cache and v_cache must share dtype and strides")
+    Hkv = k_cache.size(2)
+    for name, t in (("k_new", k_new), ("v_new", v_new)):
+        if not t.is_cuda or t.dim() != 3 or t.size(1) != Hkv or t.size(2) != _lib.HEAD_DIM \
+                or t.stride(2) != 1 or t.dtype != k_cache.dtype:
+            raise RuntimeError(f"{name} must be a CUDA [B, {Hkv}, {_lib.HEAD_DIM}] tensor of "
+                               f"{k_cache.dtype} with contiguous head_dim")
+    B = k_new.size(0)
+    if v_new.size(0) != B or v_new.stride() != k_new.stride():
+        raise RuntimeError("k_new and v_new must share shape and strides")
+    for name, t in (("kv_page_indices", kv_page_indices), ("kv_page_indptr", kv_page_indptr),
+                    ("kv_last_page_len", kv_last_page_len)):
+        check_input(t, name); check_dtype(t, torch.int32, name)
+    if kv_page_indptr.numel() != B + 1 or kv_last_page_len.numel() != B:
+        raise RuntimeError("kv_page_indptr must have B+1 and kv_last_page_len B elements")
+    for name, t, nb in (("k_int4", k_int4, _lib.INT4_RECORD_BYTES), ("meta", meta, _lib.META_RECORD_BYTES)):
+        if t is not None:
+            check_input(t, name); check_dtype(t, torch.uint8, name)
+            if t.dim() != 3 or t.size(0) != k_cache.size(0) or t.size(1) != Hkv or t.size(2) != nb:
+                raise RuntimeError(f"{name} must be uint8 [pages, kv_heads, {nb}]")
+    check_same_device(k_cache, ("v_cache", v_cache), ("k_new", k_new), ("v_new", v_new),
+                      ("kv_page_indices", kv_page_indices), ("kv_page_indptr", kv_page_indptr),
+                      ("kv_last_page_len", kv_last_page_len), ("k_int4", k_int4), ("meta", meta))
+    if B == 0:
+        return
+    with torch.cuda.device(k_cache.device):
+        rc = _lib.lib().twl_kv_append(
+            ptr(k_new), ptr(v_new), dtype_code(k_cache.dtype, "k_cache"), k_new.stride(0),
+            k_new.stride(1), ptr(k_cache), ptr(v_cache), ps, ts, hs, ptr(kv_page_indices),
+            ptr(kv_page_indptr), ptr(kv_last_page_len), B, Hkv, ptr(k_int4), ptr(meta),
+            stream_of(k_cache))
+    _lib.check(rc, "KvAppend")
+
+
 def dequant_int4(k_int4: torch.Tensor) -> torch.Tensor:
     """uint8 [pages,Hkv,1280] records -> fp32 [pages,Hkv,16,128] (nibble*scale + zero)."""
     check_input(k_int4, "k_int4"); check_dtype(k_int4, torch.uint8, "k_int4")
