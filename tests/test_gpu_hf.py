@@ -82,3 +82,35 @@ def test_decode_prunes_and_reports_budgets(dev):
     got2 = _forced_decode(model, ids2, toks[:, :3])
     assert torch.isfinite(got2).all()
     assert model.model.layers[2].self_attn._twilight_state.seq_len == 103
+
+
+def test_patch_after_prefill_and_without_hf_cache_updates(dev):
+    # (a) patching a model whose prompt was prefilled before: the first decode step pages the K / V
+    # found in the model's cache; (b) keep_hf_cache=False gives the same logits (patched layers
+    # never read the model's cache at decode) while their DynamicCache layers stop growing
+    model = _tiny_llama(layers=4, heads=4, kv_heads=2, dtype=torch.float16).to(dev)
+    ids = torch.randint(0, 97, (2, 90), generator=torch.Generator().manual_seed(4)).to(dev)
+    nxt = torch.randint(0, 97, (2, 5), generator=torch.Generator().manual_seed(5)).to(dev)
+
+    def run(patch_before, keep):
+        with torch.no_grad():
+            if patch_before:
+                hf.enable_sparse_attention(model, CFG, keep_hf_cache=keep)
+            out = model(ids, use_cache=True)
+            past = out.past_key_values
+            if not patch_before:
+                hf.enable_sparse_attention(model, CFG, keep_hf_cache=keep)
+            logits = []
+            for s in range(nxt.shape[1]):
+                out = model(nxt[:, s:s + 1], past_key_values=past, use_cache=True)
+                past = out.past_key_values
+                logits.append(out.logits[:, -1].float())
+        lens = [past.get_seq_length(i) for i in range(4)]
+        hf.disable_sparse_attention(model)
+        return torch.stack(logits), lens
+
+    a, la = run(True, True)
+    b, lb = run(False, True)
+    c, lc = run(True, False)
+    assert torch.equal(a, b) and torch.equal(a, c)
+    assert la == [95, 95, 95, 95] and lb == la and lc == [95, 95, 90, 90]

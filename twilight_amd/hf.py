@@ -89,12 +89,14 @@ class HistoryBudgetInfo:
 class _LayerState:
     """What a patched attention module carries between calls."""
 
-    def __init__(self, cfg: dict, reserve_tokens: int, budget_info: Optional[HistoryBudgetInfo]):
+    def __init__(self, cfg: dict, reserve_tokens: int, budget_info: Optional[HistoryBudgetInfo],
+                 keep_hf_cache: bool):
         self.cfg, self.reserve_tokens, self.budget_info = cfg, reserve_tokens, budget_info
+        self.keep_hf_cache = keep_hf_cache
         self.cache: Optional[PagedKVCache] = None
         self.layer: Optional[TwilightDecodeLayer] = None
         self.free: List[int] = []
-        self.seq_len = 0
+        self.seq_len = 0          # tokens of the current sequence seen by this layer
 
     def reset(self) -> None:
         self.cache, self.layer, self.free, self.seq_len = None, None, [], 0
@@ -120,18 +122,24 @@ def _twilight_attention_forward(self, hidden_states, position_embeddings=None, a
     st: _LayerState = self._twilight_state
     q_len = hidden_states.shape[1]
     if q_len > 1 or past_key_values is None:
+        if past_key_values is None or past_key_values.get_seq_length(self.layer_idx) == 0:
+            st.reset()                                    # a new sequence starts
         out = self._twilight_orig_forward(hidden_states, position_embeddings=position_embeddings,
                                           attention_mask=attention_mask,
                                           past_key_values=past_key_values, **kwargs)
-        st.reset()
-        if past_key_values is not None:
-            lay = past_key_values.layers[self.layer_idx]
-            if lay.keys.is_cuda:  # the paged cache and its kernels exist on the GPU only
-                _fill_from_prefill(st, lay.keys, lay.values, self.config.num_attention_heads)
+        st.seq_len += q_len
+        st.cache = st.layer = None                        # paged lazily at the next decode step
         return out
     if st.cache is None:
-        raise RuntimeError("decode step without a paged cache: no prefill ran through this layer "
-                           "with use_cache=True on a GPU (there is no CPU path)")
+        # first decode step after a prefill (possibly a prefill that ran before patching): page
+        # the K / V the model's own cache holds for this layer
+        lay = past_key_values.layers[self.layer_idx] if len(past_key_values.layers) > self.layer_idx else None
+        keys = getattr(lay, "keys", None)
+        if keys is None or not keys.is_cuda or keys.shape[-2] == 0:
+            raise RuntimeError("decode step without prefilled K / V of this layer on a GPU (the "
+                               "path has no CPU implementation and needs use_cache=True)")
+        n = st.seq_len if st.seq_len > 0 else past_key_values.get_seq_length(self.layer_idx)
+        _fill_from_prefill(st, keys[:, :, :n], lay.values[:, :, :n], self.config.num_attention_heads)
     B = hidden_states.shape[0]
     hidden_shape = (B, 1, -1, self.head_dim)
     q = self.q_proj(hidden_states).view(hidden_shape).transpose(1, 2)
@@ -139,7 +147,8 @@ def _twilight_attention_forward(self, hidden_states, position_embeddings=None, a
     v = self.v_proj(hidden_states).view(hidden_shape).transpose(1, 2)
     cos, sin = position_embeddings
     q, k = apply_rotary_pos_emb(q, k, cos, sin)
-    past_key_values.update(k, v, self.layer_idx)      # keeps the model's own cache consistent
+    if st.keep_hf_cache:
+        past_key_values.update(k, v, self.layer_idx)  # keeps the model's own cache consistent
     st.cache.append(k[:, :, 0], v[:, :, 0], st.free)
     st.seq_len += 1
     out = st.layer(q[:, :, 0].contiguous())           # [B, H, 128]
@@ -152,11 +161,15 @@ def _twilight_attention_forward(self, hidden_states, position_embeddings=None, a
 
 def enable_sparse_attention(model, sparse_config: Dict, enable_budget_info: bool = False,
                             enable_score_info: bool = False, reserve_tokens: int = 4096,
-                            high: str = "max") -> Tuple[Optional[HistoryBudgetInfo], None]:
+                            high: str = "max", keep_hf_cache: bool = True
+                            ) -> Tuple[Optional[HistoryBudgetInfo], None]:
     """Patch every Llama / Mistral attention module of ``model`` (twilight/pyimpl/attention.py:
     351-418, 481-493). ``sparse_config`` is the reference's JSON template
     (benchmark/configs/config_quest_twi.json). ``reserve_tokens``: decode tokens per request the
-    paged caches are sized for. Returns ``(budget_info, None)``; the accumulated-score statistic
+    paged caches are sized for. ``keep_hf_cache=False`` stops patched layers from also appending
+    decode tokens to the model's own cache (a whole-context copy per step with ``DynamicCache``);
+    it needs ``skip_first_two_layers`` (layer 0 keeps the sequence length the model asks its cache
+    for) and a sequence that is only prefilled once. Returns ``(budget_info, None)``; the accumulated-score statistic
     of the reference needs the dense attention weights, which this path never forms."""
     if enable_score_info:
         raise RuntimeError("enable_score_info needs dense attention weights; not available here")
@@ -169,6 +182,8 @@ def enable_sparse_attention(model, sparse_config: Dict, enable_budget_info: bool
     cfg = parse_sparse_config(sparse_config)
     cfg["high"] = high
     skip = 2 if sparse_config.get("skip_first_two_layers", True) else 0
+    if not keep_hf_cache and skip == 0:
+        raise RuntimeError("keep_hf_cache=False needs skip_first_two_layers")
     budget_info = HistoryBudgetInfo() if enable_budget_info else None
     patched = 0
     for name, module in model.named_modules():
@@ -180,7 +195,7 @@ def enable_sparse_attention(model, sparse_config: Dict, enable_budget_info: bool
             raise RuntimeError("enable_sparse_attention was already called on this model")
         if module.layer_idx < skip:
             continue
-        module._twilight_state = _LayerState(dict(cfg), reserve_tokens, budget_info)
+        module._twilight_state = _LayerState(dict(cfg), reserve_tokens, budget_info, keep_hf_cache)
         module._twilight_orig_forward = module.forward
         module.forward = types.MethodType(_twilight_attention_forward, module)
         patched += 1
