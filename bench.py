@@ -89,6 +89,49 @@ def cpu_baseline(N: int, H: int, budget: int, top_p: float, batch_scale: int, de
     }
 
 
+def bench_topp(args, L, dev) -> int:
+    """The pruner alone: fp32 scores [8, 32, 8192], N(0,1) background + a Zipf(1.2) spike set of
+    1..512 tokens per row at random positions; softmax + top-p + compaction in one launch
+    (twl_softmax_top_p_f32), p in {0.85, 0.95}. Four score tensors are visited round-robin."""
+    from twilight_amd import synth
+    B, H, M = 8, 32, 8192
+    rows = B * H
+    xs = [synth.topp_scores(B, H, M, seed=100 * i, max_spikes=512).to(dev) for i in range(4)]
+    idx = torch.empty((B, H, M), dtype=torch.int32, device=dev)
+    cnt = torch.empty((B, H), dtype=torch.int32, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    res = {}
+    for p in (0.85, 0.95):
+        state = {"i": 0}
+
+        def call():
+            x = xs[state["i"] % 4]
+            state["i"] += 1
+            L.twl_softmax_top_p_f32(x.data_ptr(), M, 0, rows, M, 0, p, 1, 0, 0, idx.data_ptr(), M,
+                                    cnt.data_ptr(), 0, 0, stream)
+        us = _time_calls(call, args.steps, args.warmup)
+        surv = []
+        for x in xs:
+            L.twl_softmax_top_p_f32(x.data_ptr(), M, 0, rows, M, 0, p, 1, 0, 0, idx.data_ptr(), M,
+                                    cnt.data_ptr(), 0, 0, stream)
+            torch.cuda.synchronize()
+            surv.append(cnt.float().cpu())
+        sv = torch.cat([t.flatten() for t in surv])
+        nbytes = rows * M * 4 + int(sv.mean() * rows) * 4 + rows * 4
+        res[str(p)] = {"us": round(us, 2), "survivors_median": float(sv.median()),
+                       "survivors_mean": round(float(sv.mean()), 1), "survivors_max": int(sv.max()),
+                       "bytes": nbytes, "GBps": round(nbytes / us / 1e3, 1)}
+    line = {"metric": "us/top-p call (softmax + top-p + compaction)", "value": res["0.95"]["us"],
+            "unit": "us", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": round(res["0.95"]["us"] / 1e3, 5), "higher_is_better": False,
+            "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+            "config": {"workload": "top-p pruner alone, fp32 scores [8, 32, 8192], Zipf(1.2) spike "
+                                   "sets of 1-512 tokens per row, high = row max"},
+            "per_p": res}
+    print(json.dumps(line))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -98,10 +141,10 @@ def main() -> int:
     ap.add_argument("--context", type=int, default=32768)
     ap.add_argument("--budget", type=int, default=8192)
     ap.add_argument("--top-p", type=float, default=0.95)
-    ap.add_argument("--workload", choices=["longchat", "llama3"], default="longchat",
+    ap.add_argument("--workload", choices=["longchat", "llama3", "topp"], default="longchat",
                     help="longchat: 32 MHA heads fp16 (the headline workload); llama3: GQA 32/8 "
                          "bf16, with a dense-decode baseline (the same attention kernel over "
-                         "every token)")
+                         "every token); topp: the pruner kernel alone on [8,32,8192] scores")
     ap.add_argument("--layers", type=int, default=4,
                     help="independent layer caches visited round-robin (cold-cache steps)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -128,6 +171,8 @@ def main() -> int:
     L = _lib.lib()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.workload == "topp":
+        return bench_topp(args, L, dev)
     llama = args.workload == "llama3"
     B, H, Hkv, N, D = args.batch, 32, (8 if llama else 32), args.context, 128
     npg = N // 16
