@@ -35,19 +35,11 @@ struct GemvArgs {
   float sm_scale;
 };
 
-#ifndef TWL_GEMV_THREADS
-#define TWL_GEMV_THREADS 256
-#endif
-#ifndef TWL_GEMV_PAGES_PER_WAVE
-#define TWL_GEMV_PAGES_PER_WAVE 16
-#endif
-#ifndef TWL_GEMV_UNROLL
-#define TWL_GEMV_UNROLL 4
-#endif
-constexpr int kGemvThreads = TWL_GEMV_THREADS;    // 4 wavefronts
-constexpr int kGemvPagesPerWave = TWL_GEMV_PAGES_PER_WAVE;  // <= 64: one lane per page id
+// launch shape, chosen by a sweep over (threads, pages per wave, unroll) at 8 x 32 x 32768
+constexpr int kGemvThreads = 256;       // 4 wavefronts
+constexpr int kGemvPagesPerWave = 16;   // <= 64: one lane per page id
 constexpr int kGemvPagesPerBlock = kGemvPagesPerWave * (kGemvThreads / kWave);
-constexpr int kGemvUnroll = TWL_GEMV_UNROLL;      // pages in flight per wavefront
+constexpr int kGemvUnroll = 4;          // pages in flight per wavefront
 
 // 8 nibbles of one dword against 8 q values held as 4 half2 pairs (n0,n4),(n1,n5),(n2,n6),(n3,n7).
 // A nibble moved to mantissa bits 4..7 of an fp16 with exponent 0 is exactly 1 + n/64, so one
@@ -71,14 +63,10 @@ __device__ __forceinline__ float dot8_nibbles(uint32_t w, const half2_t* qp, flo
 __device__ __forceinline__ float page_partial(const u32x4& nib, uint32_t sz, const half2_t* qp,
                                               float qsum) {
   float acc = 0.0f;
-#ifdef TWL_GEMV_NOCOMPUTE
-  acc = as_f32((nib.x ^ nib.y ^ nib.z ^ nib.w) & 0x3F800000u);
-#else
   acc = dot8_nibbles(nib.x, qp + 0, acc);
   acc = dot8_nibbles(nib.y, qp + 4, acc);
   acc = dot8_nibbles(nib.z, qp + 8, acc);
   acc = dot8_nibbles(nib.w, qp + 12, acc);
-#endif
   // sum q*nibble = 64 * (acc - sum q);  partial = scale * sum q*nibble + zero * sum q
   const float scale64 = f16_bits_to_f32(sz & 0xFFFFu) * 64.0f;
   const float zero = f16_bits_to_f32(sz >> 16);
@@ -162,43 +150,33 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_int4_kernel(GemvArgs a) {
   float* orow = a.out + (size_t)row * a.out_stride + (size_t)p0 * TWL_PAGE;
   const float ninf = -__builtin_inff();
 
-  // ---- stream: group k+1 is requested before group k is consumed -----------------------------
-  u32x4 nib[2][U];
-  uint32_t sz[2][U];
-  auto issue = [&](int grp, int buf) {
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int i = grp * U + u;
-      // entries past the run reuse entry 0: a valid address, result discarded
-      const int phys = __builtin_amdgcn_readlane(my_phys, (i < np) ? i : 0);
-      const uint8_t* rec = base + (size_t)phys * rec_stride;
-      // read-once stream: keep it out of the way of the data the other kernels reuse
-      nib[buf][u] = __builtin_nontemporal_load((const u32x4*)rec);
-      sz[buf][u] = __builtin_nontemporal_load((const uint32_t*)(rec + 1024 - 12 * lane));
-    }
-  };
-#ifndef TWL_GEMV_DBUF
-#define TWL_GEMV_DBUF 0
-#endif
+  // ---- stream: the four pages of a group are requested together, then consumed. (Requesting
+  // group k+1 before consuming group k was measured and does not help: enough wavefronts are
+  // resident to cover the latency.)
+  u32x4 nib[U];
+  uint32_t sz[U];
   static_assert(U == 4, "the output transpose below moves 4 pages x 16 tokens per store");
   // lane l stores element l of the group's 64 scores (page l/16, token l%16); it takes that value
   // from the lane that owns token l%16 and whose group index equals the page: lane 4*(l%16)+l/16
   const int src_lane4 = 4 * (4 * (lane & 15) + (lane >> 4));
-  if (TWL_GEMV_DBUF) issue(0, 0);
 #pragma unroll
   for (int grp = 0; grp < G; ++grp) {
-    const int buf = TWL_GEMV_DBUF ? (grp & 1) : 0;
-    if (TWL_GEMV_DBUF) {
-      if (grp + 1 < G && (grp + 1) * U < np) issue(grp + 1, buf ^ 1);
-    } else if (grp * U < np) {
-      issue(grp, 0);
-    }
     if (grp * U < np) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int i = grp * U + u;
+        // entries past the run reuse entry 0: a valid address, result discarded
+        const int phys = __builtin_amdgcn_readlane(my_phys, (i < np) ? i : 0);
+        const uint8_t* rec = base + (size_t)phys * rec_stride;
+        // read-once stream: keep it out of the way of the data the other kernels reuse
+        nib[u] = __builtin_nontemporal_load((const u32x4*)rec);
+        sz[u] = __builtin_nontemporal_load((const uint32_t*)(rec + 1024 - 12 * lane));
+      }
       float mine = 0.0f;  // the score this lane hands over: page g of the group, token t
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const int i = grp * U + u;
-        const float part = page_partial(nib[buf][u], sz[buf][u], qp, qsum);
+        const float part = page_partial(nib[u], sz[u], qp, qsum);
         const int logical = __builtin_amdgcn_readlane(my_logical, (i < np) ? i : 0);
         const int valid = (logical == req_pages - 1) ? last_len : TWL_PAGE;
         const float val = (t < valid) ? part * a.sm_scale : ninf;
@@ -206,16 +184,7 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_int4_kernel(GemvArgs a) {
       }
       const float sc = as_f32(__builtin_amdgcn_ds_bpermute(src_lane4, as_i32(mine)));
       // one 256-byte store per group; pages past the run are masked off
-#ifdef TWL_GEMV_NOSTORE
-      if (grp * U + (lane >> 4) < np && sc == 12345.0f)
-#else
-      if (grp * U + (lane >> 4) < np)
-#endif
-#ifdef TWL_GEMV_NTSTORE
-        __builtin_nontemporal_store(sc, orow + grp * U * TWL_PAGE + lane);
-#else
-        orow[grp * U * TWL_PAGE + lane] = sc;
-#endif
+      if (grp * U + (lane >> 4) < np) orow[grp * U * TWL_PAGE + lane] = sc;
     }
   }
 }
