@@ -37,6 +37,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 # kept under profiles/). bench.py cannot read counters itself, so the figure is reported only for
 # the exact configuration it was measured on.
 QUEST_SCORE_TRAFFIC_BYTES_DEFAULT = int((131404.9 * 2.000 + 2048.0 * 1.000) * 1024)
+# The same for select_estimate_prune_kernel (FETCH_SIZE KiB x 2.000 + WRITE_SIZE KiB x 1.000).
+ROW_KERNEL_TRAFFIC_BYTES_DEFAULT = int((213640.2 * 2.000 + 596.1 * 1.000) * 1024)
 
 
 def _time_calls(fn, iters: int, warmup: int) -> float:
@@ -253,6 +255,13 @@ def main() -> int:
                 p(l.sel_count), kp, p(c.kv_page_indices), p(c.kv_page_indptr),
                 p(c.kv_last_page_len), B, H, Hkv, kp, sm, stream)),
                 rows * M * (64 + 16 + 4) + rows * D * 2 + rows * kp * 8),
+            "select_estimate_prune": (rotating(lambda l, c, q: lambda: L.twl_select_estimate_prune(
+                p(q), qcode, p(c.meta), p(c.k_int4), p(c.kv_page_indices), p(c.kv_page_indptr),
+                p(c.kv_last_page_len), B, H, Hkv, args.budget, npg, sm, 0, args.top_p, 1,
+                p(l.sel_pages), kp, p(l.sel_count), p(l.idx), M, p(l.count), 0, 0, 0, M,
+                p(l.cand_count), stream)),
+                rows * npg * 512 + rows * M * (64 + 16) + rows * D * 2 + rows * npg * 4
+                + rows * kp * 8 + int(rows * n_bar) * 4 + rows * 12),
             "gemv_top_p": (rotating(lambda l, c, q: lambda: L.twl_gemv_top_p(
                 p(q), qcode, p(c.k_int4), p(l.sel_pages), p(l.sel_count), kp,
                 p(c.kv_page_indices), p(c.kv_page_indptr), p(c.kv_last_page_len), B, H, Hkv, kp,
@@ -275,20 +284,36 @@ def main() -> int:
                              "GBps": round(nbytes / us / 1e3, 1),
                              "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
 
-    # the kernels one layer step launches: the fused estimator + pruner unless --split-estimator
-    used = (("quest_score", "quest_topk", "gemv_int4", "softmax_top_p", "sparse_attn")
-            if args.split_estimator else ("quest_score", "quest_topk", "gemv_top_p", "sparse_attn"))
+    # the kernels one layer step launches (the choice twl_decode_layer makes)
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    row_kernel = (not args.split_estimator and H == Hkv and npg <= 8192
+                  and 2 * rows >= cus and rows <= 2 * cus)
+    if args.split_estimator:
+        used = ("quest_score", "quest_topk", "gemv_int4", "softmax_top_p", "sparse_attn")
+    elif row_kernel:
+        used = ("select_estimate_prune", "sparse_attn")
+    else:
+        used = ("quest_score", "quest_topk", "gemv_top_p", "sparse_attn")
     for name in kernels:
         kernels[name]["in_layer_step"] = name in used
     layer_bytes = sum(kernels[n]["bytes"] for n in used) if kernels else None
-    dom = kernels.get("quest_score")
+    # dominant kernel of the step: the one-launch selector + estimator + pruner when the step
+    # uses it, else the metadata stream
+    dom_name = "select_estimate_prune" if (kernels and "select_estimate_prune" in used) else "quest_score"
+    dom = kernels.get(dom_name)
     roofline = None
     if dom:
-        roofline = {"bound": "hbm", "kernel": "quest_score_kernel", "achieved": dom["GBps"],
-                    "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": dom["frac_of_hbm_peak"],
-                    "bytes_per_launch": dom["bytes"], "us_per_launch": dom["us"],
-                    "traffic": (QUEST_SCORE_TRAFFIC_BYTES_DEFAULT
-                                if (B, N, args.budget, llama) == (8, 32768, 8192, False) else None)}
+        default_cfg = (B, N, args.budget, llama) == (8, 32768, 8192, False)
+        traffic = None
+        if default_cfg:
+            traffic = (ROW_KERNEL_TRAFFIC_BYTES_DEFAULT if dom_name == "select_estimate_prune"
+                       else QUEST_SCORE_TRAFFIC_BYTES_DEFAULT)
+        roofline = {"bound": "hbm",
+                    "kernel": ("select_estimate_prune_kernel" if dom_name == "select_estimate_prune"
+                               else "quest_score_kernel"),
+                    "achieved": dom["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                    "frac": dom["frac_of_hbm_peak"], "bytes_per_launch": dom["bytes"],
+                    "us_per_launch": dom["us"], "traffic": traffic}
 
     # ---- stand-alone INT4 GEMV at 8 x 32 x 32768 candidates (all pages of every request) ----
     gemv_cfg2 = None

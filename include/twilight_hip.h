@@ -134,6 +134,28 @@ int twl_gemv_top_p(const void* q, int q_dtype, const void* k_int4, const int32_t
                    int32_t* cand_count, float* low_out, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
+ * Selector + estimator + pruner in one launch, one workgroup per (batch, head) row:
+ * twl_quest_page_scores, twl_quest_topk_pages and twl_gemv_top_p with the page scores and the
+ * page list kept on chip. Replaces: twilight/pyimpl/quest.py:17-122 + attention.py:252-255 +
+ * top_p.py:10-15 + attention.py:280-281. Outputs as those three calls give them: sel_pages /
+ * sel_count (ascending logical pages, ties at the k-th score to the lower page), idx / count,
+ * optionally page_scores_out [rows, page_score_stride], scores_out [rows, score_stride] and
+ * cand_count. max_pages_per_req <= 8192. Meant for about one row per compute unit (MHA decode at
+ * moderate batch); with GQA the three-call form reads each metadata record once per kv head and
+ * this one once per q head.
+ * ------------------------------------------------------------------------------------------- */
+int twl_select_estimate_prune(const void* q, int dtype, const void* meta, const void* k_int4,
+                              const int32_t* kv_page_indices, const int32_t* kv_page_indptr,
+                              const int32_t* kv_last_page_len, uint32_t batch,
+                              uint32_t num_q_heads, uint32_t num_kv_heads, uint32_t token_budget,
+                              uint32_t max_pages_per_req, float sm_scale, const float* p_arr,
+                              float p, int high_mode, int32_t* sel_pages, uint32_t sel_stride,
+                              int32_t* sel_count, int32_t* idx, uint32_t idx_stride,
+                              int32_t* count, float* page_scores_out, uint32_t page_score_stride,
+                              float* scores_out, uint32_t score_stride, int32_t* cand_count,
+                              void* stream);
+
+/* ---------------------------------------------------------------------------------------------
  * INT4-K score GEMV over candidate pages: out[r, c] = sm_scale * sum_d q[r,d] * dequant(K[c,d]).
  * Replaces: the estimator matmul twilight/pyimpl/attention.py:252-255 and the absent
  * ftka.cuda_ops.gemv.batched_sparse_gemv_int4_k whose call site is
@@ -336,8 +358,11 @@ typedef struct twl_layer_args {
   void* attn_workspace; uint64_t attn_workspace_bytes; /* see twl_sparse_attn */
   /* output */
   void* out;                /* [batch, num_q_heads, 128], dtype */
-  /* estimator + pruner: 0 = one fused launch (twl_gemv_top_p), 1 = twl_gemv_int4 then
-   * twl_softmax_top_p_f32. In fused mode `scores` is filled only when keep_scores != 0. */
+  /* 0 = fused: with one q head per kv head, at most one row per compute unit pair and
+   * <= 8192 pages per request the selector, estimator and pruner are ONE launch
+   * (twl_select_estimate_prune), otherwise twl_quest_select + twl_gemv_top_p; 1 = every stage its
+   * own launch (twl_quest_select, twl_gemv_int4, twl_softmax_top_p_f32). In fused mode `scores`
+   * and `page_scores` are filled only when keep_scores != 0. */
   int split_estimator;
   int keep_scores;
 } twl_layer_args;

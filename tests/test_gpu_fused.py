@@ -153,3 +153,51 @@ def test_errors(dev):
         K.sparse_gemv_int4_top_p(q, rec, ids, indptr, last, sel, cnt, 0.9, max_pages=4096)
     with pytest.raises(RuntimeError):
         K.sparse_gemv_int4_top_p(q[:, :3], rec, ids, indptr, last, sel, cnt, 0.9)
+
+
+@pytest.mark.parametrize("N,lens,budget,H,Hkv,dt", [
+    (1600, None, 320, 4, 4, torch.float16),          # 100 pages, keep 20
+    (1000, None, 100, 4, 2, torch.bfloat16),         # GQA, bf16, budget not a multiple of 16, partial page
+    (11200, None, 16384, 2, 2, torch.float16),       # budget beyond the context: every page (700)
+    (40000, None, 4096, 2, 1, torch.float16),        # 2500 pages per request (> 2048)
+    (8192 + 40, None, 8192, 2, 2, torch.float16),    # 512 selected pages: the benchmark's list length
+])
+def test_one_launch_row_kernel_equals_three_launches(dev, N, lens, budget, H, Hkv, dt):
+    """twl_select_estimate_prune against twl_quest_select + twl_gemv_top_p on a real paged cache:
+    page scores and page lists bit for bit, candidate scores bit for bit, survivor lists equal
+    (a row whose bisection meets |S - p| within rounding may differ: other reduction shape)."""
+    from twilight_amd.cache import PagedKVCache
+    B, p = 2, 0.9
+    g = torch.Generator().manual_seed(N)
+    q = torch.randn((B, H, 128), generator=g)
+    k = torch.randn((B, Hkv, N, 128), generator=g)
+    group = H // Hkv
+    for b in range(B):                               # a few heavy hitters per head
+        for h in range(H):
+            pos = torch.randint(0, N, (6,), generator=g)
+            k[b, h // group, pos] += q[b, h] * (0.3 + torch.rand(6, 1, generator=g))
+    npg = (N + 15) // 16
+    cache = PagedKVCache.from_dense(k.to(dt), k.to(dt), dev,
+                                    page_perm=torch.randperm(B * npg, generator=g))
+    qd = q.to(dt).to(dev)
+    tab = (cache.kv_page_indices, cache.kv_page_indptr, cache.kv_last_page_len)
+    selA, selcA, psA = K.quest_select(qd, cache.meta, tab[0], tab[1], budget, npg)
+    kk = selA.shape[-1]
+    idxA, cntA, candA, scA = K.sparse_gemv_int4_top_p(qd, cache.k_int4, *tab, selA, selcA, p,
+                                                     max_pages=kk, return_scores=True)
+    selB, selcB, idxB, cntB, candB, psB, scB = K.quest_gemv_int4_top_p(
+        qd, cache.meta, cache.k_int4, *tab, budget, npg, p, return_scores=True)
+    assert torch.equal(psA.view(torch.int32), psB.view(torch.int32))
+    assert torch.equal(selcA, selcB) and torch.equal(selA, selB) and torch.equal(candA, candB)
+    assert int(selcA.min()) == min(kk, npg)
+    n = int(selcA[0, 0]) * 16
+    assert torch.equal(scA[..., :n].view(torch.int32), scB[..., :n].view(torch.int32))
+    cA, cB, iA, iB = cntA.cpu(), cntB.cpu(), idxA.cpu(), idxB.cpu()
+    differ = 0
+    for b in range(B):
+        for h in range(H):
+            same = int(cA[b, h]) == int(cB[b, h]) and torch.equal(iA[b, h, :cA[b, h]], iB[b, h, :cB[b, h]])
+            differ += 0 if same else 1
+            toks = iB[b, h, :cB[b, h]].long()
+            assert torch.all(toks[1:] > toks[:-1]) and int(toks.max()) < N
+    assert differ <= 1

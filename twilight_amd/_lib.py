@@ -24,7 +24,7 @@ MAX_CANDIDATES = 32768
 # every symbol include/twilight_hip.h declares
 EXPORTS = (
     "twl_strerror", "twl_abi_version", "twl_device_count", "twl_top_p_f32", "twl_top_p_f16",
-    "twl_softmax_top_p_f32", "twl_gemv_top_p", "twl_gemv_int4", "twl_gemv_int4_nhd",
+    "twl_softmax_top_p_f32", "twl_gemv_top_p", "twl_select_estimate_prune", "twl_gemv_int4", "twl_gemv_int4_nhd",
     "twl_gemv_int8_nhd", "twl_gemv_f16_nhd", "twl_gemv_f16_single", "twl_sparse_attn",
     "twl_sparse_attn_workspace_bytes", "twl_quest_select",
     "twl_quest_page_scores", "twl_quest_topk_pages", "twl_kv_shadow_build", "twl_kv_append", "twl_dequant_int4",
@@ -79,6 +79,9 @@ def lib() -> ctypes.CDLL:
                                         vp, vp, vp]
     L.twl_gemv_top_p.argtypes = [vp, i32, vp, vp, vp, u32, vp, vp, vp, u32, u32, u32, u32, f32, vp,
                                  f32, i32, vp, u32, vp, vp, u32, vp, vp, vp]
+    L.twl_select_estimate_prune.argtypes = [vp, i32, vp, vp, vp, vp, vp, u32, u32, u32, u32, u32,
+                                            f32, vp, f32, i32, vp, u32, vp, vp, u32, vp, vp, u32,
+                                            vp, u32, vp, vp]
     L.twl_gemv_int4.argtypes = [vp, i32, vp, u32, vp, vp, vp, vp, u32, vp, vp, vp, u32, u32, u32,
                                 u32, f32, vp]
     L.twl_gemv_int4_nhd.argtypes = [vp, vp, u32, vp, vp, vp, vp, vp, vp, u32, u32, u32, u32, f32, vp]

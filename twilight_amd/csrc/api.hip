@@ -1,5 +1,5 @@
 // Library-level entry points: status strings, version, and the whole decode layer as one call
-// that enqueues the five kernels of the path back to back on the caller's stream.
+// that enqueues the kernels of the path back to back on the caller's stream.
 #include <hip/hip_runtime.h>
 
 #include "../../include/twilight_hip.h"
@@ -28,6 +28,32 @@ extern "C" int twl_device_count(void) {
   return n;
 }
 
+// compute units of the current device, looked up once per device (the only process-wide state of
+// the library; written with relaxed atomics, any racing writers store the same value)
+static int device_cu_count(int* out) {
+  static int cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) {
+    (void)hipGetLastError();
+    return TWL_ENODEVICE;
+  }
+  if (dev >= 0 && dev < 64) {
+    const int c = __atomic_load_n(&cached[dev], __ATOMIC_RELAXED);
+    if (c > 0) {
+      *out = c;
+      return TWL_OK;
+    }
+  }
+  int n = 0;
+  if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+    (void)hipGetLastError();
+    return TWL_ENODEVICE;
+  }
+  if (dev >= 0 && dev < 64) __atomic_store_n(&cached[dev], n, __ATOMIC_RELAXED);
+  *out = n;
+  return TWL_OK;
+}
+
 // twilight/pyimpl/attention.py:188-306 for q_len == 1: selector -> estimator -> pruner -> attention.
 extern "C" int twl_decode_layer(const twl_layer_args* a, void* stream) {
   if (!a) return TWL_ENULL;
@@ -45,35 +71,54 @@ extern "C" int twl_decode_layer(const twl_layer_args* a, void* stream) {
   const uint32_t ps_stride = a->page_scores ? a->page_score_stride : a->score_stride;
   if (ps_stride < a->max_pages_per_req) return TWL_EINVAL;
   if (k * TWL_PAGE > TWL_MAX_CANDIDATES) return TWL_EINVAL;
-  (void)rows;
 
-  // 1. Quest page scores + top-k pages
-  int rc = twl_quest_select(a->q, a->dtype, a->meta, a->kv_page_indices, a->kv_page_indptr,
-                            a->batch, a->num_q_heads, a->num_kv_heads, a->token_budget,
-                            a->max_pages_per_req, a->sel_pages, a->sel_stride, a->sel_count,
-                            page_scores, ps_stride, stream);
-  if (rc != TWL_OK) return rc;
-  if (!a->split_estimator) {
-    // 2+3. INT4 estimate, softmax, top-p and compaction in one launch
-    rc = twl_gemv_top_p(a->q, a->dtype, a->k_int4, a->sel_pages, a->sel_count, a->sel_stride,
-                        a->kv_page_indices, a->kv_page_indptr, a->kv_last_page_len, a->batch,
-                        a->num_q_heads, a->num_kv_heads, k, a->sm_scale, nullptr, a->top_p,
-                        a->high_mode, a->idx, a->idx_stride, a->count,
-                        a->keep_scores ? a->scores : nullptr, a->score_stride, a->cand_count,
-                        nullptr, stream);
+  int rc;
+  // one workgroup per row from the metadata to the survivor list pays off while there are about
+  // as many rows as compute units (measured: ahead from half a row to two rows per unit) and q
+  // heads do not share kv heads
+  int cus = 0;
+  const bool row_kernel = !a->split_estimator && a->num_q_heads == a->num_kv_heads &&
+                          a->max_pages_per_req <= 8192 && device_cu_count(&cus) == TWL_OK &&
+                          2u * rows >= (uint32_t)cus && rows <= 2u * (uint32_t)cus;
+  if (row_kernel) {
+    // 1+2+3. page scores, top-k pages, INT4 estimate, softmax, top-p, compaction: one launch
+    rc = twl_select_estimate_prune(
+        a->q, a->dtype, a->meta, a->k_int4, a->kv_page_indices, a->kv_page_indptr,
+        a->kv_last_page_len, a->batch, a->num_q_heads, a->num_kv_heads, a->token_budget,
+        a->max_pages_per_req, a->sm_scale, nullptr, a->top_p, a->high_mode, a->sel_pages,
+        a->sel_stride, a->sel_count, a->idx, a->idx_stride, a->count,
+        a->keep_scores ? a->page_scores : nullptr, a->page_score_stride,
+        a->keep_scores ? a->scores : nullptr, a->score_stride, a->cand_count, stream);
     if (rc != TWL_OK) return rc;
   } else {
-    // 2. INT4 estimate over the selected pages
-    rc = twl_gemv_int4(a->q, a->dtype, a->scores, a->score_stride, a->cand_count, a->k_int4,
-                       a->sel_pages, a->sel_count, a->sel_stride, a->kv_page_indices,
-                       a->kv_page_indptr, a->kv_last_page_len, a->batch, a->num_q_heads,
-                       a->num_kv_heads, k, a->sm_scale, stream);
+    // 1. Quest page scores + top-k pages
+    rc = twl_quest_select(a->q, a->dtype, a->meta, a->kv_page_indices, a->kv_page_indptr,
+                          a->batch, a->num_q_heads, a->num_kv_heads, a->token_budget,
+                          a->max_pages_per_req, a->sel_pages, a->sel_stride, a->sel_count,
+                          page_scores, ps_stride, stream);
     if (rc != TWL_OK) return rc;
-    // 3. softmax + top-p + compaction to token positions
-    rc = twl_softmax_top_p_f32(a->scores, a->score_stride, a->cand_count, rows, k * TWL_PAGE,
-                               nullptr, a->top_p, a->high_mode, a->sel_pages, a->sel_stride,
-                               a->idx, a->idx_stride, a->count, nullptr, nullptr, stream);
-    if (rc != TWL_OK) return rc;
+    if (!a->split_estimator) {
+      // 2+3. INT4 estimate, softmax, top-p and compaction in one launch
+      rc = twl_gemv_top_p(a->q, a->dtype, a->k_int4, a->sel_pages, a->sel_count, a->sel_stride,
+                          a->kv_page_indices, a->kv_page_indptr, a->kv_last_page_len, a->batch,
+                          a->num_q_heads, a->num_kv_heads, k, a->sm_scale, nullptr, a->top_p,
+                          a->high_mode, a->idx, a->idx_stride, a->count,
+                          a->keep_scores ? a->scores : nullptr, a->score_stride, a->cand_count,
+                          nullptr, stream);
+      if (rc != TWL_OK) return rc;
+    } else {
+      // 2. INT4 estimate over the selected pages
+      rc = twl_gemv_int4(a->q, a->dtype, a->scores, a->score_stride, a->cand_count, a->k_int4,
+                         a->sel_pages, a->sel_count, a->sel_stride, a->kv_page_indices,
+                         a->kv_page_indptr, a->kv_last_page_len, a->batch, a->num_q_heads,
+                         a->num_kv_heads, k, a->sm_scale, stream);
+      if (rc != TWL_OK) return rc;
+      // 3. softmax + top-p + compaction to token positions
+      rc = twl_softmax_top_p_f32(a->scores, a->score_stride, a->cand_count, rows, k * TWL_PAGE,
+                                 nullptr, a->top_p, a->high_mode, a->sel_pages, a->sel_stride,
+                                 a->idx, a->idx_stride, a->count, nullptr, nullptr, stream);
+      if (rc != TWL_OK) return rc;
+    }
   }
   // 4. exact attention over the survivors
   return twl_sparse_attn(a->q, a->out, a->dtype, a->k_cache, a->v_cache, a->page_stride,

@@ -9,7 +9,8 @@ reference benchmarks (benchmark/efficiency/bench_gemv.py:445-454).
 from .sampling import (top_p_fp16_return_mask, top_p_fp32_return_mask, top_p_select,
                        softmax_top_p)
 from .gemv import (batched_sparse_gemv, batched_sparse_gemv_int4_k, batched_sparse_gemv_int8_k,
-                   single_sparse_gemv, sparse_gemv_int4, sparse_gemv_int4_top_p)
+                   single_sparse_gemv, sparse_gemv_int4, sparse_gemv_int4_top_p,
+                   quest_gemv_int4_top_p)
 from .attention import attention_workspace_bytes, sparse_paged_decode_attention
 from .quest import quest_num_pages, quest_select
 from .kv_shadow import dequant_int4, kv_append, kv_shadow_build
@@ -18,7 +19,7 @@ from .label_ops import bgemv_int8, get_label_tensor, qk_int8_per_block
 __all__ = [
     "top_p_fp16_return_mask", "top_p_fp32_return_mask", "top_p_select", "softmax_top_p",
     "batched_sparse_gemv", "batched_sparse_gemv_int4_k", "batched_sparse_gemv_int8_k",
-    "single_sparse_gemv", "sparse_gemv_int4", "sparse_gemv_int4_top_p",
+    "single_sparse_gemv", "sparse_gemv_int4", "sparse_gemv_int4_top_p", "quest_gemv_int4_top_p",
     "sparse_paged_decode_attention",
     "attention_workspace_bytes",
     "quest_num_pages", "quest_select", "dequant_int4", "kv_shadow_build", "kv_append",

@@ -159,6 +159,80 @@ def sparse_gemv_int4_top_p(q: torch.Tensor, k_int4: torch.Tensor, kv_page_indice
     return tuple(out)
 
 
+def quest_gemv_int4_top_p(q: torch.Tensor, meta: torch.Tensor, k_int4: torch.Tensor,
+                          kv_page_indices: torch.Tensor, kv_page_indptr: torch.Tensor,
+                          kv_last_page_len: torch.Tensor, token_budget: int,
+                          max_pages_per_req: int, top_p, high: str = "max",
+                          sm_scale: Optional[float] = None, return_scores: bool = False):
+    """Selector + estimator + pruner in one launch, one workgroup per (batch, head) row:
+    :func:`twilight_amd.kernel.quest_select` followed by :func:`sparse_gemv_int4_top_p`
+    (twilight/pyimpl/quest.py:17-122, attention.py:252-255, top_p.py:10-15, attention.py:280-281)
+    with the page scores and the page list kept on chip.
+
+    Returns ``(sel_pages int32 [B,H,k], sel_count int32 [B,H], idx int32 [B,H,16k], count int32
+    [B,H], cand_count int32 [B,H])``, k = budget pages clamped to ``max_pages_per_req``; with
+    ``return_scores`` also ``page_scores`` fp32 [B,H,max_pages_per_req] and ``scores`` fp32
+    [B,H,16k].
+    """
+    from .quest import quest_num_pages
+    from .sampling import _check_p, _high_mode
+    check_input(q, "q")
+    check_dim(3, q, "q")
+    B, H, D = q.shape
+    if D != _lib.HEAD_DIM:
+        raise RuntimeError(f"head_dim must be {_lib.HEAD_DIM}, got {D}")
+    check_input(k_int4, "k_int4")
+    check_dtype(k_int4, torch.uint8, "k_int4")
+    if k_int4.dim() != 3 or k_int4.size(2) != _lib.INT4_RECORD_BYTES:
+        raise RuntimeError("k_int4 must be uint8 [pages, kv_heads, 1280]")
+    Hkv = k_int4.size(1)
+    check_input(meta, "meta")
+    check_dtype(meta, torch.uint8, "meta")
+    if meta.dim() != 3 or meta.size(1) != Hkv or meta.size(2) != _lib.META_RECORD_BYTES \
+            or meta.size(0) != k_int4.size(0):
+        raise RuntimeError("meta must be uint8 [pages, kv_heads, 512] like k_int4")
+    if H % Hkv != 0:
+        raise RuntimeError(f"num_q_heads {H} must be a multiple of num_kv_heads {Hkv}")
+    for name, t in (("kv_page_indices", kv_page_indices), ("kv_page_indptr", kv_page_indptr),
+                    ("kv_last_page_len", kv_last_page_len)):
+        check_input(t, name)
+        check_dtype(t, torch.int32, name)
+    if kv_page_indptr.numel() != B + 1 or kv_last_page_len.numel() != B:
+        raise RuntimeError("kv_page_indptr must have B+1 and kv_last_page_len B elements")
+    if token_budget <= 0 or max_pages_per_req <= 0 or max_pages_per_req > 8192:
+        raise RuntimeError("token_budget must be positive and max_pages_per_req in [1, 8192]")
+    k = quest_num_pages(token_budget, max_pages_per_req)
+    M = k * _lib.PAGE
+    if M > _lib.MAX_CANDIDATES:
+        raise RuntimeError(f"{M} candidates exceed the supported maximum {_lib.MAX_CANDIDATES}")
+    p_arr, p_val = _check_p(top_p, B * H, q)
+    check_same_device(q, ("k_int4", k_int4), ("meta", meta), ("kv_page_indices", kv_page_indices),
+                      ("kv_page_indptr", kv_page_indptr), ("kv_last_page_len", kv_last_page_len))
+    dev = q.device
+    with torch.cuda.device(dev):
+        sel = torch.zeros((B, H, k), dtype=torch.int32, device=dev)
+        selc = torch.empty((B, H), dtype=torch.int32, device=dev)
+        idx = torch.empty((B, H, M), dtype=torch.int32, device=dev)
+        count = torch.empty((B, H), dtype=torch.int32, device=dev)
+        cand = torch.empty((B, H), dtype=torch.int32, device=dev)
+        ps = (torch.zeros((B, H, max_pages_per_req), dtype=torch.float32, device=dev)
+              if return_scores else None)
+        scores = (torch.full((B, H, M), float("-inf"), dtype=torch.float32, device=dev)
+                  if return_scores else None)
+        scale = 1.0 / math.sqrt(D) if sm_scale is None else float(sm_scale)
+        rc = _lib.lib().twl_select_estimate_prune(
+            ptr(q), dtype_code(q.dtype, "q"), ptr(meta), ptr(k_int4), ptr(kv_page_indices),
+            ptr(kv_page_indptr), ptr(kv_last_page_len), B, H, Hkv, int(token_budget),
+            int(max_pages_per_req), scale, ptr(p_arr), p_val, _high_mode(high), ptr(sel), k,
+            ptr(selc), ptr(idx), M, ptr(count), ptr(ps), max_pages_per_req, ptr(scores), M,
+            ptr(cand), stream_of(q))
+    _lib.check(rc, "SelectEstimatePrune")
+    out = [sel, selc, idx, count, cand]
+    if return_scores:
+        out += [ps, scores]
+    return tuple(out)
+
+
 def batched_sparse_gemv_int4_k(q: torch.Tensor, o: torch.Tensor, k_u8: torch.Tensor,
                                quant_scales: torch.Tensor, quant_zeros: torch.Tensor,
                                kv_page_indices: torch.Tensor, kv_page_indptr: torch.Tensor,
