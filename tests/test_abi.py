@@ -93,6 +93,41 @@ def test_c_level_validation_without_gpu(hip_lib):
     assert L.twl_kv_shadow_build(fake, 0, 4096, 256, 128, 0, 0, 1, 1, 0, 0, 0) == -1
     assert L.twl_dequant_int4(fake, 0, fake, 0) == -2
     assert L.twl_decode_layer(None, 0) == -1
+    # entry points added after the first ABI version
+    f = fake
+    gtp = lambda **kw: L.twl_gemv_top_p(
+        kw.get("q", f), kw.get("dt", 0), f, kw.get("sel", f), f, kw.get("sel_stride", 4), f, f, f,
+        1, kw.get("hq", 1), kw.get("hkv", 1), kw.get("k", 4), 1.0, 0, kw.get("p", 0.9),
+        kw.get("high", 1), kw.get("idx", f), kw.get("idx_stride", 64), f, 0, 64, 0, 0, 0)
+    assert gtp(sel=0) == -1 and gtp(idx=0) == -1
+    assert gtp(dt=2) == -3
+    assert gtp(hq=3, hkv=2) == -2 and gtp(k=0) == -2 and gtp(k=4096) == -2
+    assert gtp(sel_stride=2) == -2 and gtp(idx_stride=32) == -2
+    assert gtp(p=0.0) == -2 and gtp(high=5) == -2
+    assert gtp(q=f + 8) == -4
+    sep = lambda **kw: L.twl_select_estimate_prune(
+        kw.get("q", f), kw.get("dt", 0), kw.get("meta", f), f, f, f, f, 1, kw.get("hq", 1),
+        kw.get("hkv", 1), kw.get("budget", 64), kw.get("npg", 16), 1.0, 0, kw.get("p", 0.9), 1,
+        kw.get("sel", f), kw.get("sel_stride", 4), f, f, kw.get("idx_stride", 64), f, 0, 0, 0, 64,
+        0, 0)
+    assert sep(meta=0) == -1 and sep(sel=0) == -1
+    assert sep(dt=5) == -3
+    assert sep(budget=0) == -2 and sep(npg=0) == -2 and sep(npg=9000) == -2
+    assert sep(sel_stride=3) == -2 and sep(idx_stride=63) == -2 and sep(p=2.0) == -2
+    assert sep(hq=4, hkv=3) == -2
+    assert sep(q=f + 4) == -4
+    app = lambda **kw: L.twl_kv_append(
+        kw.get("k", f), f, kw.get("dt", 0), 256, 128, f, f, 4096, kw.get("ts", 256), 128, f, f,
+        kw.get("last", f), kw.get("b", 1), 1, 0, 0, 0)
+    assert app(k=0) == -1 and app(last=0) == -1
+    assert app(dt=2) == -3 and app(b=0) == -2 and app(ts=250) == -4 and app(k=f + 2) == -4
+    qk = lambda **kw: L.twl_qk_int8_lse(
+        kw.get("q", f), f, f, f, kw.get("lse", f), 1, kw.get("hq", 1), kw.get("hkv", 1),
+        kw.get("qo", 8), kw.get("kv", 8), kw.get("d", 128), 1024, 1024, kw.get("sqn", 128),
+        1024, 1024, 128, 0)
+    assert qk(q=0) == -1 and qk(lse=0) == -1
+    assert qk(d=96) == -2 and qk(qo=0) == -2 and qk(kv=0) == -2 and qk(hq=3, hkv=2) == -2
+    assert qk(sqn=100) == -4 and qk(q=f + 1) == -4
 
 
 def test_python_ops_reject_cpu_and_malformed_tensors(hip_lib):

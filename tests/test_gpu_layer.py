@@ -208,3 +208,41 @@ def test_full_size_cfg4_layer_sampled_rows_and_properties(dev):
         assert torch.allclose(out[b, h].float().cpu(), own[0, 0, 0], rtol=tol, atol=tol), r
         compared += 1
     assert compared >= len(picks) - 1, (compared, len(picks))
+
+
+@pytest.mark.parametrize("H,Hkv", [(8, 8), (8, 2)])
+def test_layer_step_replays_from_a_hip_graph(dev, H, Hkv):
+    # a serving loop captures the decode step: every replay, with eager work and synchronisations
+    # between replays and new q / K contents each time, must equal the eager result (the library
+    # enqueues kernels only: no allocation, no memset, no host synchronisation)
+    B, N = 32, 1024                  # MHA: 256 rows -> the one-launch row kernel; GQA: three launches
+    g = torch.Generator().manual_seed(H + Hkv)
+    k = torch.randn((B, Hkv, N, 128), generator=g).half()
+    v = torch.randn((B, Hkv, N, 128), generator=g).half()
+    cache = PagedKVCache.from_dense(k, v, dev, spare_pages=B)
+    layer = TwilightDecodeLayer(cache, H, token_budget=256, top_p=0.9, reserve_pages=N // 16 + 1)
+    q = torch.randn((B, H, 128), generator=g).half().to(dev)
+    layer(q)                          # warm-up outside the capture
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        layer(q)
+    torch.cuda.synchronize()
+    for step in range(4):
+        q.copy_(torch.randn((B, H, 128), generator=g).half())      # same buffer, new contents
+        if step == 2:                 # the cache contents change under the graph too
+            cache.k_cache.mul_(-0.5)
+            cache.rebuild_shadow()
+        eager = layer(q).clone()
+        cnt_e, idx_e = layer.count.clone(), layer.idx.clone()
+        torch.cuda.synchronize()
+        layer.out.zero_(); layer.count.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(layer.out, eager), step
+        assert torch.equal(layer.count, cnt_e)
+        mx = int(cnt_e.max())
+        assert torch.equal(layer.idx[..., :mx] * (torch.arange(mx, device=dev) < cnt_e[..., None]),
+                           idx_e[..., :mx] * (torch.arange(mx, device=dev) < cnt_e[..., None]))
