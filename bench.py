@@ -372,7 +372,7 @@ def main() -> int:
         cpu = cpu_baseline(N, H, args.budget, args.top_p, B, dev)
 
     line = {
-        "metric": "us/decode-layer at 32k ctx (select+prune+attn)",
+        "metric": "\u00b5s/decode-layer at 32k ctx (select+prune+attn); GEMV & attn HBM GB/s vs peak",
         "value": round(wall_us, 2), "unit": "us", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(wall_us / 1e3, 5), "higher_is_better": False,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if llama else "f16",
