@@ -14,6 +14,11 @@ How each function is pinned (tests/test_oracle_*.py):
   top_p_unnormalized     softmax is torch's; the bisection is oracle.native.top_p_mask_f32
                          (pinned against the textbook nucleus set and brute force)
   masked_attention       reduces to softmax + matmul over gathered survivors (checked both ways)
+  get_label_tensor_ref, bgemv_int8_ref
+                         the reference's own torch checks (channel.py:82-110, bgemv_int8.py:78-93),
+                         i.e. a gather and a matmul
+  qk_int8_lse_ref        closed form: float64 base-2 logsumexp of the dequantised product plus
+                         the zero-padded tail of the last key block
 """
 from __future__ import annotations
 
