@@ -140,7 +140,10 @@ int twl_gemv_top_p(const void* q, int q_dtype, const void* k_int4, const int32_t
  * top_p.py:10-15 + attention.py:280-281. Outputs as those three calls give them: sel_pages /
  * sel_count (ascending logical pages, ties at the k-th score to the lower page), idx / count,
  * optionally page_scores_out [rows, page_score_stride], scores_out [rows, score_stride] and
- * cand_count. max_pages_per_req <= 8192. Meant for about one row per compute unit (MHA decode at
+ * cand_count. max_pages_per_req <= 8192. With meta_planes (plane layout, see
+ * twl_meta_planes_build; then meta may be NULL) the page scores are accumulated channel by channel
+ * in ascending order from the sign-selected runs; they can differ from twl_quest_page_scores in
+ * the last bits (other summation order). Meant for about one row per compute unit (MHA decode at
  * moderate batch); with GQA the three-call form reads each metadata record once per kv head and
  * this one once per q head.
  * ------------------------------------------------------------------------------------------- */
@@ -153,7 +156,7 @@ int twl_select_estimate_prune(const void* q, int dtype, const void* meta, const 
                               int32_t* sel_count, int32_t* idx, uint32_t idx_stride,
                               int32_t* count, float* page_scores_out, uint32_t page_score_stride,
                               float* scores_out, uint32_t score_stride, int32_t* cand_count,
-                              void* stream);
+                              const void* meta_planes, uint32_t plane_cap_pages, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * INT4-K score GEMV over candidate pages: out[r, c] = sm_scale * sum_d q[r,d] * dequant(K[c,d]).
@@ -274,14 +277,29 @@ int twl_kv_shadow_build(const void* k_cache, int kv_dtype, uint64_t page_stride,
  * request b the token goes to slot s = kv_last_page_len[b] (0..15) of its LAST listed page; the
  * caller has appended a fresh page to the table and set the length to 0 when the previous page was
  * full. Writes the K / V rows, the token's INT4 codes and (scale, zero) pairs (a fresh page's
- * other tokens are zeroed), folds the row into the page's min / max metadata, and stores s + 1
- * to kv_last_page_len[b]. k_int4 / meta may be NULL. Records are identical to what
+ * other tokens are zeroed), folds the row into the page's min / max metadata (records and, when
+ * meta_planes is given, the plane layout below), and stores s + 1 to kv_last_page_len[b].
+ * k_int4 / meta / meta_planes may be NULL. Records are identical to what
  * twl_kv_shadow_build gives for the same page contents. */
 int twl_kv_append(const void* k_new, const void* v_new, int kv_dtype, uint64_t new_batch_stride,
                   uint64_t new_head_stride, void* k_cache, void* v_cache, uint64_t page_stride,
                   uint64_t token_stride, uint64_t head_stride, const int32_t* kv_page_indices,
                   const int32_t* kv_page_indptr, int32_t* kv_last_page_len, uint32_t batch,
-                  uint32_t num_kv_heads, void* k_int4, void* meta, void* stream);
+                  uint32_t num_kv_heads, void* k_int4, void* meta, void* meta_planes,
+                  uint32_t plane_cap_pages, void* stream);
+
+/* Quest metadata in PLANE layout: planes[slot][kv_head][d][0 = min, 1 = max][logical page], 16-bit
+ * values in the cache dtype, plane_cap_pages (a multiple of 8) pages per run, slot = position of
+ * the request in the batch. For one query only the run selected by the sign of q_d is read
+ * (score = sum_d q_d * (q_d > 0 ? max_d : min_d), twilight/pyimpl/quest.py:37-84), so the scoring
+ * pass of twl_select_estimate_prune touches half the bytes of the record layout. Nothing in the
+ * reference corresponds to it (it recomputes the chunk maxima from K every step, quest.py:68-74).
+ * twl_meta_planes_build fills the planes of the pages of the current page table from the metadata
+ * records of twl_kv_shadow_build; twl_kv_append keeps them current when given meta_planes. */
+int twl_meta_planes_build(const void* meta, const int32_t* kv_page_indices,
+                          const int32_t* kv_page_indptr, uint32_t batch, uint32_t num_kv_heads,
+                          uint32_t max_pages_per_req, void* meta_planes, uint32_t plane_cap_pages,
+                          void* stream);
 
 /* Unpack INT4 shadow records to fp32: out [num_pages, num_kv_heads, 16, 128] (record order).
  * Exists so that tests can compare dequantised values bit for bit. */
@@ -336,6 +354,8 @@ typedef struct twl_layer_args {
   uint64_t page_stride, token_stride, head_stride; /* element strides of both caches */
   const void* k_int4;       /* INT4 shadow records */
   const void* meta;         /* Quest metadata records */
+  const void* meta_planes;  /* the same in plane layout (nullable), see twl_meta_planes_build */
+  uint32_t plane_cap_pages;
   const int32_t* kv_page_indices;
   const int32_t* kv_page_indptr;
   const int32_t* kv_last_page_len;

@@ -201,3 +201,61 @@ def test_one_launch_row_kernel_equals_three_launches(dev, N, lens, budget, H, Hk
             toks = iB[b, h, :cB[b, h]].long()
             assert torch.all(toks[1:] > toks[:-1]) and int(toks.max()) < N
     assert differ <= 1
+
+
+@pytest.mark.parametrize("N,budget,H,dt", [
+    (1600, 320, 4, torch.float16),
+    (1000, 100, 4, torch.bfloat16),          # partial last page, budget not a multiple of 16
+    (11200, 16384, 2, torch.float16),        # every page
+    (40000, 4096, 2, torch.float16),         # 2500 pages per request (four scoring passes)
+    (32768, 8192, 2, torch.float16),         # the benchmark's row shape
+])
+def test_row_kernel_with_plane_metadata(dev, N, budget, H, dt):
+    """The plane layout (minima / maxima of all pages of a request contiguous per channel) against
+    the record layout: planes hold exactly the records' numbers; page scores agree to summation
+    order; the page lists are equal except pages whose score ties the k-th within rounding; rows
+    with equal lists give identical candidate scores and survivors."""
+    from twilight_amd.cache import PagedKVCache
+    B, p = 2, 0.9
+    g = torch.Generator().manual_seed(N + 1)
+    q = torch.randn((B, H, 128), generator=g)
+    k = torch.randn((B, H, N, 128), generator=g)
+    for b in range(B):
+        for h in range(H):
+            pos = torch.randint(0, N, (6,), generator=g)
+            k[b, h, pos] += q[b, h] * (0.3 + torch.rand(6, 1, generator=g))
+    npg = (N + 15) // 16
+    cache = PagedKVCache.from_dense(k.to(dt), k.to(dt), dev,
+                                    page_perm=torch.randperm(B * npg, generator=g), plane_pages=npg + 9)
+    # planes == transposed records, bit for bit
+    cap = cache.meta_planes.shape[-1]
+    assert cap % 8 == 0 and cap >= npg
+    rec = cache.meta.view(torch.int16).reshape(-1, H, 32, 2, 4)              # [page, h, chunk, min|max, 4]
+    phys = cache.kv_page_indices.long().reshape(B, npg)
+    want = rec[phys].permute(0, 2, 3, 5, 4, 1).reshape(B, H, 128, 2, npg)    # [b, h, d, min|max, page]
+    assert torch.equal(cache.meta_planes.view(torch.int16)[..., :npg], want)
+    qd = q.to(dt).to(dev)
+    tab = (cache.kv_page_indices, cache.kv_page_indptr, cache.kv_last_page_len)
+    A = K.quest_gemv_int4_top_p(qd, cache.meta, cache.k_int4, *tab, budget, npg, p, return_scores=True)
+    Bv = K.quest_gemv_int4_top_p(qd, cache.meta, cache.k_int4, *tab, budget, npg, p, return_scores=True,
+                                 meta_planes=cache.meta_planes)
+    selA, selcA, idxA, cntA, candA, psA, scA = [t.cpu() for t in A]
+    selB, selcB, idxB, cntB, candB, psB, scB = [t.cpu() for t in Bv]
+    assert torch.allclose(psA, psB, rtol=1e-5, atol=1e-4)
+    assert torch.equal(selcA, selcB) and torch.equal(candA, candB)
+    kk = int(selcA[0, 0])
+    same_rows = 0
+    for b in range(B):
+        for h in range(H):
+            a_set, b_set = set(selA[b, h, :kk].tolist()), set(selB[b, h, :kk].tolist())
+            assert torch.all(selB[b, h, 1:kk] > selB[b, h, :kk - 1])
+            kth = torch.sort(psA[b, h, :npg], descending=True).values[kk - 1]
+            for pg in a_set ^ b_set:       # only pages tied with the k-th score may differ
+                assert abs(float(psA[b, h, pg]) - float(kth)) <= 1e-4 * max(1.0, abs(float(kth)))
+            if a_set == b_set:
+                same_rows += 1
+                n = kk * 16
+                assert torch.equal(scA[b, h, :n].view(torch.int32), scB[b, h, :n].view(torch.int32))
+                assert int(cntA[b, h]) == int(cntB[b, h])
+                assert torch.equal(idxA[b, h, :cntA[b, h]], idxB[b, h, :cntB[b, h]])
+    assert same_rows >= B * H - 1

@@ -126,13 +126,16 @@ def test_append_kernel_records_equal_bulk_build(dev, dt):
     k = (torch.randn((B, Hkv, N0 + steps, 128), generator=g) * 2).to(dt)
     v = torch.randn((B, Hkv, N0 + steps, 128), generator=g).to(dt)
     cache = PagedKVCache.from_dense(k[:, :, :N0].contiguous(), v[:, :, :N0].contiguous(), dev,
-                                    spare_pages=12)
+                                    spare_pages=12, plane_pages=8)
     free = list(range(9, 21))
     for s in range(steps):
         # a strided view (the layout a projection + transpose hands over)
         cache.append(k[:, :, N0 + s].to(dev), v[:, :, N0 + s].to(dev), free)
-    full = PagedKVCache.from_dense(k, v, dev)
+    full = PagedKVCache.from_dense(k, v, dev, plane_pages=8)
     assert torch.equal(cache.kv_last_page_len.cpu(), full.kv_last_page_len.cpu())
+    npg_now = (N0 + steps + 15) // 16
+    assert torch.equal(cache.meta_planes.view(torch.int16)[..., :npg_now],
+                       full.meta_planes.view(torch.int16)[..., :npg_now])   # plane-layout metadata too
     ia, ib = cache.kv_page_indices.long(), full.kv_page_indices.long()
     assert ia.numel() == ib.numel()
     for name in ("k_cache", "v_cache", "k_int4", "meta"):

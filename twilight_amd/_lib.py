@@ -27,7 +27,7 @@ EXPORTS = (
     "twl_softmax_top_p_f32", "twl_gemv_top_p", "twl_select_estimate_prune", "twl_gemv_int4", "twl_gemv_int4_nhd",
     "twl_gemv_int8_nhd", "twl_gemv_f16_nhd", "twl_gemv_f16_single", "twl_sparse_attn",
     "twl_sparse_attn_workspace_bytes", "twl_quest_select",
-    "twl_quest_page_scores", "twl_quest_topk_pages", "twl_kv_shadow_build", "twl_kv_append", "twl_dequant_int4",
+    "twl_quest_page_scores", "twl_quest_topk_pages", "twl_kv_shadow_build", "twl_kv_append", "twl_meta_planes_build", "twl_dequant_int4",
     "twl_decode_layer", "twl_get_label_tensor", "twl_bgemv_int8", "twl_qk_int8_lse",
 )
 
@@ -38,6 +38,7 @@ class LayerArgs(ctypes.Structure):
         ("q", c_void_p), ("dtype", c_int), ("k_cache", c_void_p), ("v_cache", c_void_p),
         ("page_stride", c_uint64), ("token_stride", c_uint64), ("head_stride", c_uint64),
         ("k_int4", c_void_p), ("meta", c_void_p),
+        ("meta_planes", c_void_p), ("plane_cap_pages", c_uint32),
         ("kv_page_indices", c_void_p), ("kv_page_indptr", c_void_p), ("kv_last_page_len", c_void_p),
         ("batch", c_uint32), ("num_q_heads", c_uint32), ("num_kv_heads", c_uint32),
         ("max_pages_per_req", c_uint32), ("token_budget", c_uint32),
@@ -81,7 +82,7 @@ def lib() -> ctypes.CDLL:
                                  f32, i32, vp, u32, vp, vp, u32, vp, vp, vp]
     L.twl_select_estimate_prune.argtypes = [vp, i32, vp, vp, vp, vp, vp, u32, u32, u32, u32, u32,
                                             f32, vp, f32, i32, vp, u32, vp, vp, u32, vp, vp, u32,
-                                            vp, u32, vp, vp]
+                                            vp, u32, vp, vp, u32, vp]
     L.twl_gemv_int4.argtypes = [vp, i32, vp, u32, vp, vp, vp, vp, u32, vp, vp, vp, u32, u32, u32,
                                 u32, f32, vp]
     L.twl_gemv_int4_nhd.argtypes = [vp, vp, u32, vp, vp, vp, vp, vp, vp, u32, u32, u32, u32, f32, vp]
@@ -101,7 +102,8 @@ def lib() -> ctypes.CDLL:
     L.twl_get_label_tensor.argtypes = [vp, vp, vp, u32, u32, u32, u32] + [c_int64] * 8 + [vp]
     L.twl_bgemv_int8.argtypes = [vp, vp, vp, vp, u32, u32, u32, u32] + [c_int64] * 11 + [vp]
     L.twl_kv_append.argtypes = [vp, vp, i32, u64, u64, vp, vp, u64, u64, u64, vp, vp, vp, u32, u32,
-                                vp, vp, vp]
+                                vp, vp, vp, u32, vp]
+    L.twl_meta_planes_build.argtypes = [vp, vp, vp, u32, u32, u32, vp, u32, vp]
     i64 = ctypes.c_int64
     L.twl_qk_int8_lse.argtypes = [vp, vp, vp, vp, vp, u32, u32, u32, u32, u32, u32, i64, i64, i64,
                                   i64, i64, i64, vp]

@@ -7,7 +7,7 @@ from typing import Optional
 import torch
 
 from . import _lib
-from .kernel import kv_append, kv_shadow_build
+from .kernel import kv_append, kv_shadow_build, meta_planes_build
 
 PAGE = _lib.PAGE
 HEAD_DIM = _lib.HEAD_DIM
@@ -36,6 +36,8 @@ class PagedKVCache:
         self.kv_last_page_len: Optional[torch.Tensor] = None
         self.max_pages_per_req = 0
         self._seq_lens = None  # host copy, for append bookkeeping
+        # Quest metadata in plane layout [batch, Hkv, 128, 2, cap] (see enable_planes)
+        self.meta_planes: Optional[torch.Tensor] = None
 
     # ---- page table ---------------------------------------------------------------------------
     def set_page_table(self, kv_page_indices: torch.Tensor, kv_page_indptr: torch.Tensor,
@@ -61,12 +63,35 @@ class PagedKVCache:
     def rebuild_shadow(self, page_ids: Optional[torch.Tensor] = None,
                        valid_len: Optional[torch.Tensor] = None) -> None:
         """(Re)build INT4 records and Quest metadata of ``page_ids`` (default: every page, all 16
-        tokens valid)."""
+        tokens valid), and the plane-layout metadata of the whole page table when enabled."""
         kv_shadow_build(self.k_cache, self.k_int4, self.meta, page_ids, valid_len)
+        self.rebuild_planes()
+
+    def enable_planes(self, cap_pages: Optional[int] = None) -> None:
+        """Keep the Quest metadata also in plane layout (per request slot, kv head and channel the
+        page minima contiguously, then the maxima), sized for requests of up to ``cap_pages`` pages
+        (default: the current longest request). The one-launch selector of MHA layers then reads
+        half the metadata bytes. Needs a page table; the batch size fixes the number of slots."""
+        if self.kv_page_indptr is None:
+            raise RuntimeError("enable_planes needs a page table (set_page_table)")
+        cap = max(int(cap_pages or 0), self.max_pages_per_req, 8)
+        cap = (cap + 7) // 8 * 8
+        self.meta_planes = torch.zeros((self.batch, self.num_kv_heads, HEAD_DIM, 2, cap),
+                                       dtype=self.dtype, device=self.device)
+        self.rebuild_planes()
+
+    def rebuild_planes(self) -> None:
+        """Refill the plane-layout metadata from the records, for the pages of the page table."""
+        if self.meta_planes is None or self.kv_page_indptr is None:
+            return
+        if self.batch != self.meta_planes.size(0) or self.max_pages_per_req > self.meta_planes.size(4):
+            raise RuntimeError("the page table no longer fits the plane buffer: call enable_planes")
+        meta_planes_build(self.meta, self.kv_page_indices, self.kv_page_indptr,
+                          self.max_pages_per_req, self.meta_planes)
 
     @classmethod
     def from_dense(cls, k: torch.Tensor, v: torch.Tensor, device, page_perm: Optional[torch.Tensor] = None,
-                   spare_pages: int = 0) -> "PagedKVCache":
+                   spare_pages: int = 0, plane_pages: Optional[int] = None) -> "PagedKVCache":
         """Page dense ``k`` / ``v`` [B, Hkv, N, 128] (prefill fill). ``page_perm`` (a permutation of
         ``B*ceil(N/16)`` ids) scatters logical pages over physical slots."""
         B, Hkv, N, D = k.shape
@@ -96,6 +121,8 @@ class PagedKVCache:
         valid[last_pages] = last
         ids = torch.arange(total + spare_pages, dtype=torch.int32)
         c.rebuild_shadow(ids.to(c.device), valid.to(c.device))
+        if plane_pages is not None:
+            c.enable_planes(plane_pages)
         return c
 
     def append(self, k_new: torch.Tensor, v_new: torch.Tensor, free_pages: Optional[list] = None) -> None:
@@ -121,6 +148,9 @@ class PagedKVCache:
             self.kv_page_indices = torch.tensor(flat, dtype=torch.int32, device=self.device)
             self.kv_page_indptr = torch.tensor(ptr, dtype=torch.int32, device=self.device)
             self.max_pages_per_req = max(len(r) for r in per_req)
+            if self.meta_planes is not None and self.max_pages_per_req > self.meta_planes.size(4):
+                raise RuntimeError("PagedKVCache.append: request outgrew the plane buffer "
+                                   "(enable_planes with a larger cap_pages)")
             # same tensor object every step, so cached argument blocks of the layer stay valid
             self.kv_last_page_len.copy_(torch.tensor(last, dtype=torch.int32))
         k_new = k_new.to(self.device, self.dtype)
@@ -129,7 +159,8 @@ class PagedKVCache:
             k_new, v_new = k_new.contiguous(), v_new.contiguous()
         # one launch: rows, INT4 codes, min/max metadata, and the device-side lengths + 1
         kv_append(k_new, v_new, self.k_cache, self.v_cache, self.kv_page_indices,
-                  self.kv_page_indptr, self.kv_last_page_len, self.k_int4, self.meta)
+                  self.kv_page_indptr, self.kv_last_page_len, self.k_int4, self.meta,
+                  self.meta_planes)
         for b in range(B):
             last[b] += 1
             self._seq_lens[b] += 1

@@ -17,7 +17,7 @@ extern "C" const char* twl_strerror(int status) {
   }
 }
 
-extern "C" int twl_abi_version(void) { return 2; }
+extern "C" int twl_abi_version(void) { return 3; }
 
 extern "C" int twl_device_count(void) {
   int n = 0;
@@ -88,7 +88,8 @@ extern "C" int twl_decode_layer(const twl_layer_args* a, void* stream) {
         a->max_pages_per_req, a->sm_scale, nullptr, a->top_p, a->high_mode, a->sel_pages,
         a->sel_stride, a->sel_count, a->idx, a->idx_stride, a->count,
         a->keep_scores ? a->page_scores : nullptr, a->page_score_stride,
-        a->keep_scores ? a->scores : nullptr, a->score_stride, a->cand_count, stream);
+        a->keep_scores ? a->scores : nullptr, a->score_stride, a->cand_count, a->meta_planes,
+        a->plane_cap_pages, stream);
     if (rc != TWL_OK) return rc;
   } else {
     // 1. Quest page scores + top-k pages

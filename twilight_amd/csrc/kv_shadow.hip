@@ -129,6 +129,8 @@ struct AppendArgs {
   uint32_t num_kv_heads;
   uint8_t* k_int4;
   uint8_t* meta;
+  uint16_t* planes;     // nullable: metadata in plane layout (meta_planes.hip)
+  uint32_t plane_cap;
 };
 
 template <int DT>
@@ -210,6 +212,26 @@ __global__ __launch_bounds__(kShThreads) void kv_append_kernel(AppendArgs a) {
       *pmin = f32_to_bits16<DT>(mn0) | (f32_to_bits16<DT>(mn1) << 16);
       *pmax = f32_to_bits16<DT>(mx0) | (f32_to_bits16<DT>(mx1) << 16);
     }
+    if (a.planes && n_pages <= (int)a.plane_cap) {
+      // the same fold in the plane layout: runs [d][min|max][logical page] of slot b
+      uint16_t* pl = a.planes + ((size_t)b * a.num_kv_heads + kvh) * (TWL_HEAD_DIM * 2) * a.plane_cap +
+                     (n_pages - 1);
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int d = 2 * lane + j;
+        const uint32_t kb = j ? (kw >> 16) : (kw & 0xFFFFu);
+        const float kv = bits16_to_f32<DT>(kb);
+        uint16_t* pmn = pl + (size_t)(2 * d) * a.plane_cap;
+        uint16_t* pmx = pl + (size_t)(2 * d + 1) * a.plane_cap;
+        float mn = kv, mx = kv;
+        if (slot > 0) {
+          mn = fminf(mn, bits16_to_f32<DT>(*pmn));
+          mx = fmaxf(mx, bits16_to_f32<DT>(*pmx));
+        }
+        *pmn = (uint16_t)f32_to_bits16<DT>(mn);
+        *pmx = (uint16_t)f32_to_bits16<DT>(mx);
+      }
+    }
   }
   if (threadIdx.x == 0) a.kv_last_page_len[b] = slot + 1;
 }
@@ -281,7 +303,7 @@ extern "C" int twl_kv_append(const void* k_new, const void* v_new, int kv_dtype,
                              uint64_t head_stride, const int32_t* kv_page_indices,
                              const int32_t* kv_page_indptr, int32_t* kv_last_page_len,
                              uint32_t batch, uint32_t num_kv_heads, void* k_int4, void* meta,
-                             void* stream) {
+                             void* meta_planes, uint32_t plane_cap_pages, void* stream) {
   if (!k_new || !v_new || !k_cache || !v_cache || !kv_page_indices || !kv_page_indptr ||
       !kv_last_page_len)
     return TWL_ENULL;
@@ -290,8 +312,10 @@ extern "C" int twl_kv_append(const void* k_new, const void* v_new, int kv_dtype,
   if ((page_stride | token_stride | head_stride | new_batch_stride | new_head_stride) & 7u)
     return TWL_EALIGN;
   if ((((uintptr_t)k_new) & 15u) || (((uintptr_t)v_new) & 15u) || (((uintptr_t)k_cache) & 15u) ||
-      (((uintptr_t)v_cache) & 15u) || (((uintptr_t)k_int4) & 15u) || (((uintptr_t)meta) & 15u))
+      (((uintptr_t)v_cache) & 15u) || (((uintptr_t)k_int4) & 15u) || (((uintptr_t)meta) & 15u) ||
+      (((uintptr_t)meta_planes) & 15u))
     return TWL_EALIGN;
+  if (meta_planes && (plane_cap_pages == 0 || (plane_cap_pages & 7u))) return TWL_EINVAL;
   twl::AppendArgs a{};
   a.k_new = k_new; a.v_new = v_new; a.new_batch_stride = new_batch_stride;
   a.new_head_stride = new_head_stride; a.k_cache = k_cache; a.v_cache = v_cache;
@@ -299,6 +323,7 @@ extern "C" int twl_kv_append(const void* k_new, const void* v_new, int kv_dtype,
   a.kv_page_indices = kv_page_indices; a.kv_page_indptr = kv_page_indptr;
   a.kv_last_page_len = kv_last_page_len; a.num_kv_heads = num_kv_heads;
   a.k_int4 = (uint8_t*)k_int4; a.meta = (uint8_t*)meta;
+  a.planes = (uint16_t*)meta_planes; a.plane_cap = plane_cap_pages;
   if (kv_dtype == TWL_F16)
     hipLaunchKernelGGL((twl::kv_append_kernel<TWL_F16>), dim3(batch), dim3(twl::kShThreads), 0,
                        (hipStream_t)stream, a);

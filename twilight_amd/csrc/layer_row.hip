@@ -29,6 +29,8 @@ struct RowArgs {
   int32_t* sel_count_out;
   float* page_scores_out;   // nullable
   uint32_t page_score_stride;
+  const uint16_t* planes;   // PLANES: metadata in plane layout (meta_planes.hip), slot = batch index
+  uint32_t plane_cap;
 };
 
 constexpr int kRowThreads = 1024;
@@ -38,7 +40,10 @@ constexpr int kRowWaves = kRowThreads / kWave;
 #endif
 constexpr int kRowUnroll = TWL_ROW_UNROLL;  // 16-byte loads in flight per lane (2 pages each)
 
-template <int QDT, int VPT, int SEL_VPT>
+// PLANES: page scores from the plane layout (half the metadata bytes: only the run the sign of
+// q_d selects is read, 2 pages per lane, channels in ascending order), else from the 512-byte
+// records through the page table.
+template <int QDT, int VPT, int SEL_VPT, bool PLANES>
 __global__ __launch_bounds__(kRowThreads) void select_estimate_prune_kernel(RowArgs a) {
   constexpr int PW = 4 * VPT;
   constexpr int RUNS = (PW + 63) / 64;
@@ -71,75 +76,111 @@ __global__ __launch_bounds__(kRowThreads) void select_estimate_prune_kernel(RowA
   const int n_req = min(max(req_pages, 0), min((int)a.max_pages_req, kRowThreads * SEL_VPT));
 
   // ---- 1. Quest page scores into LDS ---------------------------------------------------------
-  // page ids of all passes first: register r, lane l <-> pass 2r + l/32, page l%32 of the wave's
-  // 32-page slice of that pass
-  int ids[SEL_VPT];
+  if constexpr (PLANES) {
+    // lane l keeps q[l] and q[64 + l]; q_d reaches every lane as a scalar
+    const uint16_t* qrow = (const uint16_t*)a.f.q + (size_t)row * TWL_HEAD_DIM;
+    const float q_lo = bits16_to_f32<QDT>(qrow[lane]);
+    const float q_hi = bits16_to_f32<QDT>(qrow[64 + lane]);
+    const uint16_t* pl =
+        a.planes + ((size_t)b * a.f.num_kv_heads + kvh) * (TWL_HEAD_DIM * 2) * a.plane_cap;
+    constexpr int PL_PASSES = (SEL_VPT + 1) / 2;  // 16 waves x 128 pages = 2048 pages per pass
 #pragma unroll
-  for (int r = 0; r < SEL_VPT; ++r) {
-    const int pg = ((2 * r + half) * kRowWaves + wave) * 32 + c;
-    ids[r] = (pg < n_req) ? a.f.kv_page_indices[pg_begin + pg] : 0;
-  }
-  float qf[4];
-  uint32_t selmask[2];
-#pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    qf[2 * j] = bits16_to_f32<QDT>(qw[j] & 0xFFFFu);
-    qf[2 * j + 1] = bits16_to_f32<QDT>(qw[j] >> 16);
-    selmask[j] = (qf[2 * j] > 0.0f ? 0x0000FFFFu : 0u) | (qf[2 * j + 1] > 0.0f ? 0xFFFF0000u : 0u);
-  }
-  const size_t meta_stride = (size_t)a.f.num_kv_heads * TWL_META_RECORD_BYTES;
-  const uint8_t* mbase = a.meta + (size_t)kvh * TWL_META_RECORD_BYTES + 16 * c;
-#pragma unroll
-  for (int pass = 0; pass < PASSES; ++pass) {
-    const int p0 = (pass * kRowWaves + wave) * 32;
-    const int np = min(32, n_req - p0);  // wave-uniform
-    if (np > 0) {
-      const int lbase = (pass & 1) * 32;
-      float keep = 0.0f;  // lane i ends up with the score of page p0 + i
-#pragma unroll
-      for (int i0 = 0; i0 < 32; i0 += 2 * kRowUnroll) {
-        if (i0 < np) {
-          u32x4 mm[kRowUnroll];
-#pragma unroll
-          for (int u = 0; u < kRowUnroll; ++u) {
-            const int ia = i0 + 2 * u, ib = ia + 1;
-            // pages past the slice reuse its first page: a valid address, result discarded
-            const int pa = __builtin_amdgcn_readlane(ids[pass / 2], lbase + ((ia < np) ? ia : 0));
-            const int pb = __builtin_amdgcn_readlane(ids[pass / 2], lbase + ((ib < np) ? ib : 0));
-            const int phys = half ? pb : pa;
-            mm[u] = __builtin_nontemporal_load((const u32x4*)(mbase + (size_t)phys * meta_stride));
-          }
-#pragma unroll
-          for (int u = 0; u < kRowUnroll; ++u) {
-            const int ia = i0 + 2 * u;
-            // words: x,y = min[4c..4c+3], z,w = max[4c..4c+3]; q > 0 takes the max, else the min
-            const uint32_t s0 = (mm[u].z & selmask[0]) | (mm[u].x & ~selmask[0]);
-            const uint32_t s1 = (mm[u].w & selmask[1]) | (mm[u].y & ~selmask[1]);
-            float acc;
-            if (QDT == TWL_F16) {
-              acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, s0),
-                                           __builtin_bit_cast(half2_t, qw[0]), 0.0f, false);
-              acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, s1),
-                                           __builtin_bit_cast(half2_t, qw[1]), acc, false);
-            } else {
-              acc = qf[0] * as_f32(s0 << 16);
-              acc = fmaf(qf[1], as_f32(s0 & 0xFFFF0000u), acc);
-              acc = fmaf(qf[2], as_f32(s1 << 16), acc);
-              acc = fmaf(qf[3], as_f32(s1 & 0xFFFF0000u), acc);
-            }
-            acc = row16_allreduce<OpSum>(acc);
-            acc += dpp<kDppBcast15, 0xA>(0.0f, acc);  // lanes 16..31 / 48..63 hold a page total
-            const float sa = as_f32(__builtin_amdgcn_readlane(as_i32(acc), 31));
-            const float sb = as_f32(__builtin_amdgcn_readlane(as_i32(acc), 63));
-            keep = (lane == ia) ? sa : keep;
-            keep = (lane == ia + 1) ? sb : keep;
-          }
+    for (int pass = 0; pass < PL_PASSES; ++pass) {
+      const int w0 = (pass * kRowWaves + wave) * 128;  // first page of this wave's slice
+      if (w0 < n_req) {                                // wave-uniform
+        const int pg0 = w0 + 2 * lane;                 // this lane's two pages
+        const int pgc = min(pg0, (int)a.plane_cap - 2);  // loads stay inside the run
+        float s0 = 0.0f, s1 = 0.0f;
+#pragma unroll 16
+        for (int d = 0; d < TWL_HEAD_DIM; ++d) {
+          const float qd =
+              as_f32(__builtin_amdgcn_readlane(as_i32(d < 64 ? q_lo : q_hi), d & 63));
+          const int plane = qd > 0.0f ? 1 : 0;         // max run for q_d > 0, else min run
+          const uint32_t w = __builtin_nontemporal_load(
+              (const uint32_t*)(pl + (size_t)(2 * d + plane) * a.plane_cap + pgc));
+          s0 = fmaf(qd, bits16_to_f32<QDT>(w & 0xFFFFu), s0);
+          s1 = fmaf(qd, bits16_to_f32<QDT>(w >> 16), s1);
+        }
+        if (pg0 < n_req) ps_lds[pg0] = s0;
+        if (pg0 + 1 < n_req) ps_lds[pg0 + 1] = s1;
+        if (a.page_scores_out) {
+          float* po = a.page_scores_out + (size_t)row * a.page_score_stride;
+          if (pg0 < n_req) po[pg0] = s0;
+          if (pg0 + 1 < n_req) po[pg0 + 1] = s1;
         }
       }
-      if (lane < np) {
-        ps_lds[p0 + lane] = keep;
-        if (a.page_scores_out)
-          a.page_scores_out[(size_t)row * a.page_score_stride + p0 + lane] = keep;
+    }
+  } else {
+    // page ids of all passes first: register r, lane l <-> pass 2r + l/32, page l%32 of the wave's
+    // 32-page slice of that pass
+    int ids[SEL_VPT];
+#pragma unroll
+    for (int r = 0; r < SEL_VPT; ++r) {
+      const int pg = ((2 * r + half) * kRowWaves + wave) * 32 + c;
+      ids[r] = (pg < n_req) ? a.f.kv_page_indices[pg_begin + pg] : 0;
+    }
+    float qf[4];
+    uint32_t selmask[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      qf[2 * j] = bits16_to_f32<QDT>(qw[j] & 0xFFFFu);
+      qf[2 * j + 1] = bits16_to_f32<QDT>(qw[j] >> 16);
+      selmask[j] = (qf[2 * j] > 0.0f ? 0x0000FFFFu : 0u) | (qf[2 * j + 1] > 0.0f ? 0xFFFF0000u : 0u);
+    }
+    const size_t meta_stride = (size_t)a.f.num_kv_heads * TWL_META_RECORD_BYTES;
+    const uint8_t* mbase = a.meta + (size_t)kvh * TWL_META_RECORD_BYTES + 16 * c;
+#pragma unroll
+    for (int pass = 0; pass < PASSES; ++pass) {
+      const int p0 = (pass * kRowWaves + wave) * 32;
+      const int np = min(32, n_req - p0);  // wave-uniform
+      if (np > 0) {
+        const int lbase = (pass & 1) * 32;
+        float keep = 0.0f;  // lane i ends up with the score of page p0 + i
+#pragma unroll
+        for (int i0 = 0; i0 < 32; i0 += 2 * kRowUnroll) {
+          if (i0 < np) {
+            u32x4 mm[kRowUnroll];
+#pragma unroll
+            for (int u = 0; u < kRowUnroll; ++u) {
+              const int ia = i0 + 2 * u, ib = ia + 1;
+              // pages past the slice reuse its first page: a valid address, result discarded
+              const int pa = __builtin_amdgcn_readlane(ids[pass / 2], lbase + ((ia < np) ? ia : 0));
+              const int pb = __builtin_amdgcn_readlane(ids[pass / 2], lbase + ((ib < np) ? ib : 0));
+              const int phys = half ? pb : pa;
+              mm[u] = __builtin_nontemporal_load((const u32x4*)(mbase + (size_t)phys * meta_stride));
+            }
+#pragma unroll
+            for (int u = 0; u < kRowUnroll; ++u) {
+              const int ia = i0 + 2 * u;
+              // words: x,y = min[4c..4c+3], z,w = max[4c..4c+3]; q > 0 takes the max, else the min
+              const uint32_t s0 = (mm[u].z & selmask[0]) | (mm[u].x & ~selmask[0]);
+              const uint32_t s1 = (mm[u].w & selmask[1]) | (mm[u].y & ~selmask[1]);
+              float acc;
+              if (QDT == TWL_F16) {
+                acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, s0),
+                                             __builtin_bit_cast(half2_t, qw[0]), 0.0f, false);
+                acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, s1),
+                                             __builtin_bit_cast(half2_t, qw[1]), acc, false);
+              } else {
+                acc = qf[0] * as_f32(s0 << 16);
+                acc = fmaf(qf[1], as_f32(s0 & 0xFFFF0000u), acc);
+                acc = fmaf(qf[2], as_f32(s1 << 16), acc);
+                acc = fmaf(qf[3], as_f32(s1 & 0xFFFF0000u), acc);
+              }
+              acc = row16_allreduce<OpSum>(acc);
+              acc += dpp<kDppBcast15, 0xA>(0.0f, acc);  // lanes 16..31 / 48..63 hold a page total
+              const float sa = as_f32(__builtin_amdgcn_readlane(as_i32(acc), 31));
+              const float sb = as_f32(__builtin_amdgcn_readlane(as_i32(acc), 63));
+              keep = (lane == ia) ? sa : keep;
+              keep = (lane == ia + 1) ? sb : keep;
+            }
+          }
+        }
+        if (lane < np) {
+          ps_lds[p0 + lane] = keep;
+          if (a.page_scores_out)
+            a.page_scores_out[(size_t)row * a.page_score_stride + p0 + lane] = keep;
+        }
       }
     }
   }
@@ -165,11 +206,11 @@ __global__ __launch_bounds__(kRowThreads) void select_estimate_prune_kernel(RowA
                                             sel_n, my_logical, qraw);
 }
 
-template <int QDT, int SEL_VPT>
+template <int QDT, int SEL_VPT, bool PLANES>
 static void launch_row(const RowArgs& a, uint32_t rows, hipStream_t s) {
   const uint32_t k = a.f.max_pages;
 #define TWL_ROW_CASE(V)                                                                         \
-  hipLaunchKernelGGL((select_estimate_prune_kernel<QDT, V, SEL_VPT>), dim3(rows),               \
+  hipLaunchKernelGGL((select_estimate_prune_kernel<QDT, V, SEL_VPT, PLANES>), dim3(rows),       \
                      dim3(kRowThreads), 0, s, a)
   if (k <= 64) TWL_ROW_CASE(1);
   else if (k <= 128) TWL_ROW_CASE(2);
@@ -189,8 +230,9 @@ extern "C" int twl_select_estimate_prune(
     uint32_t max_pages_per_req, float sm_scale, const float* p_arr, float p, int high_mode,
     int32_t* sel_pages, uint32_t sel_stride, int32_t* sel_count, int32_t* idx, uint32_t idx_stride,
     int32_t* count, float* page_scores_out, uint32_t page_score_stride, float* scores_out,
-    uint32_t score_stride, int32_t* cand_count, void* stream) {
-  if (!q || !meta || !k_int4 || !kv_page_indices || !kv_page_indptr || !kv_last_page_len ||
+    uint32_t score_stride, int32_t* cand_count, const void* meta_planes,
+    uint32_t plane_cap_pages, void* stream) {
+  if (!q || (!meta && !meta_planes) || !k_int4 || !kv_page_indices || !kv_page_indptr || !kv_last_page_len ||
       !sel_pages || !sel_count || !idx || !count)
     return TWL_ENULL;
   if (dtype != TWL_F16 && dtype != TWL_BF16) return TWL_EDTYPE;
@@ -207,8 +249,11 @@ extern "C" int twl_select_estimate_prune(
   if (high_mode != TWL_HIGH_FIRST && high_mode != TWL_HIGH_MAX) return TWL_EINVAL;
   if (!p_arr && !(p > 0.0f && p <= 1.0f)) return TWL_EINVAL;
   if ((((uintptr_t)q) & 15u) || (((uintptr_t)k_int4) & 15u) || (((uintptr_t)meta) & 15u) ||
-      (((uintptr_t)scores_out) & 3u) || (((uintptr_t)page_scores_out) & 3u))
+      (((uintptr_t)scores_out) & 3u) || (((uintptr_t)page_scores_out) & 3u) ||
+      (((uintptr_t)meta_planes) & 15u))
     return TWL_EALIGN;
+  if (meta_planes && (plane_cap_pages < max_pages_per_req || (plane_cap_pages & 7u)))
+    return TWL_EINVAL;
   twl::RowArgs a{};
   a.f.q = q; a.f.k_int4 = (const uint8_t*)k_int4; a.f.sel_stride = sel_stride;
   a.f.kv_page_indices = kv_page_indices; a.f.kv_page_indptr = kv_page_indptr;
@@ -220,15 +265,22 @@ extern "C" int twl_select_estimate_prune(
   a.meta = (const uint8_t*)meta; a.token_budget = token_budget;
   a.max_pages_req = max_pages_per_req; a.sel_pages_out = sel_pages; a.sel_count_out = sel_count;
   a.page_scores_out = page_scores_out; a.page_score_stride = page_score_stride;
+  a.planes = (const uint16_t*)meta_planes; a.plane_cap = plane_cap_pages;
   const uint32_t rows = batch * num_q_heads;
   hipStream_t s = (hipStream_t)stream;
   const bool small = max_pages_per_req <= 2048;
-  if (dtype == TWL_F16) {
-    if (small) twl::launch_row<TWL_F16, 2>(a, rows, s);
-    else twl::launch_row<TWL_F16, 8>(a, rows, s);
-  } else {
-    if (small) twl::launch_row<TWL_BF16, 2>(a, rows, s);
-    else twl::launch_row<TWL_BF16, 8>(a, rows, s);
-  }
+#define TWL_ROW_LAUNCH(DT)                                              \
+  do {                                                                  \
+    if (meta_planes) {                                                  \
+      if (small) twl::launch_row<DT, 2, true>(a, rows, s);              \
+      else twl::launch_row<DT, 8, true>(a, rows, s);                    \
+    } else {                                                            \
+      if (small) twl::launch_row<DT, 2, false>(a, rows, s);             \
+      else twl::launch_row<DT, 8, false>(a, rows, s);                   \
+    }                                                                   \
+  } while (0)
+  if (dtype == TWL_F16) TWL_ROW_LAUNCH(TWL_F16);
+  else TWL_ROW_LAUNCH(TWL_BF16);
+#undef TWL_ROW_LAUNCH
   return hipGetLastError() == hipSuccess ? TWL_OK : TWL_ELAUNCH;
 }

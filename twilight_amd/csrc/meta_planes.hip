@@ -1,0 +1,79 @@
+// Quest metadata in plane layout, for the selector's scoring pass.
+//
+// The page score of twilight/pyimpl/quest.py:37-84 in its min/max form is
+//     score(page) = sum_d q_d * (q_d > 0 ? max_d(page) : min_d(page)),
+// so for a given query only ONE of the two numbers kept per (page, channel) is ever read. The
+// 512-byte record layout (min and max of 4 channels side by side, records indexed by physical
+// page) forces both through memory. The plane layout stores, per (request slot, kv head, channel),
+// the minima of all pages of the request contiguously and the maxima contiguously,
+//     planes[slot][kv_head][d][0 = min, 1 = max][logical page],   16-bit values, `cap` pages,
+// so a row of the decode batch streams 128 runs of `pages` values — the min run or the max run of
+// each channel, chosen by the sign of q_d — and touches half the bytes. Planes are indexed by
+// LOGICAL page of a request slot (slot = position in the batch), not by physical page: they are a
+// per-request side buffer next to the paged K / V, updated by twl_kv_append.
+#include "twl_common.h"
+
+namespace twl {
+
+struct PlanesArgs {
+  const uint8_t* meta;   // records [pages, kv_heads, 512]
+  const int32_t* kv_page_indices;
+  const int32_t* kv_page_indptr;
+  uint32_t num_kv_heads;
+  uint16_t* planes;
+  uint32_t cap;          // pages per run
+};
+
+constexpr int kPlTile = 64;  // pages per workgroup
+
+// Records -> planes for the pages of the current page table. One workgroup per (64 logical pages,
+// kv head, request): the records go through LDS and leave as 128-byte runs per (channel, plane).
+__global__ __launch_bounds__(256) void meta_planes_build_kernel(PlanesArgs a) {
+  __shared__ uint16_t tile[kPlTile][256 + 2];  // +2: rows fall on different banks
+  const uint32_t b = blockIdx.z, kvh = blockIdx.y;
+  const int p0 = blockIdx.x * kPlTile;
+  const int pg_begin = a.kv_page_indptr[b];
+  const int n_pages = min(a.kv_page_indptr[b + 1] - pg_begin, (int)a.cap);
+  if (p0 >= n_pages) return;  // uniform
+  const int np = min(kPlTile, n_pages - p0);
+  const int tx = threadIdx.x;
+  // 64 records x 512 B = 2048 16-byte pieces, 8 per thread
+  for (int i = tx; i < np * 32; i += 256) {
+    const int pg = i >> 5, piece = i & 31;
+    const int phys = a.kv_page_indices[pg_begin + p0 + pg];
+    const u32x4 v = *(const u32x4*)(a.meta + ((size_t)phys * a.num_kv_heads + kvh) *
+                                                 TWL_META_RECORD_BYTES + 16 * piece);
+    uint32_t* dst = (uint32_t*)&tile[pg][8 * piece];
+    dst[0] = v.x; dst[1] = v.y; dst[2] = v.z; dst[3] = v.w;
+  }
+  __syncthreads();
+  const int lane = tx & 63, wave = tx >> 6;
+  uint16_t* out = a.planes + ((size_t)b * a.num_kv_heads + kvh) * (TWL_HEAD_DIM * 2) * a.cap;
+  // run r = d * 2 + plane; record element of (d, plane) = (d / 4) * 8 + plane * 4 + d % 4
+  for (int r = wave; r < TWL_HEAD_DIM * 2; r += 4) {
+    const int d = r >> 1, plane = r & 1;
+    const int col = (d >> 2) * 8 + plane * 4 + (d & 3);
+    if (lane < np) out[(size_t)r * a.cap + p0 + lane] = tile[lane][col];
+  }
+}
+
+}  // namespace twl
+
+extern "C" int twl_meta_planes_build(const void* meta, const int32_t* kv_page_indices,
+                                     const int32_t* kv_page_indptr, uint32_t batch,
+                                     uint32_t num_kv_heads, uint32_t max_pages_per_req,
+                                     void* planes, uint32_t plane_cap_pages, void* stream) {
+  if (!meta || !kv_page_indices || !kv_page_indptr || !planes) return TWL_ENULL;
+  if (batch == 0 || num_kv_heads == 0 || max_pages_per_req == 0) return TWL_EINVAL;
+  if (plane_cap_pages == 0 || (plane_cap_pages & 7u) || max_pages_per_req > plane_cap_pages)
+    return TWL_EINVAL;
+  if (batch > 65535u || num_kv_heads > 65535u) return TWL_EINVAL;
+  if ((((uintptr_t)meta) & 15u) || (((uintptr_t)planes) & 15u)) return TWL_EALIGN;
+  twl::PlanesArgs a{};
+  a.meta = (const uint8_t*)meta; a.kv_page_indices = kv_page_indices;
+  a.kv_page_indptr = kv_page_indptr; a.num_kv_heads = num_kv_heads;
+  a.planes = (uint16_t*)planes; a.cap = plane_cap_pages;
+  const dim3 grid((max_pages_per_req + twl::kPlTile - 1) / twl::kPlTile, num_kv_heads, batch);
+  hipLaunchKernelGGL(twl::meta_planes_build_kernel, grid, dim3(256), 0, (hipStream_t)stream, a);
+  return hipGetLastError() == hipSuccess ? TWL_OK : TWL_ELAUNCH;
+}

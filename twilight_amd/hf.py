@@ -108,7 +108,10 @@ def _fill_from_prefill(st: _LayerState, k: torch.Tensor, v: torch.Tensor, num_q_
     B, _, N, _ = k.shape
     npg = (N + PAGE - 1) // PAGE
     spare_per_req = (st.reserve_tokens + PAGE - 1) // PAGE + 1
-    st.cache = PagedKVCache.from_dense(k, v, k.device, spare_pages=B * spare_per_req)
+    # plane-layout metadata only where the one-launch selector can use it (no GQA sharing)
+    planes = npg + spare_per_req if k.shape[1] == num_q_heads else None
+    st.cache = PagedKVCache.from_dense(k, v, k.device, spare_pages=B * spare_per_req,
+                                       plane_pages=planes)
     st.free = list(range(B * npg, B * (npg + spare_per_req)))
     st.layer = TwilightDecodeLayer(st.cache, num_q_heads, reserve_pages=npg + spare_per_req, **st.cfg)
     st.seq_len = N

@@ -13,7 +13,7 @@ from .gemv import (batched_sparse_gemv, batched_sparse_gemv_int4_k, batched_spar
                    quest_gemv_int4_top_p)
 from .attention import attention_workspace_bytes, sparse_paged_decode_attention
 from .quest import quest_num_pages, quest_select
-from .kv_shadow import dequant_int4, kv_append, kv_shadow_build
+from .kv_shadow import dequant_int4, kv_append, kv_shadow_build, meta_planes_build
 from .label_ops import bgemv_int8, get_label_tensor, qk_int8_per_block
 
 __all__ = [
@@ -22,6 +22,6 @@ __all__ = [
     "single_sparse_gemv", "sparse_gemv_int4", "sparse_gemv_int4_top_p", "quest_gemv_int4_top_p",
     "sparse_paged_decode_attention",
     "attention_workspace_bytes",
-    "quest_num_pages", "quest_select", "dequant_int4", "kv_shadow_build", "kv_append",
+    "quest_num_pages", "quest_select", "dequant_int4", "kv_shadow_build", "kv_append", "meta_planes_build",
     "get_label_tensor", "bgemv_int8", "qk_int8_per_block",
 ]

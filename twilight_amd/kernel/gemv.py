@@ -163,11 +163,16 @@ def quest_gemv_int4_top_p(q: torch.Tensor, meta: torch.Tensor, k_int4: torch.Ten
                           kv_page_indices: torch.Tensor, kv_page_indptr: torch.Tensor,
                           kv_last_page_len: torch.Tensor, token_budget: int,
                           max_pages_per_req: int, top_p, high: str = "max",
-                          sm_scale: Optional[float] = None, return_scores: bool = False):
+                          sm_scale: Optional[float] = None, return_scores: bool = False,
+                          meta_planes: Optional[torch.Tensor] = None):
     """Selector + estimator + pruner in one launch, one workgroup per (batch, head) row:
     :func:`twilight_amd.kernel.quest_select` followed by :func:`sparse_gemv_int4_top_p`
     (twilight/pyimpl/quest.py:17-122, attention.py:252-255, top_p.py:10-15, attention.py:280-281)
     with the page scores and the page list kept on chip.
+
+    ``meta_planes`` [B,Hkv,128,2,cap] (:func:`twilight_amd.kernel.meta_planes_build`) makes the
+    page-score pass read the plane layout (half the bytes; scores may differ from the record form
+    in the last bits).
 
     Returns ``(sel_pages int32 [B,H,k], sel_count int32 [B,H], idx int32 [B,H,16k], count int32
     [B,H], cand_count int32 [B,H])``, k = budget pages clamped to ``max_pages_per_req``; with
@@ -206,8 +211,15 @@ def quest_gemv_int4_top_p(q: torch.Tensor, meta: torch.Tensor, k_int4: torch.Ten
     if M > _lib.MAX_CANDIDATES:
         raise RuntimeError(f"{M} candidates exceed the supported maximum {_lib.MAX_CANDIDATES}")
     p_arr, p_val = _check_p(top_p, B * H, q)
+    cap = 0
+    if meta_planes is not None:
+        from .kv_shadow import _check_planes
+        cap = _check_planes(meta_planes, B, Hkv, q.dtype)
+        if cap < max_pages_per_req:
+            raise RuntimeError("meta_planes holds fewer pages per request than max_pages_per_req")
     check_same_device(q, ("k_int4", k_int4), ("meta", meta), ("kv_page_indices", kv_page_indices),
-                      ("kv_page_indptr", kv_page_indptr), ("kv_last_page_len", kv_last_page_len))
+                      ("kv_page_indptr", kv_page_indptr), ("kv_last_page_len", kv_last_page_len),
+                      ("meta_planes", meta_planes))
     dev = q.device
     with torch.cuda.device(dev):
         sel = torch.zeros((B, H, k), dtype=torch.int32, device=dev)
@@ -225,7 +237,7 @@ def quest_gemv_int4_top_p(q: torch.Tensor, meta: torch.Tensor, k_int4: torch.Ten
             ptr(kv_page_indptr), ptr(kv_last_page_len), B, H, Hkv, int(token_budget),
             int(max_pages_per_req), scale, ptr(p_arr), p_val, _high_mode(high), ptr(sel), k,
             ptr(selc), ptr(idx), M, ptr(count), ptr(ps), max_pages_per_req, ptr(scores), M,
-            ptr(cand), stream_of(q))
+            ptr(cand), ptr(meta_planes), cap, stream_of(q))
     _lib.check(rc, "SelectEstimatePrune")
     out = [sel, selc, idx, count, cand]
     if return_scores:
