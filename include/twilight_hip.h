@@ -300,6 +300,14 @@ int twl_meta_planes_build(const void* meta, const int32_t* kv_page_indices,
                           const int32_t* kv_page_indptr, uint32_t batch, uint32_t num_kv_heads,
                           uint32_t max_pages_per_req, void* meta_planes, uint32_t plane_cap_pages,
                           void* stream);
+/* twl_quest_page_scores from the plane layout (one q head per row reads the runs its signs
+ * select: half the bytes of the record form; with GQA the q heads of a group do not share reads
+ * here, the record form does). Scores are accumulated channel by channel in ascending order. */
+int twl_quest_page_scores_planes(const void* q, int q_dtype, const void* meta_planes,
+                                 uint32_t plane_cap_pages, const int32_t* kv_page_indptr,
+                                 uint32_t batch, uint32_t num_q_heads, uint32_t num_kv_heads,
+                                 uint32_t max_pages_per_req, float* page_scores,
+                                 uint32_t score_stride, void* stream);
 
 /* Unpack INT4 shadow records to fp32: out [num_pages, num_kv_heads, 16, 128] (record order).
  * Exists so that tests can compare dequantised values bit for bit. */

@@ -239,6 +239,15 @@ def test_row_kernel_with_plane_metadata(dev, N, budget, H, dt):
     A = K.quest_gemv_int4_top_p(qd, cache.meta, cache.k_int4, *tab, budget, npg, p, return_scores=True)
     Bv = K.quest_gemv_int4_top_p(qd, cache.meta, cache.k_int4, *tab, budget, npg, p, return_scores=True,
                                  meta_planes=cache.meta_planes)
+    # the stand-alone plane scoring kernel does the same arithmetic as the row kernel's first phase
+    from twilight_amd import _lib
+    ps2 = torch.zeros((B, H, npg), dtype=torch.float32, device=dev)
+    rc = _lib.lib().twl_quest_page_scores_planes(
+        qd.data_ptr(), 0 if dt == torch.float16 else 1, cache.meta_planes.data_ptr(), cap,
+        cache.kv_page_indptr.data_ptr(), B, H, H, npg, ps2.data_ptr(), npg,
+        torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    assert torch.equal(ps2.view(torch.int32), Bv[5].view(torch.int32))
     selA, selcA, idxA, cntA, candA, psA, scA = [t.cpu() for t in A]
     selB, selcB, idxB, cntB, candB, psB, scB = [t.cpu() for t in Bv]
     assert torch.allclose(psA, psB, rtol=1e-5, atol=1e-4)

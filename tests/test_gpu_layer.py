@@ -22,13 +22,15 @@ def _lists_to_mask(idx, count, N):
     return m
 
 
-def _run_case(dev, B, H, Hkv, N, budget, p, dt, seed, shuffle=True, n_heavy=16, fused=True):
+def _run_case(dev, B, H, Hkv, N, budget, p, dt, seed, shuffle=True, n_heavy=16, fused=True,
+              planes=False):
     q, k, v = synth.heavy_hitter_qkv(B, H, N, n_heavy=n_heavy, mass=0.6, seed=seed, dtype=dt)
     group = H // Hkv
     kk, vv = k[:, ::group].contiguous(), v[:, ::group].contiguous()        # one K/V per kv head
     npg = (N + 15) // 16
     perm = torch.randperm(B * npg, generator=torch.Generator().manual_seed(seed)) if shuffle else None
-    cache = PagedKVCache.from_dense(kk.to(dt), vv.to(dt), dev, page_perm=perm)
+    cache = PagedKVCache.from_dense(kk.to(dt), vv.to(dt), dev, page_perm=perm,
+                                    plane_pages=npg if planes else None)
     layer = TwilightDecodeLayer(cache, H, token_budget=budget, top_p=p, high="max",
                                 fused_estimator=fused, keep_scores=True)
     out = layer(q[:, :, 0].to(dt).to(dev)).cpu().float()
@@ -95,6 +97,14 @@ def test_cfg1_full_context(dev, fused):
 @pytest.mark.parametrize("fused", [True, False])
 def test_small_layer_configs(dev, B, H, Hkv, N, budget, p, dt, fused):
     _run_case(dev, B, H, Hkv, N, budget, p, dt, seed=B * 100 + H, n_heavy=8, fused=fused)
+
+
+@pytest.mark.parametrize("B,H,N,budget", [
+    (2, 8, 2048, 512),       # 16 rows: separate launches, page scores from the plane layout
+    (8, 32, 1024, 256),      # 256 rows: the one-launch row kernel reading the plane layout
+])
+def test_layer_with_plane_metadata(dev, B, H, N, budget):
+    _run_case(dev, B, H, H, N, budget, 0.95, torch.float16, seed=B + N, n_heavy=8, planes=True)
 
 
 def test_decode_append_keeps_shadow_fresh(dev):

@@ -27,7 +27,7 @@ EXPORTS = (
     "twl_softmax_top_p_f32", "twl_gemv_top_p", "twl_select_estimate_prune", "twl_gemv_int4", "twl_gemv_int4_nhd",
     "twl_gemv_int8_nhd", "twl_gemv_f16_nhd", "twl_gemv_f16_single", "twl_sparse_attn",
     "twl_sparse_attn_workspace_bytes", "twl_quest_select",
-    "twl_quest_page_scores", "twl_quest_topk_pages", "twl_kv_shadow_build", "twl_kv_append", "twl_meta_planes_build", "twl_dequant_int4",
+    "twl_quest_page_scores", "twl_quest_topk_pages", "twl_kv_shadow_build", "twl_kv_append", "twl_meta_planes_build", "twl_quest_page_scores_planes", "twl_dequant_int4",
     "twl_decode_layer", "twl_get_label_tensor", "twl_bgemv_int8", "twl_qk_int8_lse",
 )
 
@@ -104,6 +104,7 @@ def lib() -> ctypes.CDLL:
     L.twl_kv_append.argtypes = [vp, vp, i32, u64, u64, vp, vp, u64, u64, u64, vp, vp, vp, u32, u32,
                                 vp, vp, vp, u32, vp]
     L.twl_meta_planes_build.argtypes = [vp, vp, vp, u32, u32, u32, vp, u32, vp]
+    L.twl_quest_page_scores_planes.argtypes = [vp, i32, vp, u32, vp, u32, u32, u32, u32, vp, u32, vp]
     i64 = ctypes.c_int64
     L.twl_qk_int8_lse.argtypes = [vp, vp, vp, vp, vp, u32, u32, u32, u32, u32, u32, i64, i64, i64,
                                   i64, i64, i64, vp]

@@ -92,11 +92,23 @@ extern "C" int twl_decode_layer(const twl_layer_args* a, void* stream) {
         a->plane_cap_pages, stream);
     if (rc != TWL_OK) return rc;
   } else {
-    // 1. Quest page scores + top-k pages
-    rc = twl_quest_select(a->q, a->dtype, a->meta, a->kv_page_indices, a->kv_page_indptr,
-                          a->batch, a->num_q_heads, a->num_kv_heads, a->token_budget,
-                          a->max_pages_per_req, a->sel_pages, a->sel_stride, a->sel_count,
-                          page_scores, ps_stride, stream);
+    // 1. Quest page scores + top-k pages; without GQA sharing the plane layout halves the read
+    if (a->meta_planes && a->num_q_heads == a->num_kv_heads &&
+        a->plane_cap_pages >= a->max_pages_per_req) {
+      rc = twl_quest_page_scores_planes(a->q, a->dtype, a->meta_planes, a->plane_cap_pages,
+                                        a->kv_page_indptr, a->batch, a->num_q_heads,
+                                        a->num_kv_heads, a->max_pages_per_req, page_scores,
+                                        ps_stride, stream);
+      if (rc != TWL_OK) return rc;
+      rc = twl_quest_topk_pages(page_scores, ps_stride, a->kv_page_indptr, a->batch,
+                                a->num_q_heads, a->token_budget, a->max_pages_per_req,
+                                a->sel_pages, a->sel_stride, a->sel_count, stream);
+    } else {
+      rc = twl_quest_select(a->q, a->dtype, a->meta, a->kv_page_indices, a->kv_page_indptr,
+                            a->batch, a->num_q_heads, a->num_kv_heads, a->token_budget,
+                            a->max_pages_per_req, a->sel_pages, a->sel_stride, a->sel_count,
+                            page_scores, ps_stride, stream);
+    }
     if (rc != TWL_OK) return rc;
     if (!a->split_estimator) {
       // 2+3. INT4 estimate, softmax, top-p and compaction in one launch

@@ -77,3 +77,89 @@ extern "C" int twl_meta_planes_build(const void* meta, const int32_t* kv_page_in
   hipLaunchKernelGGL(twl::meta_planes_build_kernel, grid, dim3(256), 0, (hipStream_t)stream, a);
   return hipGetLastError() == hipSuccess ? TWL_OK : TWL_ELAUNCH;
 }
+
+namespace twl {
+
+struct PlaneScoreArgs {
+  const void* q;
+  const uint16_t* planes;
+  uint32_t cap;
+  const int32_t* kv_page_indptr;
+  uint32_t num_q_heads, num_kv_heads;
+  uint32_t max_pages;
+  float* page_scores;
+  uint32_t score_stride;
+};
+
+constexpr int kPsThreads = 256;
+constexpr int kPsPagesPerBlock = 2 * kPsThreads;  // 2 pages per lane
+
+// Page scores of one (batch, q head) row from the plane layout: lane = 2 pages, the 128 channels
+// in ascending order, per channel the run (min or max) that the sign of q_d selects. The same
+// arithmetic as the scoring phase of select_estimate_prune_kernel, as a kernel of its own for the
+// batch sizes where the stages run as separate launches.
+template <int DT>
+__global__ __launch_bounds__(kPsThreads) void quest_score_planes_kernel(PlaneScoreArgs a) {
+  const uint32_t row = blockIdx.y;
+  const uint32_t b = row / a.num_q_heads;
+  const uint32_t h = row - b * a.num_q_heads;
+  const uint32_t kvh = h / (a.num_q_heads / a.num_kv_heads);
+  const int lane = lane_id();
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int n_req = min(max(a.kv_page_indptr[b + 1] - a.kv_page_indptr[b], 0),
+                        min((int)a.max_pages, (int)a.cap));
+  const int w0 = blockIdx.x * kPsPagesPerBlock + wave * 128;
+  if (w0 >= n_req) return;
+  const uint16_t* qrow = (const uint16_t*)a.q + (size_t)row * TWL_HEAD_DIM;
+  const float q_lo = bits16_to_f32<DT>(qrow[lane]);
+  const float q_hi = bits16_to_f32<DT>(qrow[64 + lane]);
+  const uint16_t* pl = a.planes + ((size_t)b * a.num_kv_heads + kvh) * (TWL_HEAD_DIM * 2) * a.cap;
+  const int pg0 = w0 + 2 * lane;
+  const int pgc = min(pg0, (int)a.cap - 2);
+  float s0 = 0.0f, s1 = 0.0f;
+#pragma unroll 16
+  for (int d = 0; d < TWL_HEAD_DIM; ++d) {
+    const float qd = as_f32(__builtin_amdgcn_readlane(as_i32(d < 64 ? q_lo : q_hi), d & 63));
+    const int plane = qd > 0.0f ? 1 : 0;
+    const uint32_t w = __builtin_nontemporal_load(
+        (const uint32_t*)(pl + (size_t)(2 * d + plane) * a.cap + pgc));
+    s0 = fmaf(qd, bits16_to_f32<DT>(w & 0xFFFFu), s0);
+    s1 = fmaf(qd, bits16_to_f32<DT>(w >> 16), s1);
+  }
+  float* po = a.page_scores + (size_t)row * a.score_stride;
+  if (pg0 < n_req) po[pg0] = s0;
+  if (pg0 + 1 < n_req) po[pg0 + 1] = s1;
+}
+
+}  // namespace twl
+
+extern "C" int twl_quest_page_scores_planes(const void* q, int q_dtype, const void* meta_planes,
+                                            uint32_t plane_cap_pages,
+                                            const int32_t* kv_page_indptr, uint32_t batch,
+                                            uint32_t num_q_heads, uint32_t num_kv_heads,
+                                            uint32_t max_pages_per_req, float* page_scores,
+                                            uint32_t score_stride, void* stream) {
+  if (!q || !meta_planes || !kv_page_indptr || !page_scores) return TWL_ENULL;
+  if (q_dtype != TWL_F16 && q_dtype != TWL_BF16) return TWL_EDTYPE;
+  if (batch == 0 || num_q_heads == 0 || num_kv_heads == 0 || num_q_heads % num_kv_heads != 0)
+    return TWL_EINVAL;
+  if (max_pages_per_req == 0 || max_pages_per_req > 16384 || score_stride < max_pages_per_req)
+    return TWL_EINVAL;
+  if (plane_cap_pages < max_pages_per_req || (plane_cap_pages & 7u)) return TWL_EINVAL;
+  if ((uint64_t)batch * num_q_heads > 65535u) return TWL_EINVAL;
+  if ((((uintptr_t)q) & 1u) || (((uintptr_t)meta_planes) & 15u) || (((uintptr_t)page_scores) & 3u))
+    return TWL_EALIGN;
+  twl::PlaneScoreArgs a{};
+  a.q = q; a.planes = (const uint16_t*)meta_planes; a.cap = plane_cap_pages;
+  a.kv_page_indptr = kv_page_indptr; a.num_q_heads = num_q_heads; a.num_kv_heads = num_kv_heads;
+  a.max_pages = max_pages_per_req; a.page_scores = page_scores; a.score_stride = score_stride;
+  const dim3 grid((max_pages_per_req + twl::kPsPagesPerBlock - 1) / twl::kPsPagesPerBlock,
+                  batch * num_q_heads);
+  if (q_dtype == TWL_F16)
+    hipLaunchKernelGGL((twl::quest_score_planes_kernel<TWL_F16>), grid, dim3(twl::kPsThreads), 0,
+                       (hipStream_t)stream, a);
+  else
+    hipLaunchKernelGGL((twl::quest_score_planes_kernel<TWL_BF16>), grid, dim3(twl::kPsThreads), 0,
+                       (hipStream_t)stream, a);
+  return hipGetLastError() == hipSuccess ? TWL_OK : TWL_ELAUNCH;
+}
