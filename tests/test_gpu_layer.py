@@ -107,6 +107,25 @@ def test_layer_with_plane_metadata(dev, B, H, N, budget):
     _run_case(dev, B, H, H, N, budget, 0.95, torch.float16, seed=B + N, n_heavy=8, planes=True)
 
 
+def test_layer_at_128k_context(dev):
+    # 8192 pages per request: the widest selector shapes (8 pages per thread in the radix select,
+    # four scoring passes over the plane layout), 512 selected pages, against the dense oracle
+    _run_case(dev, 1, 4, 4, 131072, 8192, 0.95, torch.float16, seed=77, n_heavy=12, planes=True)
+    from twilight_amd.cache import PagedKVCache as C
+    g = torch.Generator().manual_seed(78)
+    k = torch.randn((1, 2, 131072, 128), generator=g).half()
+    cache = C.from_dense(k, k, dev, plane_pages=8192)
+    q = torch.randn((1, 2, 128), generator=g).half().to(dev)
+    tab = (cache.kv_page_indices, cache.kv_page_indptr, cache.kv_last_page_len)
+    import twilight_amd.kernel as K
+    a = K.quest_gemv_int4_top_p(q, cache.meta, cache.k_int4, *tab, 8192, 8192, 0.9, return_scores=True,
+                                meta_planes=cache.meta_planes)
+    sel, selc, ps = K.quest_select(q, cache.meta, *tab[:2], 8192, 8192)
+    assert torch.allclose(a[5], ps, rtol=1e-5, atol=1e-4)                  # page scores: planes vs records
+    same = [set(a[0][0, h].tolist()) == set(sel[0, h].tolist()) for h in range(2)]
+    assert all(same) or int(selc.min()) == 512
+
+
 def test_decode_append_keeps_shadow_fresh(dev):
     # append tokens one at a time (crossing a page boundary) and compare with a cache built at once
     g = torch.Generator().manual_seed(0)
