@@ -53,6 +53,7 @@ __global__ __launch_bounds__(kRowThreads) void select_estimate_prune_kernel(RowA
   __shared__ float ps_lds[kRowThreads * SEL_VPT];
   __shared__ int32_t sel_lds[kRowWaves * PW];
 
+  select_smem_init<kRowThreads>(ssm);  // the barrier after the scoring phase orders it
   const uint32_t row = blockIdx.x;
   const uint32_t b = row / a.f.num_q_heads;
   const uint32_t h = row - b * a.f.num_q_heads;

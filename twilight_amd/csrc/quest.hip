@@ -54,6 +54,8 @@ __device__ __forceinline__ void quest_select_row(const QuestArgs& a, uint32_t ro
 template <int THREADS, int VPT>
 __global__ __launch_bounds__(THREADS) void quest_select_kernel(QuestArgs a) {
   __shared__ SelSmem sm;
+  select_smem_init<THREADS>(sm);
+  __syncthreads();
   quest_select_row<THREADS, VPT>(a, blockIdx.x, sm);
 }
 

@@ -14,10 +14,19 @@ __device__ __forceinline__ int quest_budget_pages(uint32_t token_budget) {
 }
 
 struct SelSmem {
-  int hist[256];
-  int pick[2];       // chosen digit, remaining k
+  int hist[4][256];  // one histogram per radix pass (at most 4 x 8 bits), zeroed by select_smem_init
+  int pick[4][2];    // per pass: chosen digit, remaining k
+  int scr[32];       // per-wave key maxima / minima
   int wave_tot[16];
 };
+
+// Zero the histograms. Every thread of the workgroup calls it, and a barrier must lie between this
+// call and select_row_topk (any barrier of the caller will do: the select itself then needs no
+// barrier for clearing).
+template <int THREADS>
+__device__ __forceinline__ void select_smem_init(SelSmem& sm) {
+  for (int i = threadIdx.x; i < 4 * 256; i += THREADS) (&sm.hist[0][0])[i] = 0;
+}
 
 __device__ __forceinline__ uint32_t order_key(float f) {
   const uint32_t u = as_u32(f);
@@ -84,32 +93,31 @@ __device__ __forceinline__ void select_row_topk(const float* src, int n_pages, i
     kmin = min(kmin, (uint32_t)dpp<kDppBcast31, 0xC>((int)0xFFFFFFFF, (int)kmin));
   }
   if (lane == kWave - 1) {
-    sm.hist[wave] = (int)kmax;
-    sm.hist[16 + wave] = (int)kmin;
+    sm.scr[wave] = (int)kmax;
+    sm.scr[16 + wave] = (int)kmin;
   }
   __syncthreads();
   kmax = 0u; kmin = 0xFFFFFFFFu;
 #pragma unroll
   for (int w = 0; w < NWAVES; ++w) {
-    kmax = max(kmax, (uint32_t)sm.hist[w]);
-    kmin = min(kmin, (uint32_t)sm.hist[16 + w]);
+    kmax = max(kmax, (uint32_t)sm.scr[w]);
+    kmin = min(kmin, (uint32_t)sm.scr[16 + w]);
   }
-  __syncthreads();  // hist is reused below
   const uint32_t diff = kmax ^ kmin;
   int top = diff ? 32 - __builtin_clz(diff) : 0;  // low bits in which keys of the row may differ
   uint32_t prefix_mask = top >= 32 ? 0u : ~((1u << top) - 1u);
   uint32_t prefix = kmax & prefix_mask;
   int k_rem = k;
+  int pass = 0;
   while (top > 0) {
     const int bits = min(8, top);
     const int shift = top - bits;
     const uint32_t dmask = (1u << bits) - 1u;
-    for (int i = tx; i < 256; i += THREADS) sm.hist[i] = 0;
-    __syncthreads();
+    int (&hist)[256] = sm.hist[pass];  // zeroed by select_smem_init
 #pragma unroll
     for (int j = 0; j < VPT; ++j) {
       if ((key[j] & prefix_mask) == prefix && key[j] != 0u)
-        atomicAdd(&sm.hist[(key[j] >> shift) & dmask], 1);
+        atomicAdd(&hist[(key[j] >> shift) & dmask], 1);
     }
     __syncthreads();
     if (wave == 0) {
@@ -118,7 +126,7 @@ __device__ __forceinline__ void select_row_topk(const float* src, int n_pages, i
       int mine = 0;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        hcnt[j] = sm.hist[255 - 4 * lane - j];
+        hcnt[j] = hist[255 - 4 * lane - j];
         mine += hcnt[j];
       }
       const int incl = wave_inclusive_scan(mine);
@@ -127,18 +135,19 @@ __device__ __forceinline__ void select_row_topk(const float* src, int n_pages, i
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           if (run < k_rem && k_rem <= run + hcnt[j]) {
-            sm.pick[0] = 255 - 4 * lane - j;
-            sm.pick[1] = k_rem - run;
+            sm.pick[pass][0] = 255 - 4 * lane - j;
+            sm.pick[pass][1] = k_rem - run;
           }
           run += hcnt[j];
         }
       }
     }
     __syncthreads();
-    prefix |= (uint32_t)sm.pick[0] << shift;
+    prefix |= (uint32_t)sm.pick[pass][0] << shift;
     prefix_mask |= dmask << shift;
-    k_rem = sm.pick[1];
+    k_rem = sm.pick[pass][1];
     top = shift;
+    ++pass;
   }
   const uint32_t T = prefix;  // k-th largest key; k_rem of the keys equal to T are taken
 
