@@ -29,7 +29,10 @@
  *     g = d/32. Dequantised value = float(nibble) * float(scale) + float(zero), one fp32 rounding.
  *   - Quest page metadata: one 512-byte record per (physical page, kv head), ordered
  *     [page][kv_head]: 32 chunks of 16 bytes; chunk c holds fp16 min[4c..4c+3] then fp16
- *     max[4c..4c+3] over the valid tokens of the page.
+ *     max[4c..4c+3] over the valid tokens of the page ("fp16" = the cache dtype, fp16 or bf16).
+ *   - Quest page metadata, plane layout (optional second copy, see twl_meta_planes_build):
+ *     planes[slot][kv_head][d][0 = min, 1 = max][logical page], 16-bit values in the cache dtype,
+ *     plane_cap_pages pages per run, slot = position of the request in the batch.
  *   - Paged K / V caches: fp16 or bf16, addressed with explicit element strides
  *     (page, token, kv head); head_dim is contiguous.
  */
