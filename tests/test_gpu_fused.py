@@ -268,3 +268,59 @@ def test_row_kernel_with_plane_metadata(dev, N, budget, H, dt):
                 assert int(cntA[b, h]) == int(cntB[b, h])
                 assert torch.equal(idxA[b, h, :cntA[b, h]], idxB[b, h, :cntB[b, h]])
     assert same_rows >= B * H - 1
+
+
+@pytest.mark.parametrize("planes", [False, True])
+def test_row_kernel_ragged_batch(dev, planes):
+    """Requests of different lengths in one batch (one with a partial last page, one of a single
+    page, one shorter than the budget): the one-launch kernel against quest_select + gemv_top_p."""
+    from twilight_amd.cache import PagedKVCache
+    H, N, p, budget = 4, 2000, 0.9, 480
+    lens = [2000, 597, 16, 333]                       # tokens per request
+    B = len(lens)
+    g = torch.Generator().manual_seed(12)
+    q = torch.randn((B, H, 128), generator=g)
+    k = torch.randn((B, H, N, 128), generator=g)
+    for b in range(B):
+        for h in range(H):
+            pos = torch.randint(0, lens[b], (4,), generator=g)
+            k[b, h, pos] += q[b, h] * 0.5
+    npg = N // 16
+    full = PagedKVCache.from_dense(k.half(), k.half(), dev,
+                                   page_perm=torch.randperm(B * npg, generator=g))
+    phys = full.kv_page_indices.cpu().reshape(B, npg)
+    pages = [(n + 15) // 16 for n in lens]
+    ids = torch.cat([phys[b, :pages[b]] for b in range(B)])
+    indptr = torch.tensor([0] + list(np.cumsum(pages)), dtype=torch.int32)
+    last = torch.tensor([n - (pg - 1) * 16 for n, pg in zip(lens, pages)], dtype=torch.int32)
+    full.set_page_table(ids, indptr, last)
+    # last pages now hold fewer valid tokens: refresh their records
+    last_pages = torch.stack([phys[b, pages[b] - 1] for b in range(B)]).to(torch.int32).to(dev)
+    full.rebuild_shadow(last_pages, last.to(dev))
+    if planes:
+        full.enable_planes()
+    qd = q.half().to(dev)
+    tab = (full.kv_page_indices, full.kv_page_indptr, full.kv_last_page_len)
+    mp = max(pages)
+    selA, selcA, psA = K.quest_select(qd, full.meta, tab[0], tab[1], budget, mp)
+    kk = selA.shape[-1]
+    idxA, cntA, candA = K.sparse_gemv_int4_top_p(qd, full.k_int4, *tab, selA, selcA, p, max_pages=kk)
+    selB, selcB, idxB, cntB, candB = K.quest_gemv_int4_top_p(
+        qd, full.meta, full.k_int4, *tab, budget, mp, p, meta_planes=full.meta_planes)
+    assert torch.equal(selcA, selcB) and torch.equal(candA, candB)
+    want_k = [min(kk, pg) for pg in pages]
+    assert selcB.cpu()[:, 0].tolist() == want_k
+    # candidates of the last page stop at the request's length
+    assert candB.cpu()[:, 0].tolist() == [16 * w for w in want_k]
+    differ = 0
+    for b in range(B):
+        for h in range(H):
+            n = want_k[b]
+            if not torch.equal(selA[b, h, :n], selB[b, h, :n]):
+                differ += 1
+                continue
+            ca, cb = int(cntA[b, h]), int(cntB[b, h])
+            same = ca == cb and torch.equal(idxA[b, h, :ca], idxB[b, h, :cb])
+            differ += 0 if same else 1
+            assert int(idxB[b, h, :cb].max()) < lens[b]        # nothing past the request's end
+    assert differ <= 1
