@@ -389,11 +389,13 @@ typedef struct twl_layer_args {
   void* attn_workspace; uint64_t attn_workspace_bytes; /* see twl_sparse_attn */
   /* output */
   void* out;                /* [batch, num_q_heads, 128], dtype */
-  /* 0 = fused: with one q head per kv head, at most one row per compute unit pair and
-   * <= 8192 pages per request the selector, estimator and pruner are ONE launch
-   * (twl_select_estimate_prune), otherwise twl_quest_select + twl_gemv_top_p; 1 = every stage its
-   * own launch (twl_quest_select, twl_gemv_int4, twl_softmax_top_p_f32). In fused mode `scores`
-   * and `page_scores` are filled only when keep_scores != 0. */
+  /* 0 = let the library choose by batch shape: with one q head per kv head, between half a row
+   * and two rows per compute unit and <= 8192 pages per request the selector, estimator and
+   * pruner are ONE launch (twl_select_estimate_prune); with fewer rows than half the compute
+   * units every stage is its own launch (the estimator needs more workgroups than rows);
+   * otherwise twl_quest_select + twl_gemv_top_p. 1 = always every stage its own launch
+   * (twl_quest_select, twl_gemv_int4, twl_softmax_top_p_f32). The results are the same either
+   * way; with 0, `scores` and `page_scores` are guaranteed filled only when keep_scores != 0. */
   int split_estimator;
   int keep_scores;
 } twl_layer_args;

@@ -38,8 +38,10 @@ struct GemvArgs {
 // launch shape, chosen by sweeps over (threads, pages per wave, unroll) at 8 x 32 x 32768 and
 // 8 x 32 x 8192 candidates
 constexpr int kGemvThreads = 256;       // 4 wavefronts
-constexpr int kGemvPagesPerWave = 64;   // <= 64: one lane per page id
-constexpr int kGemvPagesPerBlock = kGemvPagesPerWave * (kGemvThreads / kWave);
+// pages per wavefront (<= 64: one lane per page id): 64 when the grid fills the chip anyway (long
+// runs, few large store bursts); 16 or 8 for small batches, where a wavefront's groups of four
+// pages are serial memory round trips and the launch needs more wavefronts, not longer ones
+constexpr int kGemvPagesPerWave = 64;
 constexpr int kGemvUnroll = 4;          // pages in flight per wavefront
 
 // 8 nibbles of one dword against 8 q values held as 4 half2 pairs (n0,n4),(n1,n5),(n2,n6),(n3,n7).
@@ -76,17 +78,18 @@ __device__ __forceinline__ float page_partial(const u32x4& nib, uint32_t sz, con
 
 // HAS_SEL: the row has its own page list (sel_pages / sel_count); otherwise every page of the
 // request is a candidate.
-template <int QDT, bool HAS_SEL>
+template <int QDT, bool HAS_SEL, int PW>
 __global__ __launch_bounds__(kGemvThreads) void gemv_int4_kernel(GemvArgs a) {
   constexpr int U = kGemvUnroll;
-  constexpr int G = kGemvPagesPerWave / U;  // load groups per wavefront
+  constexpr int G = PW / U;  // load groups per wavefront
+  static_assert(PW % U == 0 && PW <= 64, "one lane per page id, whole groups");
   const uint32_t row = blockIdx.y;
   const uint32_t b = row / a.num_q_heads;
   const uint32_t h = row - b * a.num_q_heads;
   const uint32_t kvh = h / (a.num_q_heads / a.num_kv_heads);
   const int lane = lane_id();
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-  const int p0 = blockIdx.x * kGemvPagesPerBlock + wave * kGemvPagesPerWave;
+  const int p0 = (blockIdx.x * (kGemvThreads / kWave) + wave) * PW;
 
   // everything that depends only on the kernel arguments is requested at once
   const int pg_begin = a.kv_page_indptr[b];
@@ -96,7 +99,7 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_int4_kernel(GemvArgs a) {
   int my_logical = p0 + lane;
   if (HAS_SEL) {
     // read ahead of the count: the slot exists whenever it is inside the row's stride
-    my_logical = (lane < kGemvPagesPerWave && (uint32_t)(p0 + lane) < a.sel_stride)
+    my_logical = (lane < PW && (uint32_t)(p0 + lane) < a.sel_stride)
                      ? a.sel_pages[(size_t)row * a.sel_stride + p0 + lane] : 0;
   }
   const int g = lane & 3;
@@ -114,7 +117,7 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_int4_kernel(GemvArgs a) {
   if (req_pages <= 0) n_pages = 0;
   if (blockIdx.x == 0 && threadIdx.x == 0 && a.out_count) a.out_count[row] = n_pages * TWL_PAGE;
   if (p0 >= n_pages) return;
-  const int np = min(kGemvPagesPerWave, n_pages - p0);
+  const int np = min(PW, n_pages - p0);
 
   // ---- page ids of this wave's run: lane i owns run entry i ---------------------------------
   my_logical = min(max(my_logical, 0), req_pages - 1);  // a corrupt list must not leave the table
@@ -195,6 +198,16 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_int4_kernel(GemvArgs a) {
     if (grp * U + (lane >> 4) < np) orow[grp * U * TWL_PAGE + lane] = held[grp];
 }
 
+template <int QDT, bool HAS_SEL>
+static void launch_gemv(const GemvArgs& a, uint32_t rows, int pw, hipStream_t st) {
+  const dim3 blk(kGemvThreads);
+  const uint32_t per_block = (uint32_t)pw * (kGemvThreads / kWave);
+  const dim3 grid((a.max_pages + per_block - 1) / per_block, rows);
+  if (pw == 64) hipLaunchKernelGGL((gemv_int4_kernel<QDT, HAS_SEL, 64>), grid, blk, 0, st, a);
+  else if (pw == 16) hipLaunchKernelGGL((gemv_int4_kernel<QDT, HAS_SEL, 16>), grid, blk, 0, st, a);
+  else hipLaunchKernelGGL((gemv_int4_kernel<QDT, HAS_SEL, 8>), grid, blk, 0, st, a);
+}
+
 }  // namespace twl
 
 extern "C" int twl_gemv_int4(const void* q, int q_dtype, float* out, uint32_t out_stride,
@@ -222,16 +235,24 @@ extern "C" int twl_gemv_int4(const void* q, int q_dtype, float* out, uint32_t ou
   a.sel_stride = sel_stride; a.kv_page_indices = kv_page_indices; a.kv_page_indptr = kv_page_indptr;
   a.kv_last_page_len = kv_last_page_len; a.num_q_heads = num_q_heads;
   a.num_kv_heads = num_kv_heads; a.max_pages = max_pages_per_row; a.sm_scale = sm_scale;
-  const uint32_t gx = (max_pages_per_row + twl::kGemvPagesPerBlock - 1) / twl::kGemvPagesPerBlock;
-  dim3 grid(gx, batch * num_q_heads);
-  const dim3 blk(twl::kGemvThreads);
+  const uint32_t rows = batch * num_q_heads;
   hipStream_t st = (hipStream_t)stream;
+  // enough wavefronts to give every SIMD of the chip two: shorter runs when the batch is small
+  const uint64_t row_pages = (uint64_t)rows * max_pages_per_row;
+  int cus = 256;
+  (void)twl::device_cu_count(&cus);
+  const uint64_t want_waves = 8ull * (uint64_t)cus;
+#ifdef TWL_GEMV_PW
+  const int pw = TWL_GEMV_PW;
+#else
+  const int pw = row_pages / 64 >= want_waves ? 64 : (row_pages / 16 >= want_waves ? 16 : 8);
+#endif
   if (q_dtype == TWL_F16) {
-    if (sel_pages) hipLaunchKernelGGL((twl::gemv_int4_kernel<TWL_F16, true>), grid, blk, 0, st, a);
-    else hipLaunchKernelGGL((twl::gemv_int4_kernel<TWL_F16, false>), grid, blk, 0, st, a);
+    if (sel_pages) twl::launch_gemv<TWL_F16, true>(a, rows, pw, st);
+    else twl::launch_gemv<TWL_F16, false>(a, rows, pw, st);
   } else {
-    if (sel_pages) hipLaunchKernelGGL((twl::gemv_int4_kernel<TWL_BF16, true>), grid, blk, 0, st, a);
-    else hipLaunchKernelGGL((twl::gemv_int4_kernel<TWL_BF16, false>), grid, blk, 0, st, a);
+    if (sel_pages) twl::launch_gemv<TWL_BF16, true>(a, rows, pw, st);
+    else twl::launch_gemv<TWL_BF16, false>(a, rows, pw, st);
   }
   return hipGetLastError() == hipSuccess ? TWL_OK : TWL_ELAUNCH;
 }

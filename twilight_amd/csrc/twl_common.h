@@ -141,5 +141,32 @@ __device__ __forceinline__ int wave_inclusive_scan(int v) {
   return v;
 }
 
+// compute units of the current device, looked up once per device (the only process-wide state of
+// the library; written with relaxed atomics, any racing writers store the same value)
+inline int device_cu_count(int* out) {
+  static int cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) {
+    (void)hipGetLastError();
+    return TWL_ENODEVICE;
+  }
+  if (dev >= 0 && dev < 64) {
+    const int c = __atomic_load_n(&cached[dev], __ATOMIC_RELAXED);
+    if (c > 0) {
+      *out = c;
+      return TWL_OK;
+    }
+  }
+  int n = 0;
+  if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+    (void)hipGetLastError();
+    return TWL_ENODEVICE;
+  }
+  if (dev >= 0 && dev < 64) __atomic_store_n(&cached[dev], n, __ATOMIC_RELAXED);
+  *out = n;
+  return TWL_OK;
+}
+
+
 }  // namespace twl
 #endif  // TWL_COMMON_H_
