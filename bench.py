@@ -284,6 +284,12 @@ def main() -> int:
                 B, H, Hkv, sm, 0, p(l.attn_workspace), l.attn_workspace.numel(), stream)),
                 int(rows * n_bar) * (2 * D * 2 + 4) + rows * D * 4),
         }
+        if layers[0].cache.meta_planes is not None and H == Hkv:
+            calls["quest_score_planes"] = (rotating(
+                lambda l, c, q: lambda: L.twl_quest_page_scores_planes(
+                    p(q), qcode, p(c.meta_planes), c.meta_planes.size(4), p(c.kv_page_indptr),
+                    B, H, Hkv, npg, p(l.page_scores), npg, stream)),
+                rows * npg * 512 + rows * npg * 4 + rows * D * 2)
         for name, (fn, nbytes) in calls.items():
             us = _time_calls(fn, it, wu)
             kernels[name] = {"us": round(us, 2), "bytes": nbytes,
@@ -292,41 +298,48 @@ def main() -> int:
         if layers[0].cache.meta_planes is not None:
             # `bytes` above is the algorithm's figure (512 B of min/max metadata per row and
             # page); with the plane layout the kernel reads only the sign-selected half of it
-            k = kernels["select_estimate_prune"]
-            k["bytes_read_by_design"] = k["bytes"] - rows * npg * 256
-            k["GBps_read_by_design"] = round(k["bytes_read_by_design"] / k["us"] / 1e3, 1)
+            for name in ("select_estimate_prune", "quest_score_planes"):
+                k = kernels.get(name)
+                if k:
+                    k["bytes_read_by_design"] = k["bytes"] - rows * npg * 256
+                    k["GBps_read_by_design"] = round(k["bytes_read_by_design"] / k["us"] / 1e3, 1)
 
     # the kernels one layer step launches (the choice twl_decode_layer makes)
     cus = torch.cuda.get_device_properties(dev).multi_processor_count
-    row_kernel = (not args.split_estimator and H == Hkv and npg <= 8192
-                  and 2 * rows >= cus and rows <= 2 * cus)
-    if args.split_estimator:
-        used = ("quest_score", "quest_topk", "gemv_int4", "softmax_top_p", "sparse_attn")
+    split = args.split_estimator or 2 * rows < cus
+    row_kernel = (not split and H == Hkv and npg <= 8192 and rows <= 2 * cus)
+    score = ("quest_score_planes" if layers[0].cache.meta_planes is not None and H == Hkv
+             else "quest_score")
+    if split:
+        used = (score, "quest_topk", "gemv_int4", "softmax_top_p", "sparse_attn")
     elif row_kernel:
         used = ("select_estimate_prune", "sparse_attn")
     else:
-        used = ("quest_score", "quest_topk", "gemv_top_p", "sparse_attn")
+        used = (score, "quest_topk", "gemv_top_p", "sparse_attn")
     for name in kernels:
         kernels[name]["in_layer_step"] = name in used
     layer_bytes = sum(kernels[n]["bytes"] for n in used) if kernels else None
     # dominant kernel of the step: the one-launch selector + estimator + pruner when the step
     # uses it, else the metadata stream
-    dom_name = "select_estimate_prune" if (kernels and "select_estimate_prune" in used) else "quest_score"
+    dom_name = "select_estimate_prune" if (kernels and "select_estimate_prune" in used) else score
     dom = kernels.get(dom_name)
     roofline = None
     if dom:
         default_cfg = (B, N, args.budget, llama) == (8, 32768, 8192, False)
         traffic = None
         if default_cfg:
-            if dom_name != "select_estimate_prune":
+            if dom_name == "quest_score":
                 traffic = QUEST_SCORE_TRAFFIC_BYTES_DEFAULT
+            elif dom_name == "quest_score_planes":
+                traffic = None  # not measured for this kernel
             elif layers[0].cache.meta_planes is not None:
                 traffic = ROW_KERNEL_TRAFFIC_BYTES_DEFAULT
             else:
                 traffic = ROW_KERNEL_TRAFFIC_BYTES_RECORDS
         roofline = {"bound": "hbm",
                     "kernel": ("select_estimate_prune_kernel" if dom_name == "select_estimate_prune"
-                               else "quest_score_kernel"),
+                               else ("quest_score_planes_kernel" if dom_name == "quest_score_planes"
+                                     else "quest_score_kernel")),
                     "achieved": dom["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                     "frac": dom["frac_of_hbm_peak"], "bytes_per_launch": dom["bytes"],
                     "us_per_launch": dom["us"], "traffic": traffic}
