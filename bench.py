@@ -203,7 +203,7 @@ def main() -> int:
         cache.k_cache, cache.v_cache = k, v
         cache.set_page_table(ids, indptr, last)
         cache.rebuild_shadow()
-        if not llama and not args.no_planes:
+        if not args.no_planes:
             cache.enable_planes()      # metadata also in plane layout: the row kernel reads half
         layers.append(TwilightDecodeLayer(cache, H, token_budget=args.budget, top_p=args.top_p,
                                           high="max", fused_estimator=not args.split_estimator))
@@ -266,7 +266,7 @@ def main() -> int:
                 p(l.sel_pages), kp, p(l.sel_count), p(l.idx), M, p(l.count), 0, 0, 0, M,
                 p(l.cand_count), p(c.meta_planes),
                 0 if c.meta_planes is None else c.meta_planes.size(4), stream)),
-                rows * npg * 512 + rows * M * (64 + 16) + rows * D * 2 + rows * npg * 4
+                B * Hkv * npg * 512 + rows * M * (64 + 16) + rows * D * 2 + rows * npg * 4
                 + rows * kp * 8 + int(rows * n_bar) * 4 + rows * 12),
             "gemv_top_p": (rotating(lambda l, c, q: lambda: L.twl_gemv_top_p(
                 p(q), qcode, p(c.k_int4), p(l.sel_pages), p(l.sel_count), kp,
@@ -301,13 +301,16 @@ def main() -> int:
             for name in ("select_estimate_prune", "quest_score_planes"):
                 k = kernels.get(name)
                 if k:
-                    k["bytes_read_by_design"] = k["bytes"] - rows * npg * 256
+                    # a (channel, plane) run stays unread when every q head of the kv head's
+                    # group has the same sign there: 2^-G of the metadata on average
+                    k["bytes_read_by_design"] = k["bytes"] - (B * Hkv * npg * 512 >> (H // Hkv))
                     k["GBps_read_by_design"] = round(k["bytes_read_by_design"] / k["us"] / 1e3, 1)
 
     # the kernels one layer step launches (the choice twl_decode_layer makes)
     cus = torch.cuda.get_device_properties(dev).multi_processor_count
     split = args.split_estimator or 2 * rows < cus
-    row_kernel = (not split and H == Hkv and npg <= 8192 and rows <= 2 * cus)
+    has_planes = layers[0].cache.meta_planes is not None
+    row_kernel = (not split and (H == Hkv or has_planes) and npg <= 8192 and rows <= 2 * cus)
     score = ("quest_score_planes" if layers[0].cache.meta_planes is not None and H == Hkv
              else "quest_score")
     if split:
@@ -345,7 +348,8 @@ def main() -> int:
                     "us_per_launch": dom["us"], "traffic": traffic}
         if "bytes_read_by_design" in dom:
             roofline["note"] = ("achieved = algorithmic bytes / time; the kernel reads only the "
-                                "sign-selected half of the min/max metadata (plane layout), so "
+                                "min or max runs that the signs of its queries select (plane "
+                                "layout: half the metadata with one q head per kv head), so "
                                 "its HBM traffic is below the algorithmic bytes: "
                                 f"{dom['bytes_read_by_design']} B by design = "
                                 f"{dom['GBps_read_by_design']} GB/s of real traffic")

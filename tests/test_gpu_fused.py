@@ -203,14 +203,16 @@ def test_one_launch_row_kernel_equals_three_launches(dev, N, lens, budget, H, Hk
     assert differ <= 1
 
 
-@pytest.mark.parametrize("N,budget,H,dt", [
-    (1600, 320, 4, torch.float16),
-    (1000, 100, 4, torch.bfloat16),          # partial last page, budget not a multiple of 16
-    (11200, 16384, 2, torch.float16),        # every page
-    (40000, 4096, 2, torch.float16),         # 2500 pages per request (four scoring passes)
-    (32768, 8192, 2, torch.float16),         # the benchmark's row shape
+@pytest.mark.parametrize("N,budget,H,Hkv,dt", [
+    (1600, 320, 4, 4, torch.float16),
+    (1000, 100, 4, 4, torch.bfloat16),       # partial last page, budget not a multiple of 16
+    (11200, 16384, 2, 2, torch.float16),     # every page
+    (40000, 4096, 2, 2, torch.float16),      # 2500 pages per request (four scoring passes)
+    (32768, 8192, 2, 2, torch.float16),      # the benchmark's row shape
+    (1600, 320, 16, 4, torch.float16),       # GQA 4:1, 32 rows: a group's rows share an XCD
+    (1000, 100, 4, 2, torch.bfloat16),       # GQA 2:1, 8 rows: rows in launch order
 ])
-def test_row_kernel_with_plane_metadata(dev, N, budget, H, dt):
+def test_row_kernel_with_plane_metadata(dev, N, budget, H, Hkv, dt):
     """The plane layout (minima / maxima of all pages of a request contiguous per channel) against
     the record layout: planes hold exactly the records' numbers; page scores agree to summation
     order; the page lists are equal except pages whose score ties the k-th within rounding; rows
@@ -219,20 +221,20 @@ def test_row_kernel_with_plane_metadata(dev, N, budget, H, dt):
     B, p = 2, 0.9
     g = torch.Generator().manual_seed(N + 1)
     q = torch.randn((B, H, 128), generator=g)
-    k = torch.randn((B, H, N, 128), generator=g)
+    k = torch.randn((B, Hkv, N, 128), generator=g)
     for b in range(B):
         for h in range(H):
             pos = torch.randint(0, N, (6,), generator=g)
-            k[b, h, pos] += q[b, h] * (0.3 + torch.rand(6, 1, generator=g))
+            k[b, h // (H // Hkv), pos] += q[b, h] * (0.3 + torch.rand(6, 1, generator=g))
     npg = (N + 15) // 16
     cache = PagedKVCache.from_dense(k.to(dt), k.to(dt), dev,
                                     page_perm=torch.randperm(B * npg, generator=g), plane_pages=npg + 9)
     # planes == transposed records, bit for bit
     cap = cache.meta_planes.shape[-1]
     assert cap % 8 == 0 and cap >= npg
-    rec = cache.meta.view(torch.int16).reshape(-1, H, 32, 2, 4)              # [page, h, chunk, min|max, 4]
+    rec = cache.meta.view(torch.int16).reshape(-1, Hkv, 32, 2, 4)            # [page, h, chunk, min|max, 4]
     phys = cache.kv_page_indices.long().reshape(B, npg)
-    want = rec[phys].permute(0, 2, 3, 5, 4, 1).reshape(B, H, 128, 2, npg)    # [b, h, d, min|max, page]
+    want = rec[phys].permute(0, 2, 3, 5, 4, 1).reshape(B, Hkv, 128, 2, npg)  # [b, h, d, min|max, page]
     assert torch.equal(cache.meta_planes.view(torch.int16)[..., :npg], want)
     qd = q.to(dt).to(dev)
     tab = (cache.kv_page_indices, cache.kv_page_indptr, cache.kv_last_page_len)
@@ -244,7 +246,7 @@ def test_row_kernel_with_plane_metadata(dev, N, budget, H, dt):
     ps2 = torch.zeros((B, H, npg), dtype=torch.float32, device=dev)
     rc = _lib.lib().twl_quest_page_scores_planes(
         qd.data_ptr(), 0 if dt == torch.float16 else 1, cache.meta_planes.data_ptr(), cap,
-        cache.kv_page_indptr.data_ptr(), B, H, H, npg, ps2.data_ptr(), npg,
+        cache.kv_page_indptr.data_ptr(), B, H, Hkv, npg, ps2.data_ptr(), npg,
         torch.cuda.current_stream().cuda_stream)
     assert rc == 0
     assert torch.equal(ps2.view(torch.int32), Bv[5].view(torch.int32))

@@ -99,12 +99,14 @@ def test_small_layer_configs(dev, B, H, Hkv, N, budget, p, dt, fused):
     _run_case(dev, B, H, Hkv, N, budget, p, dt, seed=B * 100 + H, n_heavy=8, fused=fused)
 
 
-@pytest.mark.parametrize("B,H,N,budget", [
-    (2, 8, 2048, 512),       # 16 rows: separate launches, page scores from the plane layout
-    (8, 32, 1024, 256),      # 256 rows: the one-launch row kernel reading the plane layout
+@pytest.mark.parametrize("B,H,Hkv,N,budget", [
+    (2, 8, 8, 2048, 512),    # 16 rows: separate launches, page scores from the plane layout
+    (8, 32, 32, 1024, 256),  # 256 rows: the one-launch row kernel reading the plane layout
+    (8, 32, 8, 1024, 256),   # the same with 4 q heads per kv head (a group's rows share an XCD)
+    (2, 8, 2, 2048, 512),    # GQA, 16 rows: separate launches, records (planes present, unused)
 ])
-def test_layer_with_plane_metadata(dev, B, H, N, budget):
-    _run_case(dev, B, H, H, N, budget, 0.95, torch.float16, seed=B + N, n_heavy=8, planes=True)
+def test_layer_with_plane_metadata(dev, B, H, Hkv, N, budget):
+    _run_case(dev, B, H, Hkv, N, budget, 0.95, torch.float16, seed=B + N, n_heavy=8, planes=True)
 
 
 def test_layer_at_128k_context(dev):

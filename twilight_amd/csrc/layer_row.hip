@@ -54,7 +54,18 @@ __global__ __launch_bounds__(kRowThreads) void select_estimate_prune_kernel(RowA
   __shared__ int32_t sel_lds[kRowWaves * PW];
 
   select_smem_init<kRowThreads>(ssm);  // the barrier after the scoring phase orders it
-  const uint32_t row = blockIdx.x;
+  uint32_t row = blockIdx.x;
+  {
+    // q heads that share a kv head go to the same XCD (workgroups are dealt to the 8 XCDs round
+    // robin; each XCD has its own L2), so that the group's metadata comes from HBM once and the
+    // other heads of the group find it in that L2: 65 -> 56 us at 8 x 32 q heads on 8 kv heads.
+    // Only the placement depends on how the hardware deals workgroups; the result does not.
+    const uint32_t grp = a.f.num_q_heads / a.f.num_kv_heads;
+    if (grp > 1 && gridDim.x % (8 * grp) == 0) {
+      const uint32_t xcd = blockIdx.x & 7u, s = blockIdx.x >> 3;
+      row = ((s / grp) * 8 + xcd) * grp + s % grp;
+    }
+  }
   const uint32_t b = row / a.f.num_q_heads;
   const uint32_t h = row - b * a.f.num_q_heads;
   const uint32_t kvh = h / (a.f.num_q_heads / a.f.num_kv_heads);

@@ -108,8 +108,9 @@ def _fill_from_prefill(st: _LayerState, k: torch.Tensor, v: torch.Tensor, num_q_
     B, _, N, _ = k.shape
     npg = (N + PAGE - 1) // PAGE
     spare_per_req = (st.reserve_tokens + PAGE - 1) // PAGE + 1
-    # plane-layout metadata only where the one-launch selector can use it (no GQA sharing)
-    planes = npg + spare_per_req if k.shape[1] == num_q_heads else None
+    # plane-layout metadata next to the records: the one-launch selector reads half the bytes from
+    # it (with GQA it is used at the batch sizes where that launch runs, the records otherwise)
+    planes = npg + spare_per_req
     st.cache = PagedKVCache.from_dense(k, v, k.device, spare_pages=B * spare_per_req,
                                        plane_pages=planes)
     st.free = list(range(B * npg, B * (npg + spare_per_req)))
