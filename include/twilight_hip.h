@@ -146,9 +146,10 @@ int twl_gemv_top_p(const void* q, int q_dtype, const void* k_int4, const int32_t
  * cand_count. max_pages_per_req <= 8192. With meta_planes (plane layout, see
  * twl_meta_planes_build; then meta may be NULL) the page scores are accumulated channel by channel
  * in ascending order from the sign-selected runs; they can differ from twl_quest_page_scores in
- * the last bits (other summation order). Meant for about one row per compute unit (MHA decode at
- * moderate batch); with GQA the three-call form reads each metadata record once per kv head and
- * this one once per q head.
+ * the last bits (other summation order). Meant for about one row per compute unit (decode at
+ * moderate batch). With GQA every q-head row reads its kv head's metadata; the rows of a group
+ * are placed on one XCD so that all but the first read find it in that L2 (ahead of the
+ * three-call form with meta_planes, level with it on records).
  * ------------------------------------------------------------------------------------------- */
 int twl_select_estimate_prune(const void* q, int dtype, const void* meta, const void* k_int4,
                               const int32_t* kv_page_indices, const int32_t* kv_page_indptr,
