@@ -308,9 +308,10 @@ def main() -> int:
 
     # the kernels one layer step launches (the choice twl_decode_layer makes)
     cus = torch.cuda.get_device_properties(dev).multi_processor_count
-    split = args.split_estimator or 2 * rows < cus
+    split = args.split_estimator or 2 * rows < cus or (H != Hkv and 2 * rows == cus)
     has_planes = layers[0].cache.meta_planes is not None
-    row_kernel = (not split and (H == Hkv or has_planes) and npg <= 8192 and rows <= 2 * cus)
+    row_kernel = (not split and (H == Hkv or has_planes) and npg <= 8192
+                  and (has_planes or rows <= 2 * cus))
     score = ("quest_score_planes" if layers[0].cache.meta_planes is not None and H == Hkv
              else "quest_score")
     if split:

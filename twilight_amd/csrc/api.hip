@@ -51,15 +51,20 @@ extern "C" int twl_decode_layer(const twl_layer_args* a, void* stream) {
   // each row streams its pages one memory round trip after the other, so the estimator runs as a
   // GEMV over many short wavefronts and the pruner as a launch of its own (measured at 32 q heads,
   // 32768 tokens: 57 -> 43 us at batch 1, 63 -> 56 us at batch 3, equal at batch 4).
-  const bool split = a->split_estimator || (have_cus && 2u * rows < (uint32_t)cus);
+  // (With q heads sharing kv heads the separate launches are still ahead at exactly half a row
+  // per unit: 56.6 against 59.7 us.)
+  const bool gqa = a->num_q_heads != a->num_kv_heads;
+  const bool split = a->split_estimator ||
+                     (have_cus && (2u * rows < (uint32_t)cus || (gqa && 2u * rows == (uint32_t)cus)));
   // one workgroup per row from the metadata to the survivor list pays off while there are about
-  // as many rows as compute units (measured: ahead from half a row to two rows per unit). With
+  // as many rows as compute units (measured: ahead from half a row per unit on; with the record
+  // layout up to two rows per unit, with the plane layout at every larger batch tried). With
   // q heads sharing kv heads it needs the plane layout to be ahead of the grouped scoring kernel
   // (which reads each record once per group): 56 us against 64 us, with records 65 us.
   const bool planes_fit = a->meta_planes && a->plane_cap_pages >= a->max_pages_per_req;
   const bool row_kernel = !split && (a->num_q_heads == a->num_kv_heads || planes_fit) &&
                           a->max_pages_per_req <= 8192 && have_cus &&
-                          2u * rows >= (uint32_t)cus && rows <= 2u * (uint32_t)cus;
+                          2u * rows >= (uint32_t)cus && (planes_fit || rows <= 2u * (uint32_t)cus);
   if (row_kernel) {
     // 1+2+3. page scores, top-k pages, INT4 estimate, softmax, top-p, compaction: one launch
     rc = twl_select_estimate_prune(
