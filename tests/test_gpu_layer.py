@@ -109,6 +109,21 @@ def test_layer_with_plane_metadata(dev, B, H, Hkv, N, budget):
     _run_case(dev, B, H, Hkv, N, budget, 0.95, torch.float16, seed=B + N, n_heavy=8, planes=True)
 
 
+@pytest.mark.parametrize("B,H,Hkv,planes", [
+    (20, 32, 32, True),    # 640 rows, planes: the row kernel beyond two rows per compute unit
+    (20, 32, 32, False),   # 640 rows, records: scores, top-k and fused estimator as three launches
+    (6, 32, 8, True),      # 192 rows, 4 q heads per kv head, planes: row kernel, groups per XCD
+    (5, 28, 4, True),      # 140 rows, 7 q heads per kv head: rows stay in launch order
+    (4, 32, 8, True),      # 128 rows with GQA: every stage its own launch
+    (3, 32, 32, True),     # 96 rows: every stage its own launch, short GEMV wavefronts
+])
+def test_layer_dispatch_regimes(dev, B, H, Hkv, planes):
+    """One case per branch of the layer's choice of launches (by rows per compute unit, GQA and
+    metadata layout): every branch gives the oracle's result."""
+    _run_case(dev, B, H, Hkv, 512, 128, 0.9, torch.float16, seed=B * H + Hkv, n_heavy=4,
+              planes=planes)
+
+
 def test_layer_at_128k_context(dev):
     # 8192 pages per request: the widest selector shapes (8 pages per thread in the radix select,
     # four scoring passes over the plane layout), 512 selected pages, against the dense oracle
