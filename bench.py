@@ -265,7 +265,7 @@ def main() -> int:
                 p(c.kv_last_page_len), B, H, Hkv, args.budget, npg, sm, 0, args.top_p, 1,
                 p(l.sel_pages), kp, p(l.sel_count), p(l.idx), M, p(l.count), 0, 0, 0, M,
                 p(l.cand_count), p(c.meta_planes),
-                0 if c.meta_planes is None else c.meta_planes.size(4), stream)),
+                0 if c.meta_planes is None else c.meta_planes.size(4), 0, 0, stream)),
                 B * Hkv * npg * 512 + rows * M * (64 + 16) + rows * D * 2 + rows * npg * 4
                 + rows * kp * 8 + int(rows * n_bar) * 4 + rows * 12),
             "gemv_top_p": (rotating(lambda l, c, q: lambda: L.twl_gemv_top_p(
@@ -287,7 +287,7 @@ def main() -> int:
         if layers[0].cache.meta_planes is not None and H == Hkv:
             calls["quest_score_planes"] = (rotating(
                 lambda l, c, q: lambda: L.twl_quest_page_scores_planes(
-                    p(q), qcode, p(c.meta_planes), c.meta_planes.size(4), p(c.kv_page_indptr),
+                    p(q), qcode, p(c.meta_planes), c.meta_planes.size(4), 0, 0, p(c.kv_page_indptr),
                     B, H, Hkv, npg, p(l.page_scores), npg, stream)),
                 rows * npg * 512 + rows * npg * 4 + rows * D * 2)
         for name, (fn, nbytes) in calls.items():

@@ -32,7 +32,8 @@
  *     max[4c..4c+3] over the valid tokens of the page ("fp16" = the cache dtype, fp16 or bf16).
  *   - Quest page metadata, plane layout (optional second copy, see twl_meta_planes_build):
  *     planes[slot][kv_head][d][0 = min, 1 = max][logical page], 16-bit values in the cache dtype,
- *     plane_cap_pages pages per run, slot = position of the request in the batch.
+ *     plane_cap_pages pages per run, slot = position of the request in the batch or, with a
+ *     slot table (plane_slots [batch], entries in [0, plane_num_slots)), the table's entry.
  *   - Paged K / V caches: fp16 or bf16, addressed with explicit element strides
  *     (page, token, kv head); head_dim is contiguous.
  */
@@ -160,7 +161,9 @@ int twl_select_estimate_prune(const void* q, int dtype, const void* meta, const 
                               int32_t* sel_count, int32_t* idx, uint32_t idx_stride,
                               int32_t* count, float* page_scores_out, uint32_t page_score_stride,
                               float* scores_out, uint32_t score_stride, int32_t* cand_count,
-                              const void* meta_planes, uint32_t plane_cap_pages, void* stream);
+                              const void* meta_planes, uint32_t plane_cap_pages,
+                              const int32_t* plane_slots, uint32_t plane_num_slots,
+                              void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * INT4-K score GEMV over candidate pages: out[r, c] = sm_scale * sum_d q[r,d] * dequant(K[c,d]).
@@ -290,7 +293,8 @@ int twl_kv_append(const void* k_new, const void* v_new, int kv_dtype, uint64_t n
                   uint64_t token_stride, uint64_t head_stride, const int32_t* kv_page_indices,
                   const int32_t* kv_page_indptr, int32_t* kv_last_page_len, uint32_t batch,
                   uint32_t num_kv_heads, void* k_int4, void* meta, void* meta_planes,
-                  uint32_t plane_cap_pages, void* stream);
+                  uint32_t plane_cap_pages, const int32_t* plane_slots, uint32_t plane_num_slots,
+                  void* stream);
 
 /* Quest metadata in PLANE layout: planes[slot][kv_head][d][0 = min, 1 = max][logical page], 16-bit
  * values in the cache dtype, plane_cap_pages (a multiple of 8) pages per run, slot = position of
@@ -299,16 +303,22 @@ int twl_kv_append(const void* k_new, const void* v_new, int kv_dtype, uint64_t n
  * pass of twl_select_estimate_prune touches half the bytes of the record layout. Nothing in the
  * reference corresponds to it (it recomputes the chunk maxima from K every step, quest.py:68-74).
  * twl_meta_planes_build fills the planes of the pages of the current page table from the metadata
- * records of twl_kv_shadow_build; twl_kv_append keeps them current when given meta_planes. */
+ * records of twl_kv_shadow_build; twl_kv_append keeps them current when given meta_planes.
+ * plane_slots (nullable, device, [batch]) names the slot of every batch position, so that a
+ * request keeps its planes when its position in the batch changes (continuous batching: a request
+ * leaves and the others move up); plane_num_slots is the number of slots the buffer holds, and
+ * entries outside [0, plane_num_slots) are clamped. NULL: slot = batch position. Two positions of
+ * one batch must not name the same slot. */
 int twl_meta_planes_build(const void* meta, const int32_t* kv_page_indices,
                           const int32_t* kv_page_indptr, uint32_t batch, uint32_t num_kv_heads,
                           uint32_t max_pages_per_req, void* meta_planes, uint32_t plane_cap_pages,
-                          void* stream);
+                          const int32_t* plane_slots, uint32_t plane_num_slots, void* stream);
 /* twl_quest_page_scores from the plane layout (one q head per row reads the runs its signs
  * select: half the bytes of the record form; with GQA the q heads of a group do not share reads
  * here, the record form does). Scores are accumulated channel by channel in ascending order. */
 int twl_quest_page_scores_planes(const void* q, int q_dtype, const void* meta_planes,
-                                 uint32_t plane_cap_pages, const int32_t* kv_page_indptr,
+                                 uint32_t plane_cap_pages, const int32_t* plane_slots,
+                                 uint32_t plane_num_slots, const int32_t* kv_page_indptr,
                                  uint32_t batch, uint32_t num_q_heads, uint32_t num_kv_heads,
                                  uint32_t max_pages_per_req, float* page_scores,
                                  uint32_t score_stride, void* stream);
@@ -368,6 +378,8 @@ typedef struct twl_layer_args {
   const void* meta;         /* Quest metadata records */
   const void* meta_planes;  /* the same in plane layout (nullable), see twl_meta_planes_build */
   uint32_t plane_cap_pages;
+  const int32_t* plane_slots; /* nullable: plane slot of each batch position */
+  uint32_t plane_num_slots;
   const int32_t* kv_page_indices;
   const int32_t* kv_page_indptr;
   const int32_t* kv_last_page_len;

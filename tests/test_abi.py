@@ -20,7 +20,7 @@ def test_header_symbols_are_exported(hip_lib):
     assert declared == set(_lib.EXPORTS)
     for name in declared:
         assert hasattr(hip_lib, name), name
-    assert hip_lib.twl_abi_version() == 3
+    assert hip_lib.twl_abi_version() == 4
 
 
 def test_header_compiles_as_c():
@@ -109,7 +109,7 @@ def test_c_level_validation_without_gpu(hip_lib):
         kw.get("q", f), kw.get("dt", 0), kw.get("meta", f), f, f, f, f, 1, kw.get("hq", 1),
         kw.get("hkv", 1), kw.get("budget", 64), kw.get("npg", 16), 1.0, 0, kw.get("p", 0.9), 1,
         kw.get("sel", f), kw.get("sel_stride", 4), f, f, kw.get("idx_stride", 64), f, 0, 0, 0, 64,
-        0, kw.get("planes", 0), kw.get("cap", 0), 0)
+        0, kw.get("planes", 0), kw.get("cap", 0), kw.get("slots", 0), kw.get("nslots", 0), 0)
     assert sep(meta=0) == -1 and sep(sel=0) == -1
     assert sep(dt=5) == -3
     assert sep(budget=0) == -2 and sep(npg=0) == -2 and sep(npg=9000) == -2
@@ -118,15 +118,18 @@ def test_c_level_validation_without_gpu(hip_lib):
     assert sep(q=f + 4) == -4
     assert sep(meta=0, planes=f, cap=16, budget=0) == -2  # planes alone pass the NULL check
     assert sep(planes=f, cap=8) == -2 and sep(planes=f, cap=20) == -2   # cap < pages, cap % 8
+    assert sep(planes=f, cap=16, slots=f, nslots=0) == -2               # slot table, no slots
     app = lambda **kw: L.twl_kv_append(
         kw.get("k", f), f, kw.get("dt", 0), 256, 128, f, f, 4096, kw.get("ts", 256), 128, f, f,
-        kw.get("last", f), kw.get("b", 1), 1, 0, 0, kw.get("planes", 0), kw.get("cap", 0), 0)
+        kw.get("last", f), kw.get("b", 1), 1, 0, 0, kw.get("planes", 0), kw.get("cap", 0),
+        kw.get("slots", 0), kw.get("nslots", 0), 0)
     assert app(k=0) == -1 and app(last=0) == -1
     assert app(dt=2) == -3 and app(b=0) == -2 and app(ts=250) == -4 and app(k=f + 2) == -4
-    assert app(planes=f, cap=12) == -2
+    assert app(planes=f, cap=12) == -2 and app(planes=f, cap=16, slots=f, nslots=0) == -2
     pb = lambda **kw: L.twl_meta_planes_build(kw.get("meta", f), f, f, 1, 1, kw.get("npg", 8),
-                                              kw.get("planes", f), kw.get("cap", 8), 0)
-    assert pb(meta=0) == -1 and pb(planes=0) == -1
+                                              kw.get("planes", f), kw.get("cap", 8),
+                                              kw.get("slots", 0), kw.get("nslots", 0), 0)
+    assert pb(meta=0) == -1 and pb(planes=0) == -1 and pb(slots=f, nslots=0) == -2
     assert pb(cap=12) == -2 and pb(npg=16) == -2 and pb(npg=0) == -2 and pb(planes=f + 8) == -4
     qk = lambda **kw: L.twl_qk_int8_lse(
         kw.get("q", f), f, f, f, kw.get("lse", f), 1, kw.get("hq", 1), kw.get("hkv", 1),

@@ -295,3 +295,69 @@ def test_layer_step_replays_from_a_hip_graph(dev, H, Hkv):
         mx = int(cnt_e.max())
         assert torch.equal(layer.idx[..., :mx] * (torch.arange(mx, device=dev) < cnt_e[..., None]),
                            idx_e[..., :mx] * (torch.arange(mx, device=dev) < cnt_e[..., None]))
+
+
+def test_plane_slot_table(dev):
+    """Plane-layout metadata addressed through a slot table: requests sit in any slots of a larger
+    buffer, a request leaves the batch and the others keep their planes, appends go to the right
+    slot. Everything is compared bit for bit with slot = batch position on the same data."""
+    from twilight_amd import kernel as K
+    g = torch.Generator().manual_seed(21)
+    B, H, N, budget, p = 3, 4, 700, 160, 0.9
+    npg = (N + 15) // 16
+    q = torch.randn((B, H, 128), generator=g).half()
+    k = torch.randn((B, H, N + 20, 128), generator=g).half()
+    v = torch.randn((B, H, N + 20, 128), generator=g).half()
+
+    def fresh(**kw):
+        return PagedKVCache.from_dense(k[:, :, :N].contiguous(), v[:, :, :N].contiguous(), dev,
+                                       page_perm=torch.randperm(B * npg, generator=torch.Generator().manual_seed(3)),
+                                       spare_pages=2 * B, **kw)
+
+    plain = fresh(plane_pages=npg + 8)
+    slotted = fresh()
+    slots = torch.tensor([4, 0, 2], dtype=torch.int32)
+    slotted.enable_planes(npg + 8, num_slots=5, slots=slots)
+    assert slotted.meta_planes.shape[0] == 5
+    pl = slotted.meta_planes.view(torch.int16)
+    assert torch.equal(pl[slots.long()], plain.meta_planes.view(torch.int16))
+    assert not pl[1].any() and not pl[3].any()                   # slots of nobody stay untouched
+    qd = q.to(dev)
+
+    def run(c, qq):
+        return K.quest_gemv_int4_top_p(qq, c.meta, c.k_int4, c.kv_page_indices, c.kv_page_indptr,
+                                       c.kv_last_page_len, budget, c.max_pages_per_req, p,
+                                       return_scores=True, meta_planes=c.meta_planes,
+                                       plane_slots=c.plane_slots)
+    want, got = run(plain, qd), run(slotted, qd)
+    for a, b in zip(want, got):
+        assert torch.equal(a, b)
+    # the whole layer, and the separate-launch scoring kernel (12 rows: the split path)
+    la = TwilightDecodeLayer(plain, H, token_budget=budget, top_p=p)
+    lb = TwilightDecodeLayer(slotted, H, token_budget=budget, top_p=p)
+    assert torch.equal(la(qd), lb(qd)) and torch.equal(la.idx, lb.idx)
+    # decode appends across a page boundary land in the request's own slot
+    free_a, free_b = list(range(B * npg, B * npg + 2 * B)), list(range(B * npg, B * npg + 2 * B))
+    for s in range(20):
+        plain.append(k[:, :, N + s].to(dev), v[:, :, N + s].to(dev), free_a)
+        slotted.append(k[:, :, N + s].to(dev), v[:, :, N + s].to(dev), free_b)
+    pl = slotted.meta_planes.view(torch.int16)
+    assert torch.equal(pl[slots.long()], plain.meta_planes.view(torch.int16))
+    assert not pl[1].any() and not pl[3].any()
+    # request 1 leaves: requests 0 and 2 move to positions 0 and 1, their planes stay in place
+    per = [plain._per_req[b] for b in (0, 2)]
+    ids = torch.tensor(per[0] + per[1], dtype=torch.int32)
+    indptr = torch.tensor([0, len(per[0]), len(per[0]) + len(per[1])], dtype=torch.int32)
+    last = torch.tensor([plain._last[0], plain._last[2]], dtype=torch.int32)
+    before = slotted.meta_planes.clone()
+    slotted.set_page_table(ids, indptr, last)
+    slotted.set_plane_slots(torch.tensor([4, 2], dtype=torch.int32))
+    assert torch.equal(before, slotted.meta_planes)              # nothing was rebuilt
+    got2 = run(slotted, qd[[0, 2]].contiguous())
+    want2 = run(plain, qd)
+    for a, b in zip(want2, got2):
+        assert torch.equal(a[[0, 2]], b)
+    with pytest.raises(RuntimeError):
+        slotted.set_plane_slots(torch.tensor([4, 4], dtype=torch.int32))   # one slot, two requests
+    with pytest.raises(RuntimeError):
+        slotted.set_plane_slots(torch.tensor([4, 5], dtype=torch.int32))   # outside the buffer

@@ -39,6 +39,7 @@ class LayerArgs(ctypes.Structure):
         ("page_stride", c_uint64), ("token_stride", c_uint64), ("head_stride", c_uint64),
         ("k_int4", c_void_p), ("meta", c_void_p),
         ("meta_planes", c_void_p), ("plane_cap_pages", c_uint32),
+        ("plane_slots", c_void_p), ("plane_num_slots", c_uint32),
         ("kv_page_indices", c_void_p), ("kv_page_indptr", c_void_p), ("kv_last_page_len", c_void_p),
         ("batch", c_uint32), ("num_q_heads", c_uint32), ("num_kv_heads", c_uint32),
         ("max_pages_per_req", c_uint32), ("token_budget", c_uint32),
@@ -82,7 +83,7 @@ def lib() -> ctypes.CDLL:
                                  f32, i32, vp, u32, vp, vp, u32, vp, vp, vp]
     L.twl_select_estimate_prune.argtypes = [vp, i32, vp, vp, vp, vp, vp, u32, u32, u32, u32, u32,
                                             f32, vp, f32, i32, vp, u32, vp, vp, u32, vp, vp, u32,
-                                            vp, u32, vp, vp, u32, vp]
+                                            vp, u32, vp, vp, u32, vp, u32, vp]
     L.twl_gemv_int4.argtypes = [vp, i32, vp, u32, vp, vp, vp, vp, u32, vp, vp, vp, u32, u32, u32,
                                 u32, f32, vp]
     L.twl_gemv_int4_nhd.argtypes = [vp, vp, u32, vp, vp, vp, vp, vp, vp, u32, u32, u32, u32, f32, vp]
@@ -102,9 +103,10 @@ def lib() -> ctypes.CDLL:
     L.twl_get_label_tensor.argtypes = [vp, vp, vp, u32, u32, u32, u32] + [c_int64] * 8 + [vp]
     L.twl_bgemv_int8.argtypes = [vp, vp, vp, vp, u32, u32, u32, u32] + [c_int64] * 11 + [vp]
     L.twl_kv_append.argtypes = [vp, vp, i32, u64, u64, vp, vp, u64, u64, u64, vp, vp, vp, u32, u32,
-                                vp, vp, vp, u32, vp]
-    L.twl_meta_planes_build.argtypes = [vp, vp, vp, u32, u32, u32, vp, u32, vp]
-    L.twl_quest_page_scores_planes.argtypes = [vp, i32, vp, u32, vp, u32, u32, u32, u32, vp, u32, vp]
+                                vp, vp, vp, u32, vp, u32, vp]
+    L.twl_meta_planes_build.argtypes = [vp, vp, vp, u32, u32, u32, vp, u32, vp, u32, vp]
+    L.twl_quest_page_scores_planes.argtypes = [vp, i32, vp, u32, vp, u32, vp, u32, u32, u32, u32, vp,
+                                               u32, vp]
     i64 = ctypes.c_int64
     L.twl_qk_int8_lse.argtypes = [vp, vp, vp, vp, vp, u32, u32, u32, u32, u32, u32, i64, i64, i64,
                                   i64, i64, i64, vp]

@@ -36,8 +36,10 @@ class PagedKVCache:
         self.kv_last_page_len: Optional[torch.Tensor] = None
         self.max_pages_per_req = 0
         self._seq_lens = None  # host copy, for append bookkeeping
-        # Quest metadata in plane layout [batch, Hkv, 128, 2, cap] (see enable_planes)
+        # Quest metadata in plane layout [slots, Hkv, 128, 2, cap] (see enable_planes) and the
+        # slot of every request of the batch (None: slot = position in the batch)
         self.meta_planes: Optional[torch.Tensor] = None
+        self.plane_slots: Optional[torch.Tensor] = None
 
     # ---- page table ---------------------------------------------------------------------------
     def set_page_table(self, kv_page_indices: torch.Tensor, kv_page_indptr: torch.Tensor,
@@ -67,27 +69,54 @@ class PagedKVCache:
         kv_shadow_build(self.k_cache, self.k_int4, self.meta, page_ids, valid_len)
         self.rebuild_planes()
 
-    def enable_planes(self, cap_pages: Optional[int] = None) -> None:
+    def enable_planes(self, cap_pages: Optional[int] = None, num_slots: Optional[int] = None,
+                      slots: Optional[torch.Tensor] = None) -> None:
         """Keep the Quest metadata also in plane layout (per request slot, kv head and channel the
         page minima contiguously, then the maxima), sized for requests of up to ``cap_pages`` pages
-        (default: the current longest request). The one-launch selector of MHA layers then reads
-        half the metadata bytes. Needs a page table; the batch size fixes the number of slots."""
+        (default: the current longest request). The one-launch selector then reads half the
+        metadata bytes. Needs a page table. ``num_slots`` (default: the batch size) is the number
+        of requests the buffer can hold; ``slots`` int32 [batch] names the slot of each request of
+        the current batch (default: its position), see :meth:`set_plane_slots`."""
         if self.kv_page_indptr is None:
             raise RuntimeError("enable_planes needs a page table (set_page_table)")
         cap = max(int(cap_pages or 0), self.max_pages_per_req, 8)
         cap = (cap + 7) // 8 * 8
-        self.meta_planes = torch.zeros((self.batch, self.num_kv_heads, HEAD_DIM, 2, cap),
+        n = max(int(num_slots or 0), self.batch)
+        self.meta_planes = torch.zeros((n, self.num_kv_heads, HEAD_DIM, 2, cap),
                                        dtype=self.dtype, device=self.device)
+        self.plane_slots = None
+        if slots is not None:
+            self.set_plane_slots(slots, rebuild=False)
         self.rebuild_planes()
+
+    def set_plane_slots(self, slots: Optional[torch.Tensor], rebuild: bool = False) -> None:
+        """Name the plane slot of every request of the current batch (int32 [batch], distinct
+        values in [0, slots of the buffer)); ``None`` goes back to slot = position. When the batch
+        changes composition (a request leaves, the others move up) the page table and this table
+        change and the planes stay where they are; ``rebuild`` refills the named slots from the
+        records (for requests that are new to the buffer)."""
+        if slots is not None:
+            host = [int(x) for x in slots.cpu().tolist()]
+            n = 0 if self.meta_planes is None else self.meta_planes.size(0)
+            if len(host) != self.batch or len(set(host)) != len(host) or \
+                    any(x < 0 or x >= n for x in host):
+                raise RuntimeError("plane slots must be distinct, one per request, inside the buffer")
+            slots = slots.to(self.device, torch.int32).contiguous()
+        self.plane_slots = slots
+        if rebuild:
+            self.rebuild_planes()
 
     def rebuild_planes(self) -> None:
         """Refill the plane-layout metadata from the records, for the pages of the page table."""
         if self.meta_planes is None or self.kv_page_indptr is None:
             return
-        if self.batch != self.meta_planes.size(0) or self.max_pages_per_req > self.meta_planes.size(4):
-            raise RuntimeError("the page table no longer fits the plane buffer: call enable_planes")
+        fits = (self.batch <= self.meta_planes.size(0) if self.plane_slots is None
+                else self.plane_slots.numel() == self.batch)
+        if not fits or self.max_pages_per_req > self.meta_planes.size(4):
+            raise RuntimeError("the page table no longer fits the plane buffer: call enable_planes "
+                               "(or set_plane_slots for the new batch)")
         meta_planes_build(self.meta, self.kv_page_indices, self.kv_page_indptr,
-                          self.max_pages_per_req, self.meta_planes)
+                          self.max_pages_per_req, self.meta_planes, self.plane_slots)
 
     @classmethod
     def from_dense(cls, k: torch.Tensor, v: torch.Tensor, device, page_perm: Optional[torch.Tensor] = None,
@@ -160,7 +189,7 @@ class PagedKVCache:
         # one launch: rows, INT4 codes, min/max metadata, and the device-side lengths + 1
         kv_append(k_new, v_new, self.k_cache, self.v_cache, self.kv_page_indices,
                   self.kv_page_indptr, self.kv_last_page_len, self.k_int4, self.meta,
-                  self.meta_planes)
+                  self.meta_planes, self.plane_slots if self.meta_planes is not None else None)
         for b in range(B):
             last[b] += 1
             self._seq_lens[b] += 1

@@ -131,6 +131,8 @@ struct AppendArgs {
   uint8_t* meta;
   uint16_t* planes;     // nullable: metadata in plane layout (meta_planes.hip)
   uint32_t plane_cap;
+  const int32_t* plane_slots;  // nullable: plane slot of each batch position
+  uint32_t plane_num_slots;
 };
 
 template <int DT>
@@ -213,8 +215,10 @@ __global__ __launch_bounds__(kShThreads) void kv_append_kernel(AppendArgs a) {
       *pmax = f32_to_bits16<DT>(mx0) | (f32_to_bits16<DT>(mx1) << 16);
     }
     if (a.planes && n_pages <= (int)a.plane_cap) {
-      // the same fold in the plane layout: runs [d][min|max][logical page] of slot b
-      uint16_t* pl = a.planes + ((size_t)b * a.num_kv_heads + kvh) * (TWL_HEAD_DIM * 2) * a.plane_cap +
+      // the same fold in the plane layout: runs [d][min|max][logical page] of the request's slot
+      const uint32_t pslot = plane_slot(a.plane_slots, a.plane_num_slots, b);
+      uint16_t* pl = a.planes +
+                     ((size_t)pslot * a.num_kv_heads + kvh) * (TWL_HEAD_DIM * 2) * a.plane_cap +
                      (n_pages - 1);
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
@@ -303,7 +307,8 @@ extern "C" int twl_kv_append(const void* k_new, const void* v_new, int kv_dtype,
                              uint64_t head_stride, const int32_t* kv_page_indices,
                              const int32_t* kv_page_indptr, int32_t* kv_last_page_len,
                              uint32_t batch, uint32_t num_kv_heads, void* k_int4, void* meta,
-                             void* meta_planes, uint32_t plane_cap_pages, void* stream) {
+                             void* meta_planes, uint32_t plane_cap_pages,
+                             const int32_t* plane_slots, uint32_t plane_num_slots, void* stream) {
   if (!k_new || !v_new || !k_cache || !v_cache || !kv_page_indices || !kv_page_indptr ||
       !kv_last_page_len)
     return TWL_ENULL;
@@ -316,6 +321,7 @@ extern "C" int twl_kv_append(const void* k_new, const void* v_new, int kv_dtype,
       (((uintptr_t)meta_planes) & 15u))
     return TWL_EALIGN;
   if (meta_planes && (plane_cap_pages == 0 || (plane_cap_pages & 7u))) return TWL_EINVAL;
+  if (meta_planes && plane_slots && plane_num_slots == 0) return TWL_EINVAL;
   twl::AppendArgs a{};
   a.k_new = k_new; a.v_new = v_new; a.new_batch_stride = new_batch_stride;
   a.new_head_stride = new_head_stride; a.k_cache = k_cache; a.v_cache = v_cache;
@@ -324,6 +330,7 @@ extern "C" int twl_kv_append(const void* k_new, const void* v_new, int kv_dtype,
   a.kv_last_page_len = kv_last_page_len; a.num_kv_heads = num_kv_heads;
   a.k_int4 = (uint8_t*)k_int4; a.meta = (uint8_t*)meta;
   a.planes = (uint16_t*)meta_planes; a.plane_cap = plane_cap_pages;
+  a.plane_slots = plane_slots; a.plane_num_slots = plane_num_slots;
   if (kv_dtype == TWL_F16)
     hipLaunchKernelGGL((twl::kv_append_kernel<TWL_F16>), dim3(batch), dim3(twl::kShThreads), 0,
                        (hipStream_t)stream, a);

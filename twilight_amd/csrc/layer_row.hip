@@ -29,8 +29,10 @@ struct RowArgs {
   int32_t* sel_count_out;
   float* page_scores_out;   // nullable
   uint32_t page_score_stride;
-  const uint16_t* planes;   // PLANES: metadata in plane layout (meta_planes.hip), slot = batch index
+  const uint16_t* planes;   // PLANES: metadata in plane layout (meta_planes.hip)
   uint32_t plane_cap;
+  const int32_t* plane_slots;  // nullable: slot of each batch position (else slot = position)
+  uint32_t plane_num_slots;
 };
 
 constexpr int kRowThreads = 1024;
@@ -93,8 +95,9 @@ __global__ __launch_bounds__(kRowThreads) void select_estimate_prune_kernel(RowA
     const uint16_t* qrow = (const uint16_t*)a.f.q + (size_t)row * TWL_HEAD_DIM;
     const float q_lo = bits16_to_f32<QDT>(qrow[lane]);
     const float q_hi = bits16_to_f32<QDT>(qrow[64 + lane]);
+    const uint32_t slot = plane_slot(a.plane_slots, a.plane_num_slots, b);
     const uint16_t* pl =
-        a.planes + ((size_t)b * a.f.num_kv_heads + kvh) * (TWL_HEAD_DIM * 2) * a.plane_cap;
+        a.planes + ((size_t)slot * a.f.num_kv_heads + kvh) * (TWL_HEAD_DIM * 2) * a.plane_cap;
     constexpr int PL_PASSES = (SEL_VPT + 1) / 2;  // 16 waves x 128 pages = 2048 pages per pass
 #pragma unroll
     for (int pass = 0; pass < PL_PASSES; ++pass) {
@@ -243,7 +246,7 @@ extern "C" int twl_select_estimate_prune(
     int32_t* sel_pages, uint32_t sel_stride, int32_t* sel_count, int32_t* idx, uint32_t idx_stride,
     int32_t* count, float* page_scores_out, uint32_t page_score_stride, float* scores_out,
     uint32_t score_stride, int32_t* cand_count, const void* meta_planes,
-    uint32_t plane_cap_pages, void* stream) {
+    uint32_t plane_cap_pages, const int32_t* plane_slots, uint32_t plane_num_slots, void* stream) {
   if (!q || (!meta && !meta_planes) || !k_int4 || !kv_page_indices || !kv_page_indptr || !kv_last_page_len ||
       !sel_pages || !sel_count || !idx || !count)
     return TWL_ENULL;
@@ -266,6 +269,7 @@ extern "C" int twl_select_estimate_prune(
     return TWL_EALIGN;
   if (meta_planes && (plane_cap_pages < max_pages_per_req || (plane_cap_pages & 7u)))
     return TWL_EINVAL;
+  if (meta_planes && plane_slots && plane_num_slots == 0) return TWL_EINVAL;
   twl::RowArgs a{};
   a.f.q = q; a.f.k_int4 = (const uint8_t*)k_int4; a.f.sel_stride = sel_stride;
   a.f.kv_page_indices = kv_page_indices; a.f.kv_page_indptr = kv_page_indptr;
@@ -278,6 +282,7 @@ extern "C" int twl_select_estimate_prune(
   a.max_pages_req = max_pages_per_req; a.sel_pages_out = sel_pages; a.sel_count_out = sel_count;
   a.page_scores_out = page_scores_out; a.page_score_stride = page_score_stride;
   a.planes = (const uint16_t*)meta_planes; a.plane_cap = plane_cap_pages;
+  a.plane_slots = plane_slots; a.plane_num_slots = plane_num_slots;
   const uint32_t rows = batch * num_q_heads;
   hipStream_t s = (hipStream_t)stream;
   const bool small = max_pages_per_req <= 2048;

@@ -10,7 +10,9 @@
 // so a row of the decode batch streams 128 runs of `pages` values — the min run or the max run of
 // each channel, chosen by the sign of q_d — and touches half the bytes. Planes are indexed by
 // LOGICAL page of a request slot (slot = position in the batch), not by physical page: they are a
-// per-request side buffer next to the paged K / V, updated by twl_kv_append.
+// per-request side buffer next to the paged K / V, updated by twl_kv_append. The slot of a request is its position in the batch, or, with a slot
+// table (plane_slots), any slot of the buffer: then a batch whose composition changes keeps the
+// planes of its requests where they are.
 #include "twl_common.h"
 
 namespace twl {
@@ -22,6 +24,8 @@ struct PlanesArgs {
   uint32_t num_kv_heads;
   uint16_t* planes;
   uint32_t cap;          // pages per run
+  const int32_t* slots;  // nullable: slot of each batch position
+  uint32_t num_slots;
 };
 
 constexpr int kPlTile = 64;  // pages per workgroup
@@ -48,7 +52,8 @@ __global__ __launch_bounds__(256) void meta_planes_build_kernel(PlanesArgs a) {
   }
   __syncthreads();
   const int lane = tx & 63, wave = tx >> 6;
-  uint16_t* out = a.planes + ((size_t)b * a.num_kv_heads + kvh) * (TWL_HEAD_DIM * 2) * a.cap;
+  const uint32_t slot = plane_slot(a.slots, a.num_slots, b);
+  uint16_t* out = a.planes + ((size_t)slot * a.num_kv_heads + kvh) * (TWL_HEAD_DIM * 2) * a.cap;
   // run r = d * 2 + plane; record element of (d, plane) = (d / 4) * 8 + plane * 4 + d % 4
   for (int r = wave; r < TWL_HEAD_DIM * 2; r += 4) {
     const int d = r >> 1, plane = r & 1;
@@ -62,17 +67,21 @@ __global__ __launch_bounds__(256) void meta_planes_build_kernel(PlanesArgs a) {
 extern "C" int twl_meta_planes_build(const void* meta, const int32_t* kv_page_indices,
                                      const int32_t* kv_page_indptr, uint32_t batch,
                                      uint32_t num_kv_heads, uint32_t max_pages_per_req,
-                                     void* planes, uint32_t plane_cap_pages, void* stream) {
+                                     void* planes, uint32_t plane_cap_pages,
+                                     const int32_t* plane_slots, uint32_t plane_num_slots,
+                                     void* stream) {
   if (!meta || !kv_page_indices || !kv_page_indptr || !planes) return TWL_ENULL;
   if (batch == 0 || num_kv_heads == 0 || max_pages_per_req == 0) return TWL_EINVAL;
   if (plane_cap_pages == 0 || (plane_cap_pages & 7u) || max_pages_per_req > plane_cap_pages)
     return TWL_EINVAL;
   if (batch > 65535u || num_kv_heads > 65535u) return TWL_EINVAL;
+  if (plane_slots && plane_num_slots == 0) return TWL_EINVAL;
   if ((((uintptr_t)meta) & 15u) || (((uintptr_t)planes) & 15u)) return TWL_EALIGN;
   twl::PlanesArgs a{};
   a.meta = (const uint8_t*)meta; a.kv_page_indices = kv_page_indices;
   a.kv_page_indptr = kv_page_indptr; a.num_kv_heads = num_kv_heads;
   a.planes = (uint16_t*)planes; a.cap = plane_cap_pages;
+  a.slots = plane_slots; a.num_slots = plane_num_slots;
   const dim3 grid((max_pages_per_req + twl::kPlTile - 1) / twl::kPlTile, num_kv_heads, batch);
   hipLaunchKernelGGL(twl::meta_planes_build_kernel, grid, dim3(256), 0, (hipStream_t)stream, a);
   return hipGetLastError() == hipSuccess ? TWL_OK : TWL_ELAUNCH;
@@ -84,6 +93,8 @@ struct PlaneScoreArgs {
   const void* q;
   const uint16_t* planes;
   uint32_t cap;
+  const int32_t* slots;  // nullable: slot of each batch position
+  uint32_t num_slots;
   const int32_t* kv_page_indptr;
   uint32_t num_q_heads, num_kv_heads;
   uint32_t max_pages;
@@ -115,7 +126,9 @@ __global__ __launch_bounds__(kPsThreads) void quest_score_planes_kernel(PlaneSco
   const uint16_t* qrow = (const uint16_t*)a.q + (size_t)row * TWL_HEAD_DIM;
   const float q_lo = bits16_to_f32<DT>(qrow[lane]);
   const float q_hi = bits16_to_f32<DT>(qrow[64 + lane]);
-  const uint16_t* pl = a.planes + ((size_t)b * a.num_kv_heads + kvh) * (TWL_HEAD_DIM * 2) * a.cap;
+  const uint32_t slot = plane_slot(a.slots, a.num_slots, b);
+  const uint16_t* pl =
+      a.planes + ((size_t)slot * a.num_kv_heads + kvh) * (TWL_HEAD_DIM * 2) * a.cap;
   const int pg0 = w0 + 2 * lane;
   const int pgc = min(pg0, (int)a.cap - 2);
   float s0 = 0.0f, s1 = 0.0f;
@@ -137,6 +150,7 @@ __global__ __launch_bounds__(kPsThreads) void quest_score_planes_kernel(PlaneSco
 
 extern "C" int twl_quest_page_scores_planes(const void* q, int q_dtype, const void* meta_planes,
                                             uint32_t plane_cap_pages,
+                                            const int32_t* plane_slots, uint32_t plane_num_slots,
                                             const int32_t* kv_page_indptr, uint32_t batch,
                                             uint32_t num_q_heads, uint32_t num_kv_heads,
                                             uint32_t max_pages_per_req, float* page_scores,
@@ -148,11 +162,13 @@ extern "C" int twl_quest_page_scores_planes(const void* q, int q_dtype, const vo
   if (max_pages_per_req == 0 || max_pages_per_req > 16384 || score_stride < max_pages_per_req)
     return TWL_EINVAL;
   if (plane_cap_pages < max_pages_per_req || (plane_cap_pages & 7u)) return TWL_EINVAL;
+  if (plane_slots && plane_num_slots == 0) return TWL_EINVAL;
   if ((uint64_t)batch * num_q_heads > 65535u) return TWL_EINVAL;
   if ((((uintptr_t)q) & 1u) || (((uintptr_t)meta_planes) & 15u) || (((uintptr_t)page_scores) & 3u))
     return TWL_EALIGN;
   twl::PlaneScoreArgs a{};
   a.q = q; a.planes = (const uint16_t*)meta_planes; a.cap = plane_cap_pages;
+  a.slots = plane_slots; a.num_slots = plane_num_slots;
   a.kv_page_indptr = kv_page_indptr; a.num_q_heads = num_q_heads; a.num_kv_heads = num_kv_heads;
   a.max_pages = max_pages_per_req; a.page_scores = page_scores; a.score_stride = score_stride;
   const dim3 grid((max_pages_per_req + twl::kPsPagesPerBlock - 1) / twl::kPsPagesPerBlock,

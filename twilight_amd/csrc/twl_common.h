@@ -141,6 +141,14 @@ __device__ __forceinline__ int wave_inclusive_scan(int v) {
   return v;
 }
 
+// Slot of a request's plane-layout metadata: the request's position in the batch, or, with a slot
+// table, the entry of that position (clamped, so that a corrupt table cannot leave the buffer).
+__device__ __forceinline__ uint32_t plane_slot(const int32_t* slots, uint32_t num_slots, uint32_t b) {
+  if (!slots) return b;
+  const int s = slots[b];
+  return (uint32_t)min(max(s, 0), (int)num_slots - 1);
+}
+
 // compute units of the current device, looked up once per device (the only process-wide state of
 // the library; written with relaxed atomics, any racing writers store the same value)
 inline int device_cu_count(int* out) {

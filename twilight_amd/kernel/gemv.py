@@ -164,15 +164,17 @@ def quest_gemv_int4_top_p(q: torch.Tensor, meta: torch.Tensor, k_int4: torch.Ten
                           kv_last_page_len: torch.Tensor, token_budget: int,
                           max_pages_per_req: int, top_p, high: str = "max",
                           sm_scale: Optional[float] = None, return_scores: bool = False,
-                          meta_planes: Optional[torch.Tensor] = None):
+                          meta_planes: Optional[torch.Tensor] = None,
+                          plane_slots: Optional[torch.Tensor] = None):
     """Selector + estimator + pruner in one launch, one workgroup per (batch, head) row:
     :func:`twilight_amd.kernel.quest_select` followed by :func:`sparse_gemv_int4_top_p`
     (twilight/pyimpl/quest.py:17-122, attention.py:252-255, top_p.py:10-15, attention.py:280-281)
     with the page scores and the page list kept on chip.
 
-    ``meta_planes`` [B,Hkv,128,2,cap] (:func:`twilight_amd.kernel.meta_planes_build`) makes the
-    page-score pass read the plane layout (half the bytes; scores may differ from the record form
-    in the last bits).
+    ``meta_planes`` [slots,Hkv,128,2,cap] (:func:`twilight_amd.kernel.meta_planes_build`) makes
+    the page-score pass read the plane layout (half the bytes; scores may differ from the record
+    form in the last bits); ``plane_slots`` int32 [B] names each request's slot (default: its
+    position in the batch).
 
     Returns ``(sel_pages int32 [B,H,k], sel_count int32 [B,H], idx int32 [B,H,16k], count int32
     [B,H], cand_count int32 [B,H])``, k = budget pages clamped to ``max_pages_per_req``; with
@@ -214,12 +216,14 @@ def quest_gemv_int4_top_p(q: torch.Tensor, meta: torch.Tensor, k_int4: torch.Ten
     cap = 0
     if meta_planes is not None:
         from .kv_shadow import _check_planes
-        cap = _check_planes(meta_planes, B, Hkv, q.dtype)
+        cap = _check_planes(meta_planes, B, Hkv, q.dtype, plane_slots)
         if cap < max_pages_per_req:
             raise RuntimeError("meta_planes holds fewer pages per request than max_pages_per_req")
+    elif plane_slots is not None:
+        raise RuntimeError("plane_slots given without meta_planes")
     check_same_device(q, ("k_int4", k_int4), ("meta", meta), ("kv_page_indices", kv_page_indices),
                       ("kv_page_indptr", kv_page_indptr), ("kv_last_page_len", kv_last_page_len),
-                      ("meta_planes", meta_planes))
+                      ("meta_planes", meta_planes), ("plane_slots", plane_slots))
     dev = q.device
     with torch.cuda.device(dev):
         sel = torch.zeros((B, H, k), dtype=torch.int32, device=dev)
@@ -237,7 +241,8 @@ def quest_gemv_int4_top_p(q: torch.Tensor, meta: torch.Tensor, k_int4: torch.Ten
             ptr(kv_page_indptr), ptr(kv_last_page_len), B, H, Hkv, int(token_budget),
             int(max_pages_per_req), scale, ptr(p_arr), p_val, _high_mode(high), ptr(sel), k,
             ptr(selc), ptr(idx), M, ptr(count), ptr(ps), max_pages_per_req, ptr(scores), M,
-            ptr(cand), ptr(meta_planes), cap, stream_of(q))
+            ptr(cand), ptr(meta_planes), cap, ptr(plane_slots),
+            0 if meta_planes is None else meta_planes.size(0), stream_of(q))
     _lib.check(rc, "SelectEstimatePrune")
     out = [sel, selc, idx, count, cand]
     if return_scores:

@@ -100,10 +100,15 @@ class TwilightDecodeLayer:
         a.page_stride, a.token_stride, a.head_stride = ks[0], ks[1], ks[2]
         a.k_int4, a.meta = ptr(c.k_int4), ptr(c.meta)
         planes = getattr(c, "meta_planes", None)
-        if planes is not None and planes.size(0) >= c.batch and planes.size(4) >= c.max_pages_per_req:
+        slots = getattr(c, "plane_slots", None)
+        fits = planes is not None and planes.size(4) >= c.max_pages_per_req and \
+            (planes.size(0) >= c.batch if slots is None else slots.numel() == c.batch)
+        if fits:
             a.meta_planes, a.plane_cap_pages = ptr(planes), planes.size(4)
+            a.plane_slots, a.plane_num_slots = ptr(slots), planes.size(0)
         else:
             a.meta_planes, a.plane_cap_pages = None, 0
+            a.plane_slots, a.plane_num_slots = None, 0
         a.kv_page_indices, a.kv_page_indptr = ptr(c.kv_page_indices), ptr(c.kv_page_indptr)
         a.kv_last_page_len = ptr(c.kv_last_page_len)
         a.batch, a.num_q_heads, a.num_kv_heads = c.batch, self.H, c.num_kv_heads
@@ -138,7 +143,8 @@ class TwilightDecodeLayer:
         key = (q.data_ptr(), c.k_cache.data_ptr(), c.v_cache.data_ptr(), c.k_int4.data_ptr(),
                c.meta.data_ptr(), c.kv_page_indices.data_ptr(), c.kv_page_indptr.data_ptr(),
                c.kv_last_page_len.data_ptr(), c.max_pages_per_req,
-               0 if c.meta_planes is None else c.meta_planes.data_ptr())
+               0 if c.meta_planes is None else c.meta_planes.data_ptr(),
+               0 if c.plane_slots is None else c.plane_slots.data_ptr())
         if self._args_key != key:
             self._args, self._args_key = self._build_args(q), key
         a = self._args
