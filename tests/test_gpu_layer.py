@@ -188,17 +188,24 @@ def test_append_kernel_records_equal_bulk_build(dev, dt):
         assert torch.equal(getattr(cache, name)[ia], getattr(full, name)[ib]), name
 
 
-def test_full_size_cfg4_layer_sampled_rows_and_properties(dev):
-    # BASELINE config 4 at its full size: B=16, 32 MHA heads, ctx 32768, fp16 paged KV (shuffled
-    # pages), Quest budget 8192, p = 0.95. The oracle (dense, CPU) checks a sample of (batch, head)
-    # rows end to end; size-independent properties check every row.
-    B, H, N, budget, p = 16, 32, 32768, 8192, 0.95
+@pytest.mark.parametrize("B,H,Hkv,dt,p,planes", [
+    (16, 32, 32, torch.float16, 0.95, False),   # BASELINE config 4 (Longchat-7B shape), records
+    (16, 32, 32, torch.float16, 0.95, True),    # the same through the plane-layout metadata
+    (8, 32, 8, torch.bfloat16, 0.90, True),     # BASELINE config 5 (Llama-3-8B shape: GQA, bf16)
+])
+def test_full_size_layer_sampled_rows_and_properties(dev, B, H, Hkv, dt, p, planes):
+    # BASELINE configs 4 and 5 at their full size: ctx 32768, paged KV (shuffled pages), Quest
+    # budget 8192. The oracle (dense, CPU) checks a sample of (batch, head) rows end to end;
+    # size-independent properties check every row.
+    N, budget = 32768, 8192
     npg = N // 16
-    q, k, v, (ids, indptr, last) = synth.layer_inputs_device(B, H, H, N, torch.float16, dev, seed=3)
-    cache = PagedKVCache(B * npg, H, torch.float16, dev)
+    q, k, v, (ids, indptr, last) = synth.layer_inputs_device(B, H, Hkv, N, dt, dev, seed=3)
+    cache = PagedKVCache(B * npg, Hkv, dt, dev)
     cache.k_cache, cache.v_cache = k, v
     cache.set_page_table(ids, indptr, last)
     cache.rebuild_shadow()
+    if planes:
+        cache.enable_planes()
     layer = TwilightDecodeLayer(cache, H, token_budget=budget, top_p=p, high="max",
                                 keep_scores=True)
     out = layer(q).clone()
@@ -230,17 +237,18 @@ def test_full_size_cfg4_layer_sampled_rows_and_properties(dev):
     rng = np.random.default_rng(0)
     long_row = int(np.argmax(cnt))
     picks = sorted(set([long_row] + [int(r) for r in rng.integers(0, rows, 5)]))
-    tol = 1e-3
+    tol = 1e-3 if dt == torch.float16 else 8e-3
     compared = 0
     for r in picks:
         b, h = divmod(r, H)
+        kvh = h // (H // Hkv)
         phys = ids_c[b * npg:(b + 1) * npg].to(dev)
-        kd = k[phys, :, h].reshape(N, 128).float().cpu()[None, None]
-        vd = v[phys, :, h].reshape(N, 128).float().cpu()[None, None]
+        kd = k[phys, :, kvh].reshape(N, 128).float().cpu()[None, None]
+        vd = v[phys, :, kvh].reshape(N, 128).float().cpu()[None, None]
         qd = q[b, h].float().cpu()[None, None, None]
         ref = P.decode_layer_dense(qd, kd, vd, top_p=p, token_budget=budget,
                                    high_mode=native.HIGH_MAX, quant="storage",
-                                   prob_dtype=torch.float16)
+                                   prob_dtype=dt)
         m0 = np.zeros(N, dtype=bool)
         for pg in sel[r, :selc[r]].cpu().numpy():
             m0[pg * 16:(pg + 1) * 16] = True
@@ -253,7 +261,7 @@ def test_full_size_cfg4_layer_sampled_rows_and_properties(dev):
         assert_top_p_parity(pr, p, gm, ref["mask"].reshape(1, N).numpy(), ref["low"], margin,
                             margin_tol=5e-6)
         own = P.masked_attention(qd, kd, vd, torch.from_numpy(gm).reshape(1, 1, 1, N),
-                                 prob_dtype=torch.float16 if cnt[r] <= 128 else torch.float32)
+                                 prob_dtype=dt if cnt[r] <= 128 else torch.float32)
         assert torch.allclose(out[b, h].float().cpu(), own[0, 0, 0], rtol=tol, atol=tol), r
         compared += 1
     assert compared >= len(picks) - 1, (compared, len(picks))
