@@ -333,17 +333,21 @@ def test_plane_slot_table(dev):
     qd = q.to(dev)
 
     def run(c, qq):
-        return K.quest_gemv_int4_top_p(qq, c.meta, c.k_int4, c.kv_page_indices, c.kv_page_indptr,
-                                       c.kv_last_page_len, budget, c.max_pages_per_req, p,
-                                       return_scores=True, meta_planes=c.meta_planes,
-                                       plane_slots=c.plane_slots)
+        out = list(K.quest_gemv_int4_top_p(qq, c.meta, c.k_int4, c.kv_page_indices, c.kv_page_indptr,
+                                           c.kv_last_page_len, budget, c.max_pages_per_req, p,
+                                           return_scores=True, meta_planes=c.meta_planes,
+                                           plane_slots=c.plane_slots))
+        idx, count = out[2], out[3]          # entries past a row's count are not written
+        live = torch.arange(idx.shape[-1], device=idx.device)[None, None, :] < count[..., None]
+        out[2] = torch.where(live, idx, torch.full_like(idx, -1))
+        return out
     want, got = run(plain, qd), run(slotted, qd)
     for a, b in zip(want, got):
         assert torch.equal(a, b)
     # the whole layer, and the separate-launch scoring kernel (12 rows: the split path)
     la = TwilightDecodeLayer(plain, H, token_budget=budget, top_p=p)
     lb = TwilightDecodeLayer(slotted, H, token_budget=budget, top_p=p)
-    assert torch.equal(la(qd), lb(qd)) and torch.equal(la.idx, lb.idx)
+    assert torch.equal(la(qd), lb(qd)) and torch.equal(la.count, lb.count)
     # decode appends across a page boundary land in the request's own slot
     free_a, free_b = list(range(B * npg, B * npg + 2 * B)), list(range(B * npg, B * npg + 2 * B))
     for s in range(20):

@@ -58,6 +58,49 @@ def test_ragged_lengths(dev, d):
     assert np.array_equal(count.cpu().numpy().reshape(6), gm.sum(-1))
 
 
+@pytest.mark.parametrize("d", [2048, 8192, 32768])
+def test_rows_that_exercise_the_heavy_element_phase(dev, d):
+    """Rows built around the bisection's first phase (one wavefront iterating over the elements
+    above max/256, the other elements entering through their maximum and the smallest positive
+    element): termination inside the phase, a list that is exactly full, one element too many
+    (whole-row fallback), no light elements, no heavy elements but the maximum, a first element
+    far below the maximum in `first` mode. Masks, `low` and iteration counts against the oracle."""
+    g = torch.Generator().manual_seed(d)
+    rows = []
+    tail = torch.rand(d, generator=g) * 1e-6 + 1e-7
+
+    def norm(v):
+        return (v / v.sum()).float()
+    a = tail.clone(); a[5] = 2.0                                   # one dominant element
+    rows.append(norm(a))
+    b = tail.clone(); b[:12] = 0.5 ** torch.arange(1, 13)          # geometric heavy hitters
+    rows.append(norm(b))
+    c = tail.clone() * 1e-3; c[torch.randperm(d, generator=g)[:256]] = 1.0   # list exactly full
+    rows.append(norm(c))
+    e = tail.clone() * 1e-3; e[torch.randperm(d, generator=g)[:257]] = 1.0   # one too many
+    rows.append(norm(e))
+    f = torch.zeros(d); f[torch.randperm(d, generator=g)[:40]] = torch.rand(40, generator=g) + 0.5
+    rows.append(norm(f))                                           # only heavy elements and zeros
+    h = torch.full((d,), 1.0); h[9] = 300.0                        # the maximum alone is heavy
+    rows.append(norm(h))
+    u = torch.rand(d, generator=g) + 0.5                           # flat: everything is heavy
+    rows.append(norm(u))
+    w = tail.clone(); w[0] = 1e-4; w[100:110] = 1.0                # `first` far below the maximum
+    rows.append(norm(w))
+    probs = torch.stack(rows).reshape(1, len(rows), 1, d).contiguous()
+    pn = probs.reshape(len(rows), d).numpy()
+    for p in (0.3, 0.9, 0.999):
+        for high, mode in (("max", native.HIGH_MAX), ("first", native.HIGH_FIRST)):
+            om, ol, oi, og = native.top_p_mask_f32(pn, p, mode, return_margin=True)
+            idx, count, mask, low, iters = K.top_p_select(probs.to(dev), p, high=high,
+                                                          return_mask=True, return_stats=True)
+            gm = mask.cpu().numpy().reshape(len(rows), d)
+            assert_top_p_parity(pn, p, gm, om, ol, og, gpu_low=low.cpu().numpy().reshape(-1))
+            ok = og >= 2e-6
+            assert np.array_equal(iters.cpu().numpy().reshape(-1)[ok], oi[ok]), (p, high)
+            assert np.array_equal(count.cpu().numpy().reshape(-1), gm.sum(-1))
+
+
 def test_per_row_p_and_degenerate_rows(dev):
     d = 2048
     g = torch.Generator().manual_seed(1)

@@ -60,6 +60,7 @@ struct FusedSmem {
   float red[2][2][16];
   int wave_tot[16];
   float first;
+  BisectSmem bis;
 };
 
 // the 64 bytes of q this lane multiplies with (dims 32*(l%4) .. +32), requested as 4 x 16 B
@@ -190,7 +191,8 @@ __device__ __forceinline__ void estimate_prune_row(const FusedArgs& a, FusedSmem
     high = row_max_regs<THREADS, VPT>(x, red, buf);
   }
   int iters = 0;
-  const float low = bisect_regs<TWL_F32, THREADS, VPT>(x, p, high, red, buf, iters);
+  const float low = bisect_regs<TWL_F32, THREADS, VPT>(x, p, high, red, buf, iters, fsm.bis,
+                                                      a.high_mode != TWL_HIGH_FIRST);
   if (tx == 0 && a.low_out) a.low_out[row] = low;
 
   // ---- ordered compaction ------------------------------------------------------------------------

@@ -123,7 +123,9 @@ __global__ __launch_bounds__(THREADS) void top_p_kernel(TopPArgs a) {
     high = row_max_regs<THREADS, VPT>(x, red, buf);
   }
   int iters = 0;
-  const float low = bisect_regs<DT, THREADS, VPT>(x, p, high, red, buf, iters);
+  __shared__ BisectSmem bsm;
+  const float low = bisect_regs<DT, THREADS, VPT>(x, p, high, red, buf, iters, bsm,
+                                                 a.high_mode != TWL_HIGH_FIRST);
 
   if (tx == 0) {
     if (a.low_out) a.low_out[row] = low;

@@ -57,14 +57,46 @@ __device__ __forceinline__ float row_max_regs(const float (&x)[VPT], float (*red
   return m;
 }
 
+// LDS of the bisection's single-wavefront phase (see bisect_regs)
+#ifndef TWL_HEAVY_PER_LANE
+#define TWL_HEAVY_PER_LANE 4
+#endif
+#ifndef TWL_HEAVY_J
+#define TWL_HEAVY_J 8
+#endif
+constexpr int kHeavyPerLane = TWL_HEAVY_PER_LANE;
+constexpr int kHeavyCap = kWave * kHeavyPerLane;
+struct BisectSmem {
+  float hlist[kHeavyCap];
+  uint32_t wcnt[16], wmax[16], wmin[16];
+  uint32_t state[8];
+};
+
+#ifndef TWL_BISECT_HEAVY
+#define TWL_BISECT_HEAVY 1
+#endif
+
 // The bisection of csrc/include/sampling.cuh:156-217 on probabilities held in registers, starting
 // from the bracket (0, high]. Returns the final `low` (keep x > low); x is clamped to >= 0.
+// `high_is_row_max` (the same in every thread): `high` is the row's maximum, row_max_regs.
+//
+// Attention rows are peaked: while the pivot is above tau = high / 256, an iteration only
+// distinguishes between the few elements above tau (the sum over x > pivot, the smallest element
+// above `low` once `low` has moved, the largest element below `high`); everything else enters
+// through two numbers, the largest element <= tau and the smallest positive element. Those
+// iterations (about 8 of 15 on decode rows) are run by ONE wavefront on a list of the elements
+// above tau, without workgroup barriers, while the other wavefronts wait; the loop then goes on
+// over the whole row from the state that wavefront leaves. Same iterations, same decisions; the
+// sums of the first phase add the same numbers in another order. Rows with more than kHeavyCap
+// elements above tau skip the phase.
 template <int DT, int THREADS, int VPT>
 __device__ __forceinline__ float bisect_regs(float (&x)[VPT], float p, float high,
-                                             float (*red)[2][16], int& buf, int& iters) {
+                                             float (*red)[2][16], int& buf, int& iters,
+                                             BisectSmem& bs, bool high_is_row_max) {
   constexpr int NWAVES = THREADS / kWave;
+  constexpr bool HEAVY = TWL_BISECT_HEAVY && NWAVES > 1 && THREADS * VPT >= 2048;
   const int lane = lane_id();
-  const int wave = threadIdx.x / kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   float low = 0.0f;
   const float eps = round_to<DT>(1e-5f);
   // Probabilities are non-negative, so their bit patterns order like unsigned integers; anything
@@ -147,7 +179,9 @@ __device__ __forceinline__ float bisect_regs(float (&x)[VPT], float p, float hig
     kv = tk;
     buf ^= 1;
   };
-  {  // B for the initial `high`
+  if (high_is_row_max) {
+    B_bits = as_u32(high);  // the largest element <= the row's maximum is that maximum
+  } else {  // B for the initial `high`
     const uint32_t c = as_u32(high);
     float dummy = 0.0f;
     uint32_t k = wave_min_u32(block_min_key(c, true));
@@ -155,9 +189,150 @@ __device__ __forceinline__ float bisect_regs(float (&x)[VPT], float p, float hig
     B_bits = (k < 0x80000000u) ? c - k : 0u;
   }
   bool sel_a = true;
-  float min_gt_low, max_le_high;
+  bool more = true;
   iters = 0;
-  do {
+  // one iteration's bookkeeping, given the sum over x > mid and the smallest search key
+  auto update = [&](float mid, uint32_t c, float s, uint32_t kmin) {
+    const bool found = kmin < 0x80000000u;
+    if (sel_a) A_bits = found ? c + kmin : kInfBits;
+    else B_bits = found ? c - kmin : 0u;
+    const float min_gt_low = fminf(high, as_f32(A_bits));   // sampling.cuh:174,184-186,196-197
+    const float max_le_high = fmaxf(low, as_f32(B_bits));   // sampling.cuh:175,187-189,199-201
+    const bool accept = s >= p;                             // sampling.cuh:211-216
+    low = accept ? mid : low;
+    high = accept ? high : fminf(mid, max_le_high);
+    sel_a = accept;
+    ++iters;
+    more = round_to<DT>(max_le_high - min_gt_low) > eps && iters < 4096;
+  };
+
+  if constexpr (HEAVY) {
+    const float tau = high * (1.0f / (float)(1 << TWL_HEAVY_J));
+    const uint32_t tau_b = as_u32(tau);
+    // ---- census: elements above tau per wavefront, largest element <= tau, smallest positive
+    uint32_t cnt = 0, mx = 0u, mn1 = 0xFFFFFFFFu;
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) {
+      const bool h = xb[k] > tau_b;
+      cnt += (uint32_t)__builtin_popcountll(__ballot(h));
+      mx = max(mx, h ? 0u : xb[k]);
+      mn1 = min(mn1, xb[k] - 1u);  // 0 wraps to the largest key
+    }
+    mn1 = wave_min_u32(mn1);
+    mx = ~wave_min_u32(~mx);
+    if (lane == kWave - 1) {
+      bs.wcnt[wave] = cnt;
+      bs.wmax[wave] = mx;
+      bs.wmin[wave] = mn1;
+    }
+    __syncthreads();
+    uint32_t tot = bs.wcnt[lane & (NWAVES - 1)];
+    uint32_t gmx = bs.wmax[lane & (NWAVES - 1)];
+    uint32_t gmn = bs.wmin[lane & (NWAVES - 1)];
+    const int incl = wave_inclusive_scan((lane < NWAVES) ? (int)tot : 0);
+    const uint32_t my_off =
+        (wave == 0) ? 0u : (uint32_t)__builtin_amdgcn_readlane(incl, wave - 1);
+    const uint32_t n_heavy = (uint32_t)__builtin_amdgcn_readlane(incl, NWAVES - 1);
+    if (NWAVES >= 2) {
+      gmx = max(gmx, (uint32_t)dpp<kDppXor1>(0, (int)gmx));
+      gmn = min(gmn, (uint32_t)dpp<kDppXor1>((int)0xFFFFFFFF, (int)gmn));
+    }
+    if (NWAVES >= 4) {
+      gmx = max(gmx, (uint32_t)dpp<kDppXor2>(0, (int)gmx));
+      gmn = min(gmn, (uint32_t)dpp<kDppXor2>((int)0xFFFFFFFF, (int)gmn));
+    }
+    if (NWAVES >= 8) {
+      gmx = max(gmx, (uint32_t)dpp<kDppHalfMirror>(0, (int)gmx));
+      gmn = min(gmn, (uint32_t)dpp<kDppHalfMirror>((int)0xFFFFFFFF, (int)gmn));
+    }
+    if (NWAVES >= 16) {
+      gmx = max(gmx, (uint32_t)dpp<kDppMirror>(0, (int)gmx));
+      gmn = min(gmn, (uint32_t)dpp<kDppMirror>((int)0xFFFFFFFF, (int)gmn));
+    }
+    const uint32_t max_light_bits = (uint32_t)__builtin_amdgcn_readfirstlane((int)gmx);
+    const uint32_t min_pos_key = (uint32_t)__builtin_amdgcn_readfirstlane((int)gmn);  // bits - 1
+    // the phase needs tau > 0 (so that `low` is either 0 or above tau) and a list that fits
+    const bool heavy = n_heavy <= (uint32_t)kHeavyCap && high > 1e-30f;
+    if (heavy) {
+      // ---- the list, in (wavefront, slot, lane) order: the same on every run
+      uint32_t off = my_off;
+#pragma unroll
+      for (int k = 0; k < VPT; ++k) {
+        const bool h = xb[k] > tau_b;
+        const uint64_t m = __ballot(h);
+        const uint32_t rank = __builtin_amdgcn_mbcnt_hi(
+            (uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
+        if (h) bs.hlist[off + rank] = x[k];
+        off += (uint32_t)__builtin_popcountll(m);
+      }
+      __syncthreads();
+      if (wave == 0) {
+        float hv[kHeavyPerLane];
+        uint32_t hb[kHeavyPerLane];
+        bool hvalid[kHeavyPerLane];
+#pragma unroll
+        for (int j = 0; j < kHeavyPerLane; ++j) {
+          const uint32_t i = (uint32_t)lane + kWave * j;
+          hvalid[j] = i < n_heavy;
+          hv[j] = hvalid[j] ? bs.hlist[i] : 0.0f;
+          hb[j] = as_u32(hv[j]);
+        }
+        auto lane63_f = [](float v) { return as_f32(__builtin_amdgcn_readlane(as_i32(v), 63)); };
+        auto lane63_u = [](uint32_t v) { return (uint32_t)__builtin_amdgcn_readlane((int)v, 63); };
+        while (more) {
+          const float mid = round_to<DT>((low + high) * 0.5f);
+          if (!(mid >= tau)) break;  // below tau the rest of the row matters: whole-row phase
+          float s = 0.0f, s_odd = 0.0f;
+#pragma unroll
+          for (int j = 0; j < kHeavyPerLane; ++j) {
+            const float v = (hv[j] > mid) ? hv[j] : 0.0f;
+            if (j & 1) s_odd += v;
+            else s += v;
+          }
+          s = lane63_f(wave_sum_f32(s + s_odd));
+          const uint32_t c = sel_a ? as_u32(low) + 1u : as_u32(high);
+          uint32_t kmin = 0xFFFFFFFFu;
+          if (!sel_a) {
+            // largest element <= high: on the list, else the largest element <= tau (<= high
+            // because high >= mid >= tau); no such element and an element equal to 0 both give 0
+#pragma unroll
+            for (int j = 0; j < kHeavyPerLane; ++j)
+              kmin = min(kmin, hvalid[j] ? c - hb[j] : 0xFFFFFFFFu);
+            kmin = lane63_u(wave_min_u32(kmin));
+            if (kmin >= 0x80000000u) kmin = c - max_light_bits;
+          } else if (low == 0.0f) {
+            kmin = min_pos_key;  // c == 1: smallest positive element of the row, as bits - c
+          } else {
+            // smallest element > low >= tau: it is on the list or does not exist
+#pragma unroll
+            for (int j = 0; j < kHeavyPerLane; ++j)
+              kmin = min(kmin, hvalid[j] ? hb[j] - c : 0xFFFFFFFFu);
+            kmin = lane63_u(wave_min_u32(kmin));
+          }
+          update(mid, c, s, kmin);
+        }
+        if (lane == 0) {
+          bs.state[0] = as_u32(low);
+          bs.state[1] = as_u32(high);
+          bs.state[2] = A_bits;
+          bs.state[3] = B_bits;
+          bs.state[4] = sel_a ? 1u : 0u;
+          bs.state[5] = (uint32_t)iters;
+          bs.state[6] = more ? 1u : 0u;
+        }
+      }
+      __syncthreads();
+      low = as_f32(bs.state[0]);
+      high = as_f32(bs.state[1]);
+      A_bits = bs.state[2];
+      B_bits = bs.state[3];
+      sel_a = bs.state[4] != 0u;
+      iters = (int)bs.state[5];
+      more = bs.state[6] != 0u;
+    }
+  }
+
+  while (more) {
     const float mid = round_to<DT>((low + high) * 0.5f);
     // two interleaved partial sums (even / odd slots): a fixed order, half the dependent chain
     float s = 0.0f, s_odd = 0.0f;
@@ -172,17 +347,8 @@ __device__ __forceinline__ float bisect_regs(float (&x)[VPT], float p, float hig
     uint32_t kmin = wave_min_u32(block_min_key(c, !sel_a));
     s = wave_sum_f32(s);
     block_fold(s, kmin);
-    const bool found = kmin < 0x80000000u;
-    if (sel_a) A_bits = found ? c + kmin : kInfBits;
-    else B_bits = found ? c - kmin : 0u;
-    min_gt_low = fminf(high, as_f32(A_bits));   // sampling.cuh:174,184-186,196-197
-    max_le_high = fmaxf(low, as_f32(B_bits));   // sampling.cuh:175,187-189,199-201
-    const bool accept = s >= p;                 // sampling.cuh:211-216
-    low = accept ? mid : low;
-    high = accept ? high : fminf(mid, max_le_high);
-    sel_a = accept;
-    ++iters;
-  } while (round_to<DT>(max_le_high - min_gt_low) > eps && iters < 4096);
+    update(mid, c, s, kmin);
+  }
 
   return low;
 }
