@@ -124,6 +124,22 @@ def test_layer_dispatch_regimes(dev, B, H, Hkv, planes):
               planes=planes)
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_layer_random_shapes(dev, seed):
+    """Shapes drawn at random (batch, head counts and grouping, context with a partial last page,
+    budget, p, dtype, metadata layout, fused / split launches): every draw against the oracle."""
+    rng = np.random.default_rng(1000 + seed)
+    Hkv = int(rng.choice([1, 2, 3, 4, 8]))
+    H = Hkv * int(rng.choice([1, 1, 2, 4, 7]))
+    B = int(rng.integers(1, 9))
+    N = int(rng.integers(20, 1500))
+    budget = int(rng.choice([16, 40, 128, 300, 512, 4096]))
+    p = float(rng.choice([0.5, 0.85, 0.9, 0.95, 0.99]))
+    dt = torch.float16 if rng.random() < 0.6 else torch.bfloat16
+    _run_case(dev, B, H, Hkv, N, budget, p, dt, seed=seed, n_heavy=int(rng.integers(1, 12)),
+              fused=bool(rng.random() < 0.7), planes=bool(rng.random() < 0.5))
+
+
 def test_layer_at_128k_context(dev):
     # 8192 pages per request: the widest selector shapes (8 pages per thread in the radix select,
     # four scoring passes over the plane layout), 512 selected pages, against the dense oracle
