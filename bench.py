@@ -39,7 +39,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 QUEST_SCORE_TRAFFIC_BYTES_DEFAULT = int((131404.9 * 2.000 + 2048.0 * 1.000) * 1024)
 # The same for select_estimate_prune_kernel (FETCH_SIZE KiB x 2.000 + WRITE_SIZE KiB x 1.000).
 ROW_KERNEL_TRAFFIC_BYTES_RECORDS = int((213640.2 * 2.000 + 596.1 * 1.000) * 1024)  # --no-planes
-ROW_KERNEL_TRAFFIC_BYTES_DEFAULT = int((147987.0 * 2.000 + 596.0 * 1.000) * 1024)  # plane layout
+ROW_KERNEL_TRAFFIC_BYTES_DEFAULT = int((148008.5 * 2.000 + 596.0 * 1.000) * 1024)  # plane layout
 
 
 def _time_calls(fn, iters: int, warmup: int) -> float:
@@ -289,7 +289,7 @@ def main() -> int:
                 lambda l, c, q: lambda: L.twl_quest_page_scores_planes(
                     p(q), qcode, p(c.meta_planes), c.meta_planes.size(4), 0, 0, p(c.kv_page_indptr),
                     B, H, Hkv, npg, p(l.page_scores), npg, stream)),
-                rows * npg * 512 + rows * npg * 4 + rows * D * 2)
+                rows * npg * 256 + rows * npg * 4 + rows * D * 2)   # the sign-selected runs only
         for name, (fn, nbytes) in calls.items():
             us = _time_calls(fn, it, wu)
             kernels[name] = {"us": round(us, 2), "bytes": nbytes,
@@ -298,7 +298,7 @@ def main() -> int:
         if layers[0].cache.meta_planes is not None:
             # `bytes` above is the algorithm's figure (512 B of min/max metadata per row and
             # page); with the plane layout the kernel reads only the sign-selected half of it
-            for name in ("select_estimate_prune", "quest_score_planes"):
+            for name in ("select_estimate_prune",):
                 k = kernels.get(name)
                 if k:
                     # a (channel, plane) run stays unread when every q head of the kv head's
