@@ -180,7 +180,7 @@ __device__ __forceinline__ void estimate_prune_row(const FusedArgs& a, FusedSmem
 
   // ---- softmax + bisection in place (top_p_core.h) ---------------------------------------------
   int buf = 0;
-  softmax_regs<THREADS, VPT>(x, red, buf);
+  const float max_prob = softmax_regs<THREADS, VPT>(x, red, buf);
   const float p = a.p_arr ? a.p_arr[row] : a.p;
   float high;
   if (a.high_mode == TWL_HIGH_FIRST) {
@@ -188,7 +188,7 @@ __device__ __forceinline__ void estimate_prune_row(const FusedArgs& a, FusedSmem
     __syncthreads();
     high = first;
   } else {
-    high = row_max_regs<THREADS, VPT>(x, red, buf);
+    high = max_prob;  // the row maximum, without another reduction
   }
   int iters = 0;
   const float low = bisect_regs<TWL_F32, THREADS, VPT>(x, p, high, red, buf, iters, fsm.bis,

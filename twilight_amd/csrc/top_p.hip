@@ -96,8 +96,9 @@ __global__ __launch_bounds__(THREADS) void top_p_kernel(TopPArgs a) {
 
   int buf = 0;
   // ---- softmax in registers (fused entry) -------------------------------------------------
+  float max_prob = 0.0f;
   if (FUSED_SOFTMAX) {
-    softmax_regs<THREADS, VPT>(x, red, buf);
+    max_prob = softmax_regs<THREADS, VPT>(x, red, buf);
     if (a.probs_out) {
       float* dst = a.probs_out + (size_t)row * a.in_stride;
 #pragma unroll
@@ -119,6 +120,8 @@ __global__ __launch_bounds__(THREADS) void top_p_kernel(TopPArgs a) {
     if (tx == 0) first = (len > 0) ? x[0] : 0.0f;
     __syncthreads();
     high = first;
+  } else if (FUSED_SOFTMAX) {
+    high = max_prob;  // the row maximum, without another reduction
   } else {
     high = row_max_regs<THREADS, VPT>(x, red, buf);
   }

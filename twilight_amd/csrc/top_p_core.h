@@ -10,9 +10,13 @@
 namespace twl {
 
 // x <- softmax(x) in fp32 (twilight/pyimpl/top_p.py:11-13); -inf entries get probability 0.
+// Returns the largest probability of the row: the element(s) equal to the row maximum get
+// exp2(0) = 1 exactly and no correction, i.e. 1 * (1 / sum); every other element multiplies the
+// same 1 / sum by a factor <= 1. An empty row returns 0.
 template <int THREADS, int VPT>
-__device__ __forceinline__ void softmax_regs(float (&x)[VPT], float (*red)[2][16], int& buf) {
+__device__ __forceinline__ float softmax_regs(float (&x)[VPT], float (*red)[2][16], int& buf) {
   constexpr int NWAVES = THREADS / kWave;
+  float row_max_prob = 0.0f;
     float m = -__builtin_inff();
 #pragma unroll
     for (int k = 0; k < VPT; ++k) m = fmaxf(m, x[k]);
@@ -41,7 +45,9 @@ __device__ __forceinline__ void softmax_regs(float (&x)[VPT], float (*red)[2][16
       const float rz = 1.0f / z;
 #pragma unroll
       for (int k = 0; k < VPT; ++k) x[k] *= rz;
+      row_max_prob = rz;
     }
+    return row_max_prob;
 }
 
 // Maximum of the (non-negative) row, in every thread.
