@@ -320,6 +320,8 @@ def main() -> int:
         used = ("select_estimate_prune", "sparse_attn")
     else:
         used = (score, "quest_topk", "gemv_top_p", "sparse_attn")
+    if not row_kernel and kp == npg:
+        used = tuple(n for n in used if n != score)   # every page is kept: no scoring launch
     for name in kernels:
         kernels[name]["in_layer_step"] = name in used
     layer_bytes = sum(kernels[n]["bytes"] for n in used) if kernels else None

@@ -78,8 +78,14 @@ extern "C" int twl_decode_layer(const twl_layer_args* a, void* stream) {
     if (rc != TWL_OK) return rc;
   } else {
     // 1. Quest page scores + top-k pages; without GQA sharing the plane layout halves the read
-    if (a->meta_planes && a->num_q_heads == a->num_kv_heads &&
-        a->plane_cap_pages >= a->max_pages_per_req) {
+    if (k == a->max_pages_per_req && !a->keep_scores) {
+      // no request is longer than the budget: every page is kept, no metadata is read (the
+      // selection does not look at the scores when it keeps everything)
+      rc = twl_quest_topk_pages(page_scores, ps_stride, a->kv_page_indptr, a->batch,
+                                a->num_q_heads, a->token_budget, a->max_pages_per_req,
+                                a->sel_pages, a->sel_stride, a->sel_count, stream);
+    } else if (a->meta_planes && a->num_q_heads == a->num_kv_heads &&
+               a->plane_cap_pages >= a->max_pages_per_req) {
       rc = twl_quest_page_scores_planes(a->q, a->dtype, a->meta_planes, a->plane_cap_pages,
                                         a->plane_slots, a->plane_num_slots, a->kv_page_indptr, a->batch, a->num_q_heads,
                                         a->num_kv_heads, a->max_pages_per_req, page_scores,

@@ -88,6 +88,10 @@ __global__ __launch_bounds__(kRowThreads) void select_estimate_prune_kernel(RowA
   }
   const int req_pages = pg_end - pg_begin;
   const int n_req = min(max(req_pages, 0), min((int)a.max_pages_req, kRowThreads * SEL_VPT));
+  const int sel_n = min(min(quest_budget_pages(a.token_budget), n_req), (int)a.f.max_pages);
+  // a request no longer than the budget keeps every page: its metadata is not read at all (unless
+  // the caller asked for the page scores)
+  const int n_score = (sel_n < n_req || a.page_scores_out) ? n_req : 0;
 
   // ---- 1. Quest page scores into LDS ---------------------------------------------------------
   if constexpr (PLANES) {
@@ -102,7 +106,7 @@ __global__ __launch_bounds__(kRowThreads) void select_estimate_prune_kernel(RowA
 #pragma unroll
     for (int pass = 0; pass < PL_PASSES; ++pass) {
       const int w0 = (pass * kRowWaves + wave) * 128;  // first page of this wave's slice
-      if (w0 < n_req) {                                // wave-uniform
+      if (w0 < n_score) {                                // wave-uniform
         const int pg0 = w0 + 2 * lane;                 // this lane's two pages
         const int pgc = min(pg0, (int)a.plane_cap - 2);  // loads stay inside the run
         float s0 = 0.0f, s1 = 0.0f;
@@ -116,12 +120,12 @@ __global__ __launch_bounds__(kRowThreads) void select_estimate_prune_kernel(RowA
           s0 = fmaf(qd, bits16_to_f32<QDT>(w & 0xFFFFu), s0);
           s1 = fmaf(qd, bits16_to_f32<QDT>(w >> 16), s1);
         }
-        if (pg0 < n_req) ps_lds[pg0] = s0;
-        if (pg0 + 1 < n_req) ps_lds[pg0 + 1] = s1;
+        if (pg0 < n_score) ps_lds[pg0] = s0;
+        if (pg0 + 1 < n_score) ps_lds[pg0 + 1] = s1;
         if (a.page_scores_out) {
           float* po = a.page_scores_out + (size_t)row * a.page_score_stride;
-          if (pg0 < n_req) po[pg0] = s0;
-          if (pg0 + 1 < n_req) po[pg0 + 1] = s1;
+          if (pg0 < n_score) po[pg0] = s0;
+          if (pg0 + 1 < n_score) po[pg0 + 1] = s1;
         }
       }
     }
@@ -132,7 +136,7 @@ __global__ __launch_bounds__(kRowThreads) void select_estimate_prune_kernel(RowA
 #pragma unroll
     for (int r = 0; r < SEL_VPT; ++r) {
       const int pg = ((2 * r + half) * kRowWaves + wave) * 32 + c;
-      ids[r] = (pg < n_req) ? a.f.kv_page_indices[pg_begin + pg] : 0;
+      ids[r] = (pg < n_score) ? a.f.kv_page_indices[pg_begin + pg] : 0;
     }
     float qf[4];
     uint32_t selmask[2];
@@ -147,7 +151,7 @@ __global__ __launch_bounds__(kRowThreads) void select_estimate_prune_kernel(RowA
 #pragma unroll
     for (int pass = 0; pass < PASSES; ++pass) {
       const int p0 = (pass * kRowWaves + wave) * 32;
-      const int np = min(32, n_req - p0);  // wave-uniform
+      const int np = min(32, n_score - p0);  // wave-uniform
       if (np > 0) {
         const int lbase = (pass & 1) * 32;
         float keep = 0.0f;  // lane i ends up with the score of page p0 + i
@@ -202,7 +206,6 @@ __global__ __launch_bounds__(kRowThreads) void select_estimate_prune_kernel(RowA
   __syncthreads();
 
   // ---- 2. top-k pages: list to LDS (and to memory for the caller) ----------------------------
-  const int sel_n = min(min(quest_budget_pages(a.token_budget), n_req), (int)a.f.max_pages);
   if (threadIdx.x == 0) a.sel_count_out[row] = sel_n;
   if (sel_n > 0)
     select_row_topk<kRowThreads, SEL_VPT>(ps_lds, n_req, sel_n,
