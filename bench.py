@@ -327,7 +327,12 @@ def main() -> int:
     layer_bytes = sum(kernels[n]["bytes"] for n in used) if kernels else None
     # dominant kernel of the step: the one-launch selector + estimator + pruner when the step
     # uses it, else the metadata stream
-    dom_name = "select_estimate_prune" if (kernels and "select_estimate_prune" in used) else score
+    if "select_estimate_prune" in used:
+        dom_name = "select_estimate_prune"
+    elif score in used:
+        dom_name = score
+    else:                                    # no scoring launch: the INT4 stream dominates
+        dom_name = "gemv_top_p" if "gemv_top_p" in used else "gemv_int4"
     dom = kernels.get(dom_name)
     roofline = None
     if dom:
@@ -343,9 +348,8 @@ def main() -> int:
             else:
                 traffic = ROW_KERNEL_TRAFFIC_BYTES_RECORDS
         roofline = {"bound": "hbm",
-                    "kernel": ("select_estimate_prune_kernel" if dom_name == "select_estimate_prune"
-                               else ("quest_score_planes_kernel" if dom_name == "quest_score_planes"
-                                     else "quest_score_kernel")),
+                    "kernel": ("quest_score_kernel" if dom_name == "quest_score"
+                               else dom_name + "_kernel"),
                     "achieved": dom["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                     "frac": dom["frac_of_hbm_peak"], "bytes_per_launch": dom["bytes"],
                     "us_per_launch": dom["us"], "traffic": traffic}
