@@ -183,7 +183,7 @@ def test_ftka_shaped_entry(dev):
 
 @pytest.mark.parametrize("paged", [False, True])
 def test_gemv_full_size_cfg2_sampled_and_linear(dev, paged):
-    # BASELINE config 2 shape: B=8, H=32, 32768 candidates per head. The oracle checks a sample of
+    # the stand-alone GEMV benchmark shape: B=8, H=32, 32768 candidates per head. The oracle checks a sample of
     # (row, page) pairs; linearity in q checks every output: f(q1) + f(q2) == f(q1 + q2) when q1, q2
     # have disjoint supports (exact up to fp32 accumulation order).
     B, H, npg = 8, 32, 2048

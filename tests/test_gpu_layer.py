@@ -81,7 +81,7 @@ def _run_case(dev, B, H, Hkv, N, budget, p, dt, seed, shuffle=True, n_heavy=16, 
 
 @pytest.mark.parametrize("fused", [True, False])
 def test_cfg1_full_context(dev, fused):
-    # BASELINE config 1: B=1, 32 heads MHA, D=128, N=4096, 16 heavy hitters with ~60 % of the mass,
+    # the reference's CPU-runnable case: B=1, 32 heads MHA, D=128, N=4096, 16 heavy hitters with ~60 % of the mass,
     # all tokens are candidates, p = 0.95
     layer, ref = _run_case(dev, 1, 32, 32, 4096, 4096, 0.95, torch.float16, seed=0, fused=fused)
     cnt = layer.count.cpu().float()
@@ -205,12 +205,12 @@ def test_append_kernel_records_equal_bulk_build(dev, dt):
 
 
 @pytest.mark.parametrize("B,H,Hkv,dt,p,planes", [
-    (16, 32, 32, torch.float16, 0.95, False),   # BASELINE config 4 (Longchat-7B shape), records
+    (16, 32, 32, torch.float16, 0.95, False),   # Longchat-7B shape (32 MHA heads, fp16), records
     (16, 32, 32, torch.float16, 0.95, True),    # the same through the plane-layout metadata
-    (8, 32, 8, torch.bfloat16, 0.90, True),     # BASELINE config 5 (Llama-3-8B shape: GQA, bf16)
+    (8, 32, 8, torch.bfloat16, 0.90, True),     # Llama-3-8B shape (32 q / 8 kv heads, bf16)
 ])
 def test_full_size_layer_sampled_rows_and_properties(dev, B, H, Hkv, dt, p, planes):
-    # BASELINE configs 4 and 5 at their full size: ctx 32768, paged KV (shuffled pages), Quest
+    # The two model shapes of the headline benchmark at their full size: ctx 32768, paged KV (shuffled pages), Quest
     # budget 8192. The oracle (dense, CPU) checks a sample of (batch, head) rows end to end;
     # size-independent properties check every row.
     N, budget = 32768, 8192

@@ -20,7 +20,7 @@ def _softmax(x):
 @pytest.mark.parametrize("p", [0.85, 0.95])
 @pytest.mark.parametrize("first_is_max", [True, False])
 def test_mask_dropin_cfg3(dev, p, first_is_max):
-    # BASELINE config 3: [8, 32, 8192] Zipf-spiked rows
+    # the pruner-alone benchmark shape: [8, 32, 8192] Zipf-spiked rows
     x = synth.topp_scores(8, 32, 8192, seed=0, first_is_max=first_is_max)
     probs = _softmax(x).reshape(8, 32, 1, 8192)
     pn = probs.reshape(256, 8192).numpy()
