@@ -1,5 +1,7 @@
 """End-to-end GPU parity of the decode layer (select -> INT4 estimate -> top-p -> attention)
 against the oracle's dense-masked restatement of twilight/pyimpl/attention.py:188-306."""
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -124,7 +126,7 @@ def test_layer_dispatch_regimes(dev, B, H, Hkv, planes):
               planes=planes)
 
 
-@pytest.mark.parametrize("seed", range(12))
+@pytest.mark.parametrize("seed", range(int(os.environ.get("TWL_RANDOM_SHAPES", "12"))))
 def test_layer_random_shapes(dev, seed):
     """Shapes drawn at random (batch, head counts and grouping, context with a partial last page,
     budget, p, dtype, metadata layout, fused / split launches): every draw against the oracle."""
@@ -132,7 +134,7 @@ def test_layer_random_shapes(dev, seed):
     Hkv = int(rng.choice([1, 2, 3, 4, 8]))
     H = Hkv * int(rng.choice([1, 1, 2, 4, 7]))
     B = int(rng.integers(1, 9))
-    N = int(rng.integers(20, 1500))
+    N = int(rng.integers(20, 1500)) if seed % 3 else int(rng.integers(1500, 9000))
     budget = int(rng.choice([16, 40, 128, 300, 512, 4096]))
     p = float(rng.choice([0.5, 0.85, 0.9, 0.95, 0.99]))
     dt = torch.float16 if rng.random() < 0.6 else torch.bfloat16
