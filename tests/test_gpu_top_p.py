@@ -1,5 +1,7 @@
 """GPU parity of the top-p pruner (through the C-ABI) against the oracle's restatement of
 csrc/include/sampling.cuh:156-231 and twilight/pyimpl/top_p.py:10-15."""
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -99,6 +101,50 @@ def test_rows_that_exercise_the_heavy_element_phase(dev, d):
             ok = og >= 2e-6
             assert np.array_equal(iters.cpu().numpy().reshape(-1)[ok], oi[ok]), (p, high)
             assert np.array_equal(count.cpu().numpy().reshape(-1), gm.sum(-1))
+
+
+@pytest.mark.parametrize("seed", range(int(os.environ.get("TWL_RANDOM_SHAPES", "12"))))
+def test_random_rows(dev, seed):
+    """Row length, sharpness, number and weight of spikes, zeros, p and the `high` mode drawn at
+    random: masks, `low` and iteration counts against the oracle."""
+    rng = np.random.default_rng(500 + seed)
+    d = int(rng.choice([int(rng.integers(1, 300)), int(rng.integers(300, 5000)),
+                        int(rng.integers(5000, 32769))]))
+    rows = int(rng.integers(1, 9))
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn((rows, d), generator=g) * float(rng.choice([0.3, 1.0, 3.0, 8.0]))
+    for r in range(rows):
+        n_spike = int(rng.integers(0, min(d, 40) + 1))
+        if n_spike:
+            pos = torch.randperm(d, generator=g)[:n_spike]
+            x[r, pos] += float(rng.choice([2.0, 6.0, 12.0])) * torch.rand(n_spike, generator=g)
+        if rng.random() < 0.3:                     # masked candidates: probability exactly 0
+            x[r, torch.rand(d, generator=g) < 0.4] = float("-inf")
+            x[r, int(rng.integers(0, d))] = 0.0    # at least one live element
+    probs = _softmax(x).reshape(1, rows, 1, d).contiguous()
+    pn = probs.reshape(rows, d).numpy()
+    p = float(rng.choice([0.1, 0.5, 0.85, 0.9, 0.95, 0.99, 1.0]))
+    high, mode = (("max", native.HIGH_MAX) if rng.random() < 0.6 else ("first", native.HIGH_FIRST))
+    om, ol, oi, og = native.top_p_mask_f32(pn, p, mode, return_margin=True)
+    idx, count, mask, low, iters = K.top_p_select(probs.to(dev), p, high=high, return_mask=True,
+                                                  return_stats=True)
+    gm = mask.cpu().numpy().reshape(rows, d)
+    assert_top_p_parity(pn, p, gm, om, ol, og, gpu_low=low.cpu().numpy().reshape(-1))
+    ok = og >= 2e-6
+    assert np.array_equal(iters.cpu().numpy().reshape(-1)[ok], oi[ok])
+    assert np.array_equal(count.cpu().numpy().reshape(-1), gm.sum(-1))
+    # the fused softmax + top-p entry on the raw scores of the same rows (top_p.py:10-15)
+    idx2, count2, probs2 = K.softmax_top_p(x.reshape(1, rows, d).contiguous().to(dev), p, high=high,
+                                           return_probs=True)
+    # fp32 normalisers of up to 32768 terms, summed in different orders: a common factor per row
+    np.testing.assert_allclose(probs2.cpu().numpy().reshape(rows, d), pn, rtol=1e-5, atol=1e-12)
+    gm2 = np.zeros((rows, d), dtype=bool)
+    c2 = count2.cpu().numpy().reshape(-1)
+    i2 = idx2.cpu().numpy().reshape(rows, d)
+    for r in range(rows):
+        assert np.all(np.diff(i2[r, :c2[r]]) > 0)
+        gm2[r, i2[r, :c2[r]]] = True
+    assert_top_p_parity(pn, p, gm2, om, ol, og, margin_tol=5e-6)
 
 
 def test_per_row_p_and_degenerate_rows(dev):
