@@ -135,6 +135,103 @@ def bench_topp(args, L, dev) -> int:
     return 0
 
 
+def bench_ftka(args, dev) -> int:
+    """The GEMV call shapes of benchmark/efficiency/bench_gemv.py (32 heads, head_dim 128, token
+    pages, page lists shared by the heads of a request) and the Double-Sparse label ops, at batch
+    8 and 32768 tokens per request. Unlike the reference's bench every request has pages of its own
+    (its requests all point at the same 32768 pages, which a cache then serves 7 times out of 8)
+    and two caches are visited in turn, so every call streams cold data."""
+    import twilight_amd.kernel as K
+    B, H, D, N = args.batch, 32, 128, args.context
+    g = torch.Generator(device=dev); g.manual_seed(0)
+    pages = B * N
+    idx = torch.arange(pages, dtype=torch.int32, device=dev)
+    indptr = (torch.arange(B + 1, dtype=torch.int32) * N).to(dev)
+    last = torch.ones(B, dtype=torch.int32, device=dev)
+    q = torch.randn((B, H, D), device=dev, generator=g, dtype=torch.float16)
+    res = {}
+
+    def timed(name, make, nbytes, note=None):
+        fns = [make(i) for i in range(2)]
+        state = {"i": 0}
+
+        def call():
+            fns[state["i"] & 1]()
+            state["i"] += 1
+        us = _time_calls(call, max(args.steps // 4, 20), 4)
+        res[name] = {"us": round(us, 2), "bytes": nbytes, "GBps": round(nbytes / us / 1e3, 1),
+                     "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+        if note:
+            res[name]["note"] = note
+
+    # fp16 K (bench_gemv.py:191-247)
+    k16 = [torch.randn((pages, 1, H, D), device=dev, generator=g, dtype=torch.float16) for _ in range(2)]
+    o16 = torch.empty((B, H, 1, N), dtype=torch.float16, device=dev)
+    timed("batched_sparse_gemv", lambda i: lambda: K.batched_sparse_gemv(q, o16, k16[i], idx, indptr, last),
+          pages * H * D * 2 + B * H * N * 2 + pages * 4)
+    del k16
+    # int8 K + per-token scale / zero (bench_gemv.py:67-147)
+    k8 = [torch.randint(0, 256, (pages, 1, H, D), device=dev, generator=g, dtype=torch.uint8) for _ in range(2)]
+    sc = [torch.rand((pages, 1, H), device=dev, generator=g).half() * 0.02 + 0.001 for _ in range(2)]
+    zr = [torch.randn((pages, 1, H), device=dev, generator=g).half() * 0.1 for _ in range(2)]
+    o8 = torch.empty((B, H, N), dtype=torch.float16, device=dev)
+    timed("batched_sparse_gemv_int8_k",
+          lambda i: lambda: K.batched_sparse_gemv_int8_k(q, o8, k8[i], sc[i], zr[i], idx, indptr, last),
+          pages * H * (D + 4) + B * H * N * 2 + pages * 4)
+    del k8
+    # int4 K, two nibbles per byte (bench_gemv.py:377-454)
+    k4 = [torch.randint(0, 256, (pages, 1, H, D // 2), device=dev, generator=g, dtype=torch.uint8) for _ in range(2)]
+    timed("batched_sparse_gemv_int4_k",
+          lambda i: lambda: K.batched_sparse_gemv_int4_k(q, o8, k4[i], sc[i], zr[i], idx, indptr, last),
+          pages * H * (D // 2 + 4) + B * H * N * 2 + pages * 4)
+    del k4, sc, zr
+    # one request, contiguous K (bench_gemv.py:13-53; its largest length is 16384)
+    ks = [torch.randn((16384, H, D), device=dev, generator=g, dtype=torch.float16) for _ in range(2)]
+    os_ = torch.empty((H, 16384), dtype=torch.float16, device=dev)
+    timed("single_sparse_gemv", lambda i: lambda: K.single_sparse_gemv(q[0], os_, ks[i]),
+          16384 * H * D * 2 + H * 16384 * 2, note="one request of 16384 tokens")
+    del ks
+    # Double-Sparse label ops (twilight/pyimpl/double_sparse.py:17): 16 heavy channels
+    r = 16
+    chan = torch.stack([torch.randperm(D, device=dev, generator=g)[:r] for _ in range(H)]).to(torch.int64)
+    xk = [torch.randn((B * N, H, D), device=dev, generator=g, dtype=torch.float16) for _ in range(2)]
+    lab = torch.empty((B * N, H, r), dtype=torch.float16, device=dev)
+    timed("get_label_tensor", lambda i: lambda: K.get_label_tensor(xk[i], chan, lab, r),
+          B * N * H * r * 2 * 2, note="gather of 16 of 128 channels: counts the bytes it needs, "
+                                       "32-byte sectors of 256-byte rows are what it touches")
+    del xk
+    ql = torch.randn((B, H, r), device=dev, generator=g, dtype=torch.float16)
+    kl = [torch.randint(-128, 128, (B * N, H, r), device=dev, generator=g, dtype=torch.int8) for _ in range(2)]
+    ksc = [torch.rand((B * N, H), device=dev, generator=g).half() for _ in range(2)]
+    ob = torch.empty((B, H, N), dtype=torch.float16, device=dev)
+    timed("bgemv_int8", lambda i: lambda: K.bgemv_int8(ql, kl[i], ksc[i], ob),
+          B * N * H * (r + 2) + B * H * N * 2)
+    del kl, ksc
+    # per-block int8 QK^T log-sum-exp, prefill shape (qk_int8_per_block.py:111-143)
+    bq, hq, nq = 1, 32, 4096
+    qi = torch.randint(-128, 128, (bq, hq, nq, D), device=dev, generator=g, dtype=torch.int8)
+    ki = torch.randint(-128, 128, (bq, hq, nq, D), device=dev, generator=g, dtype=torch.int8)
+    qs = torch.rand((bq, hq, nq // 128), device=dev, generator=g) * 0.01
+    kss = torch.rand((bq, hq, nq // 64), device=dev, generator=g) * 0.01
+    us = _time_calls(lambda: K.qk_int8_per_block(qi, ki, qs, kss, return_lse=True), 20, 3)
+    ops = 2.0 * bq * hq * nq * nq * D
+    res["qk_int8_per_block"] = {"us": round(us, 2), "int8_TOPs": round(ops / us / 1e6, 1),
+                                "frac_of_int8_mfma_peak": round(ops / us / 1e6 / 5000.0, 4),
+                                "note": "1 x 32 heads x 4096 x 4096 x 128, includes allocating and "
+                                        "zeroing the reference's first output"}
+    line = {"metric": "us per call, ftka GEMV call shapes and Double-Sparse ops",
+            "value": res["batched_sparse_gemv_int4_k"]["us"], "unit": "us", "n_gpus": 1,
+            "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": round(res["batched_sparse_gemv_int4_k"]["us"] / 1e3, 5),
+            "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+            "data": "synthetic",
+            "config": {"workload": f"ftka-shaped GEMVs and label ops, B={B}, 32 heads, head_dim 128, "
+                                   f"{N} tokens per request, token pages; value = the INT4 GEMV"},
+            "ops": res}
+    print(json.dumps(line))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -144,10 +241,12 @@ def main() -> int:
     ap.add_argument("--context", type=int, default=32768)
     ap.add_argument("--budget", type=int, default=8192)
     ap.add_argument("--top-p", type=float, default=0.95)
-    ap.add_argument("--workload", choices=["longchat", "llama3", "topp"], default="longchat",
+    ap.add_argument("--workload", choices=["longchat", "llama3", "topp", "ftka"], default="longchat",
                     help="longchat: 32 MHA heads fp16 (the headline workload); llama3: GQA 32/8 "
                          "bf16, with a dense-decode baseline (the same attention kernel over "
-                         "every token); topp: the pruner kernel alone on [8,32,8192] scores")
+                         "every token); topp: the pruner kernel alone on [8,32,8192] scores; "
+                         "ftka: the NHD GEMV call shapes of the reference's bench_gemv.py and the "
+                         "Double-Sparse label ops")
     ap.add_argument("--layers", type=int, default=4,
                     help="independent layer caches visited round-robin (cold-cache steps)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -178,6 +277,8 @@ def main() -> int:
     torch.cuda.set_device(dev)
     if args.workload == "topp":
         return bench_topp(args, L, dev)
+    if args.workload == "ftka":
+        return bench_ftka(args, dev)
     llama = args.workload == "llama3"
     B, H, Hkv, N, D = args.batch, 32, (8 if llama else 32), args.context, 128
     npg = N // 16

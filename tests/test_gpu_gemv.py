@@ -151,9 +151,10 @@ def test_gemv_matches_quantised_k_of_a_real_cache(dev):
     assert np.all(np.isneginf(got[:, 1000:]))
 
 
-def test_ftka_shaped_entry(dev):
+@pytest.mark.parametrize("H", [4, 6, 32])   # 6: a head count that does not divide the workgroup
+def test_ftka_shaped_entry(dev, H):
     # call shape of benchmark/efficiency/bench_gemv.py:445-454: NHD uint8 cache, per-token scale/zero
-    B, H, page_size, pages = 2, 4, 4, 30
+    B, page_size, pages = 2, 4, 30
     g = torch.Generator().manual_seed(10)
     k_u8 = torch.randint(0, 256, (pages, page_size, H, 64), dtype=torch.uint8, generator=g)
     scales = (torch.rand((pages, page_size, H), generator=g) * 0.1 + 0.01).half()
@@ -210,10 +211,11 @@ def test_gemv_full_size_cfg2_sampled_and_linear(dev, paged):
     assert err < 2e-5, err
 
 
-def test_ftka_shaped_fp16_int8_and_single_entries(dev):
+@pytest.mark.parametrize("H", [4, 6, 32])
+def test_ftka_shaped_fp16_int8_and_single_entries(dev, H):
     # call shapes of benchmark/efficiency/bench_gemv.py:33 (single), :135-144 (int8), :234-241 (fp16);
     # the references there are plain matmuls (:36-42, :181, :259-296)
-    B, H, page_size, pages = 2, 4, 2, 40
+    B, page_size, pages = 2, 2, 40
     g = torch.Generator().manual_seed(12)
     q = torch.randn((B, H, 128), generator=g).half()
     k16 = torch.randn((pages, page_size, H, 128), generator=g).half()
