@@ -44,6 +44,31 @@ def test_bgemv_int8_reference_selftest_shape(dev):
     assert torch.allclose(out.cpu().float(), ref, atol=1e-3, rtol=0)
 
 
+@pytest.mark.parametrize("B,H,N,r", [
+    (2, 32, 1000, 16),     # the Double-Sparse shape: 32 heads, 16 heavy channels; partial last tile
+    (3, 8, 517, 32),       # two 16-byte pieces per head
+    (1, 16, 2051, 64),     # four pieces per head
+    (2, 64, 300, 8),       # 8-byte pieces, more pieces per token than threads
+    (1, 4, 77, 16),        # fewer pieces per token than a wavefront
+])
+def test_bgemv_int8_dense_layout(dev, B, H, N, r):
+    # dense operands take the streaming kernel (strided ones the general one): same numbers
+    g = torch.Generator().manual_seed(B * N + r)
+    q = torch.randn((B, H, r), generator=g).half()
+    k8 = torch.randint(-128, 128, (B * N, H, r), generator=g, dtype=torch.int16).to(torch.int8)
+    scales = (torch.rand((B * N, H), generator=g) * 0.01).half()
+    out = torch.full((B, H, N), 5.0, dtype=torch.float16, device=dev)
+    K.bgemv_int8(q.to(dev), k8.to(dev), scales.to(dev), out)
+    ref = P.bgemv_int8_ref(q, k8, scales)
+    assert torch.allclose(out.cpu().float(), ref, atol=2e-3, rtol=2e-3)
+    # the same through strided views (general kernel)
+    kpad = torch.zeros((B * N, H, r + 3), dtype=torch.int8)
+    kpad[..., :r] = k8
+    out2 = torch.empty((B, H, N), dtype=torch.float16, device=dev)
+    K.bgemv_int8(q.to(dev), kpad.to(dev)[..., :r], scales.to(dev), out2)
+    assert torch.allclose(out2.cpu().float(), out.cpu().float(), atol=1e-3, rtol=1e-3)
+
+
 def test_bgemv_int8_ragged(dev):
     B, H, N, r = 3, 5, 131, 16
     g = torch.Generator().manual_seed(1)
