@@ -197,8 +197,8 @@ def bench_ftka(args, dev) -> int:
     xk = [torch.randn((B * N, H, D), device=dev, generator=g, dtype=torch.float16) for _ in range(2)]
     lab = torch.empty((B * N, H, r), dtype=torch.float16, device=dev)
     timed("get_label_tensor", lambda i: lambda: K.get_label_tensor(xk[i], chan, lab, r),
-          B * N * H * r * 2 * 2, note="gather of 16 of 128 channels: counts the bytes it needs, "
-                                       "32-byte sectors of 256-byte rows are what it touches")
+          B * N * H * (D + r) * 2, note="16 of 128 channels at random positions touch every "
+                                        "32-byte sector of a 256-byte row: the rows are counted whole")
     del xk
     ql = torch.randn((B, H, r), device=dev, generator=g, dtype=torch.float16)
     kl = [torch.randint(-128, 128, (B * N, H, r), device=dev, generator=g, dtype=torch.int8) for _ in range(2)]

@@ -35,6 +35,47 @@ __global__ __launch_bounds__(256) void get_label_tensor_kernel(LabelArgs a) {
   }
 }
 
+// Dense 16-bit X [L][H][D]: rows are read whole and coalesced (the channels of a head are spread
+// over the row, so every 32-byte sector of it is touched anyway), parked in LDS and picked from
+// there; Out [L][H][r] leaves in memory order. Measured against the element-wise gather above at
+// 262144 x 32 rows of 128 channels, 16 picked: 490 -> 423 us (5.7 TB/s over the rows and the output).
+constexpr int kLabRows = 32;  // (l, h) rows per tile
+
+struct LabelFastArgs {
+  const uint16_t* x;
+  const int64_t* channel;
+  uint16_t* out;
+  int64_t sc_h, sc_c;
+  uint64_t rows;  // L * H
+  uint32_t H, r, D;
+};
+
+__global__ __launch_bounds__(256) void get_label_tensor_rows_kernel(LabelFastArgs a) {
+  extern __shared__ __align__(16) uint8_t smem[];
+  uint16_t* chan = (uint16_t*)smem;                 // [H][r] channel numbers
+  uint16_t* tile = chan + ((a.H * a.r + 7u) & ~7u); // [kLabRows][D]
+  const uint32_t tid = threadIdx.x;
+  for (uint32_t i = tid; i < a.H * a.r; i += 256) {
+    const uint32_t h = i / a.r, c = i - h * a.r;
+    chan[i] = (uint16_t)a.channel[h * a.sc_h + c * a.sc_c];
+  }
+  const uint32_t ppr = a.D / 8;  // 16-byte pieces per row
+  const uint64_t tiles = (a.rows + kLabRows - 1) / kLabRows;
+  for (uint64_t tl = blockIdx.x; tl < tiles; tl += gridDim.x) {
+    const uint64_t row0 = tl * kLabRows;
+    const uint32_t nr = (uint32_t)min((uint64_t)kLabRows, a.rows - row0);
+    __syncthreads();  // the previous tile has been read (first round: the channel table is there)
+    for (uint32_t i = tid; i < nr * ppr; i += 256)
+      ((u32x4*)tile)[i] = __builtin_nontemporal_load((const u32x4*)(a.x + row0 * a.D) + i);
+    __syncthreads();
+    for (uint32_t i = tid; i < nr * a.r; i += 256) {
+      const uint32_t rw = i / a.r, c = i - rw * a.r;
+      const uint32_t h = (uint32_t)((row0 + rw) % a.H);
+      a.out[row0 * a.r + i] = tile[rw * a.D + chan[h * a.r + c]];
+    }
+  }
+}
+
 struct BgemvArgs {
   const uint16_t* q;       // fp16 [B,H,r]
   const int8_t* k;         // int8 [B*N,H,r]
@@ -190,6 +231,21 @@ extern "C" int twl_get_label_tensor(const void* x, const int64_t* channel, void*
   if (L == 0 || H == 0 || r == 0) return TWL_EINVAL;
   if ((((uintptr_t)x) | ((uintptr_t)out)) & (elem_bytes - 1)) return TWL_EALIGN;
   if (((uintptr_t)channel) & 7u) return TWL_EALIGN;
+  // dense 16-bit rows of D = sx_h channels (a multiple of 8, so that rows are 16-byte pieces)
+  const bool dense = elem_bytes == 2 && sx_d == 1 && H > 1 && sx_h > 0 && sx_h <= 1024 &&
+                     (sx_h & 7) == 0 && sx_l == (int64_t)H * sx_h && so_c == 1 &&
+                     so_h == (int64_t)r && so_l == (int64_t)H * r && r <= (uint32_t)sx_h &&
+                     (uint64_t)H * r <= 16384 && (((uintptr_t)x) & 15u) == 0;
+  if (dense) {
+    twl::LabelFastArgs f{(const uint16_t*)x, channel, (uint16_t*)out, sc_h, sc_c,
+                         (uint64_t)L * H, H, r, (uint32_t)sx_h};
+    const uint64_t tiles = (f.rows + twl::kLabRows - 1) / twl::kLabRows;
+    const uint32_t blocks = (uint32_t)(tiles < 8192 ? tiles : 8192);
+    const size_t lds = (((size_t)H * r + 7) & ~(size_t)7) * 2 + (size_t)twl::kLabRows * f.D * 2;
+    hipLaunchKernelGGL(twl::get_label_tensor_rows_kernel, dim3(blocks), dim3(256), lds,
+                       (hipStream_t)stream, f);
+    return hipGetLastError() == hipSuccess ? TWL_OK : TWL_ELAUNCH;
+  }
   twl::LabelArgs a{x, channel, out, sx_l, sx_h, sx_d, sc_h, sc_c, so_l, so_h, so_c, L, H, r};
   const uint64_t total = (uint64_t)L * H * r;
   const uint32_t blocks = (uint32_t)((total + 255) / 256 < 65536 ? (total + 255) / 256 : 65536);
