@@ -10,7 +10,7 @@
 // (masked tl.load, :36-37) and therefore count as s = 0; the same is done here.
 //
 // Tiling: a workgroup of 4 wavefronts takes 128 query rows (the q_scale block), a wavefront 32 of
-// them. Products run on v_mfma_i32_32x32x32_i8 with the KEY tile as the A operand (rows of the
+// them; the key tile of a block goes through LDS once for all four. Products run on v_mfma_i32_32x32x32_i8 with the KEY tile as the A operand (rows of the
 // product) and the wave's 32 queries as the B operand (columns), so a lane's 16 accumulators all
 // belong to ONE query (column = lane % 32) and the running (max, sum) of the online softmax lives
 // per lane without any cross-lane traffic; the two lane halves of a query are merged once at the
@@ -61,41 +61,83 @@ __global__ __launch_bounds__(256) void qk_int8_lse_kernel(QkArgs a) {
     for (int kc = 0; kc < KC; ++kc)
       qb[kc] = (m < a.qo_len) ? *(const v4i*)(qrow + 32 * kc) : v4i{0, 0, 0, 0};
   }
-  const int8_t* kbase = a.k + b * a.sk_b + kvh * a.sk_h + 16 * g;
+  // The key tile of a block (64 keys x HEAD_DIM bytes) is fetched once per workgroup and shared by
+  // its four wavefronts through LDS, double-buffered: the next tile is requested before this one
+  // is multiplied and stored after, one barrier per block. (Every wavefront fetching the tile for
+  // itself made the kernel wait on the L2: 4x the traffic.) Rows are padded by 16 bytes so that
+  // the 32 rows an operand load touches spread over the banks.
+  constexpr int ROW = HEAD_DIM + 16;
+  constexpr int PPK = HEAD_DIM / 16;               // 16-byte pieces per key
+  constexpr int PPT = kQkBlockN * PPK / 256;       // pieces per thread and tile (1 or 2)
+  __shared__ __align__(16) int8_t ktile[2][kQkBlockN][ROW];
+  const int8_t* kbase = a.k + b * a.sk_b + kvh * a.sk_h;
+  v4i stage[PPT];
+  auto fetch = [&](uint32_t nb) {
+#pragma unroll
+    for (int i = 0; i < PPT; ++i) {
+      const uint32_t p = threadIdx.x + 256 * i;
+      const uint32_t key = p / PPK, part = p % PPK;
+      const uint32_t n = nb * kQkBlockN + key;
+      stage[i] = (n < a.kv_len) ? *(const v4i*)(kbase + (int64_t)n * a.sk_n + 16 * part)
+                                : v4i{0, 0, 0, 0};
+    }
+  };
+  auto park = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < PPT; ++i) {
+      const uint32_t p = threadIdx.x + 256 * i;
+      *(v4i*)&ktile[buf][p / PPK][16 * (p % PPK)] = stage[i];
+    }
+  };
+  fetch(0);
+  park(0);
+  __syncthreads();
 
   float run_m = -__builtin_inff(), run_l = 1.0f;  // qk_int8_per_block.py:79-80
   for (uint32_t nb = 0; nb < n_blocks; ++nb) {
+    const int buf = nb & 1;
+    if (nb + 1 < n_blocks) fetch(nb + 1);
     const float sc = ks[nb];
     v16i acc[2];
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
-      const uint32_t n = nb * kQkBlockN + 32 * s + c;
-      const int8_t* krow = kbase + (int64_t)n * a.sk_n;
       v4i ka[KC];
 #pragma unroll
-      for (int kc = 0; kc < KC; ++kc)
-        ka[kc] = (n < a.kv_len) ? *(const v4i*)(krow + 32 * kc) : v4i{0, 0, 0, 0};
+      for (int kc = 0; kc < KC; ++kc) ka[kc] = *(const v4i*)&ktile[buf][32 * s + c][32 * kc + 16 * g];
       v16i z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
       for (int kc = 0; kc < KC; ++kc)
         z = __builtin_amdgcn_mfma_i32_32x32x32_i8(ka[kc], qb[kc], z, 0, 0, 0);
       acc[s] = z;
     }
-    // online softmax of this lane's 32 scores (qk_int8_per_block.py:39-48)
-    float sv[32];
-    float tmax = run_m;
+    // online softmax of this lane's 32 scores (qk_int8_per_block.py:39-48). The kernel is bound by
+    // this part, not by the matrix cores (8 matrix instructions against 32 exponentials per lane
+    // and key block), so it is kept to one integer max, one convert, one fma and one exp2 per
+    // score: the block's largest score is the scale times the largest (smallest, for a negative
+    // scale) integer product.
+    const float s2 = qs * sc;
+    int imax = acc[0][0], imin = acc[0][0];
 #pragma unroll
     for (int s = 0; s < 2; ++s)
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        sv[16 * s + v] = (float)acc[s][v] * qs * sc;
-        tmax = fmaxf(tmax, sv[16 * s + v]);
+        imax = max(imax, acc[s][v]);
+        imin = min(imin, acc[s][v]);
       }
-    float add = 0.0f;
+    const float tmax = fmaxf(run_m, fmaxf((float)imax * s2, (float)imin * s2));
+    float add = 0.0f, add2 = 0.0f;
 #pragma unroll
-    for (int i = 0; i < 32; ++i) add += __builtin_amdgcn_exp2f(sv[i] - tmax);
-    run_l = run_l * __builtin_amdgcn_exp2f(run_m - tmax) + add;
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const float e = __builtin_amdgcn_exp2f(fmaf((float)acc[s][v], s2, -tmax));
+        if (v & 1) add2 += e;
+        else add += e;
+      }
+    run_l = run_l * __builtin_amdgcn_exp2f(run_m - tmax) + (add + add2);
     run_m = tmax;
+    if (nb + 1 < n_blocks) park(buf ^ 1);  // last read two barriers ago
+    __syncthreads();
   }
   // merge the two lane halves of a query: lane c and lane c + 32
   const float om = as_f32(__builtin_amdgcn_ds_bpermute(4 * (lane ^ 32), as_i32(run_m)));
