@@ -198,6 +198,120 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_int4_kernel(GemvArgs a) {
     if (grp * U + (lane >> 4) < np) orow[grp * U * TWL_PAGE + lane] = held[grp];
 }
 
+// One workgroup of 16 wavefronts per (batch, head) row, the row's scores parked in LDS and written
+// out in one burst when the row is done. With about one row per compute unit (the stand-alone
+// benchmark shape: 256 rows of 2048 pages) every compute unit streams for the whole kernel and
+// the score writes (4 bytes per token, 5 % of the bytes) no longer interleave with the read
+// stream, which costs this HBM far more than their share: see the dispatch in twl_gemv_int4.
+constexpr int kGemvRowThreads = 1024;
+
+template <int QDT, bool HAS_SEL>
+__global__ __launch_bounds__(kGemvRowThreads) void gemv_int4_rows_kernel(GemvArgs a, int wide) {
+  constexpr int U = kGemvUnroll;
+  constexpr int PW = 64;
+  constexpr int G = PW / U;
+  extern __shared__ __align__(16) float row_scores[];  // [max_pages * 16]
+  const uint32_t row = blockIdx.x;
+  const uint32_t b = row / a.num_q_heads;
+  const uint32_t h = row - b * a.num_q_heads;
+  const uint32_t kvh = h / (a.num_q_heads / a.num_kv_heads);
+  const int lane = lane_id();
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int pg_begin = a.kv_page_indptr[b];
+  const int pg_end = a.kv_page_indptr[b + 1];
+  const int last_len = a.kv_last_page_len[b];
+  const int sel_n = HAS_SEL ? (a.sel_count ? a.sel_count[row] : (int)a.sel_stride) : 0;
+  const int g = lane & 3;
+  const int t = lane >> 2;
+  u32x4 qraw[4];
+  {
+    const uint16_t* qrow = (const uint16_t*)a.q + (size_t)row * TWL_HEAD_DIM + 32 * g;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) qraw[i] = *(const u32x4*)(qrow + 8 * i);
+  }
+  const int req_pages = pg_end - pg_begin;
+  int n_pages = HAS_SEL ? sel_n : req_pages;
+  n_pages = min(max(n_pages, 0), (int)a.max_pages);
+  if (req_pages <= 0) n_pages = 0;
+  if (threadIdx.x == 0 && a.out_count) a.out_count[row] = n_pages * TWL_PAGE;
+  if (n_pages == 0) return;  // uniform
+
+  half2_t qp[16];
+  float qsum = 0.0f;
+  {
+    float qf[32];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t ws[4] = {qraw[i].x, qraw[i].y, qraw[i].z, qraw[i].w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        qf[8 * i + 2 * j] = bits16_to_f32<QDT>(ws[j] & 0xFFFFu);
+        qf[8 * i + 2 * j + 1] = bits16_to_f32<QDT>(ws[j] >> 16);
+      }
+    }
+#pragma unroll
+    for (int w = 0; w < 4; ++w)
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        half2_t pr = {(_Float16)qf[8 * w + s], (_Float16)qf[8 * w + s + 4]};
+        qp[4 * w + s] = pr;
+      }
+#pragma unroll
+    for (int i = 0; i < 32; ++i) qsum += (float)(_Float16)qf[i];
+  }
+  const size_t rec_stride = (size_t)a.num_kv_heads * TWL_INT4_RECORD_BYTES;
+  const uint8_t* base = a.k_int4 + (size_t)kvh * TWL_INT4_RECORD_BYTES + 16 * lane;
+  const float ninf = -__builtin_inff();
+  const int src_lane4 = 4 * (4 * (lane & 15) + (lane >> 4));
+
+  for (int p0 = wave * PW; p0 < n_pages; p0 += (kGemvRowThreads / kWave) * PW) {
+    const int np = min(PW, n_pages - p0);
+    int my_logical = p0 + lane;
+    if (HAS_SEL)
+      my_logical = ((uint32_t)(p0 + lane) < a.sel_stride)
+                       ? a.sel_pages[(size_t)row * a.sel_stride + p0 + lane] : 0;
+    my_logical = min(max(my_logical, 0), req_pages - 1);
+    int my_phys = 0;
+    if (lane < np) my_phys = a.kv_page_indices[pg_begin + my_logical];
+    u32x4 nib[U];
+    uint32_t sz[U];
+#pragma unroll
+    for (int grp = 0; grp < G; ++grp) {
+      if (grp * U < np) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const int i = grp * U + u;
+          const int phys = __builtin_amdgcn_readlane(my_phys, (i < np) ? i : 0);
+          const uint8_t* rec = base + (size_t)phys * rec_stride;
+          nib[u] = __builtin_nontemporal_load((const u32x4*)rec);
+          sz[u] = __builtin_nontemporal_load((const uint32_t*)(rec + 1024 - 12 * lane));
+        }
+        float mine = 0.0f;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const int i = grp * U + u;
+          const float part = page_partial(nib[u], sz[u], qp, qsum);
+          const int logical = __builtin_amdgcn_readlane(my_logical, (i < np) ? i : 0);
+          const int valid = (logical == req_pages - 1) ? last_len : TWL_PAGE;
+          const float val = (t < valid) ? part * a.sm_scale : ninf;
+          mine = (g == u) ? val : mine;
+        }
+        const float v = as_f32(__builtin_amdgcn_ds_bpermute(src_lane4, as_i32(mine)));
+        if (grp * U + (lane >> 4) < np) row_scores[(p0 + grp * U) * TWL_PAGE + lane] = v;
+      }
+    }
+  }
+  __syncthreads();
+  float* orow = a.out + (size_t)row * a.out_stride;
+  const int total = n_pages * TWL_PAGE;  // a multiple of 16
+  if (wide) {
+    for (int i = 4 * threadIdx.x; i < total; i += 4 * kGemvRowThreads)
+      *(f32x4*)(orow + i) = *(const f32x4*)(row_scores + i);
+  } else {
+    for (int i = threadIdx.x; i < total; i += kGemvRowThreads) orow[i] = row_scores[i];
+  }
+}
+
 template <int QDT, bool HAS_SEL>
 static void launch_gemv(const GemvArgs& a, uint32_t rows, int pw, hipStream_t st) {
   const dim3 blk(kGemvThreads);
@@ -242,6 +356,32 @@ extern "C" int twl_gemv_int4(const void* q, int q_dtype, float* out, uint32_t ou
   int cus = 256;
   (void)twl::device_cu_count(&cus);
   const uint64_t want_waves = 8ull * (uint64_t)cus;
+  // about one row per compute unit and a row of scores that fits LDS: a workgroup per row
+#ifndef TWL_GEMV_NO_ROWS
+  // (measured at 256 rows: 2048 pages per row 122.7 -> 114.2 us, 512 pages per row no change)
+  if (max_pages_per_row > 512u && max_pages_per_row <= 2048u && 2u * rows >= (uint32_t)cus &&
+      rows <= 2u * (uint32_t)cus) {
+    const int wide = ((((uintptr_t)out) & 15u) == 0 && (out_stride & 3u) == 0) ? 1 : 0;
+    const size_t lds = (size_t)max_pages_per_row * TWL_PAGE * sizeof(float);
+    const dim3 grid_r(rows), blk_r(twl::kGemvRowThreads);
+#define TWL_GEMV_ROWS(DT, SEL)                                                              \
+  do {                                                                                        \
+    if (lds > 48 * 1024)                                                                      \
+      (void)hipFuncSetAttribute((const void*)twl::gemv_int4_rows_kernel<DT, SEL>,             \
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);        \
+    hipLaunchKernelGGL((twl::gemv_int4_rows_kernel<DT, SEL>), grid_r, blk_r, lds, st, a, wide); \
+  } while (0)
+    if (q_dtype == TWL_F16) {
+      if (sel_pages) TWL_GEMV_ROWS(TWL_F16, true);
+      else TWL_GEMV_ROWS(TWL_F16, false);
+    } else {
+      if (sel_pages) TWL_GEMV_ROWS(TWL_BF16, true);
+      else TWL_GEMV_ROWS(TWL_BF16, false);
+    }
+#undef TWL_GEMV_ROWS
+    return hipGetLastError() == hipSuccess ? TWL_OK : TWL_ELAUNCH;
+  }
+#endif
 #ifdef TWL_GEMV_PW
   const int pw = TWL_GEMV_PW;
 #else
