@@ -388,7 +388,8 @@ def main() -> int:
         if layers[0].cache.meta_planes is not None and H == Hkv:
             calls["quest_score_planes"] = (rotating(
                 lambda l, c, q: lambda: L.twl_quest_page_scores_planes(
-                    p(q), qcode, p(c.meta_planes), c.meta_planes.size(4), 0, 0, p(c.kv_page_indptr),
+                    p(q), qcode, p(c.meta_planes), c.meta_planes.size(4), 0, 0, p(c.meta),
+                    p(c.kv_page_indices), p(c.kv_page_indptr),
                     B, H, Hkv, npg, p(l.page_scores), npg, stream)),
                 rows * npg * 256 + rows * npg * 4 + rows * D * 2)   # the sign-selected runs only
         for name, (fn, nbytes) in calls.items():

@@ -145,7 +145,8 @@ int twl_gemv_top_p(const void* q, int q_dtype, const void* k_int4, const int32_t
  * sel_count (ascending logical pages, ties at the k-th score to the lower page), idx / count,
  * optionally page_scores_out [rows, page_score_stride], scores_out [rows, score_stride] and
  * cand_count. max_pages_per_req <= 8192. With meta_planes (plane layout, see
- * twl_meta_planes_build; then meta may be NULL) the page scores are accumulated channel by channel
+ * twl_meta_planes_build; meta is still needed: a request's last page is scored from its record)
+ * the page scores are accumulated channel by channel
  * in ascending order from the sign-selected runs; they can differ from twl_quest_page_scores in
  * the last bits (other summation order). Meant for about one row per compute unit (decode at
  * moderate batch). With GQA every q-head row reads its kv head's metadata; the rows of a group
@@ -303,7 +304,10 @@ int twl_kv_append(const void* k_new, const void* v_new, int kv_dtype, uint64_t n
  * pass of twl_select_estimate_prune touches half the bytes of the record layout. Nothing in the
  * reference corresponds to it (it recomputes the chunk maxima from K every step, quest.py:68-74).
  * twl_meta_planes_build fills the planes of the pages of the current page table from the metadata
- * records of twl_kv_shadow_build; twl_kv_append keeps them current when given meta_planes.
+ * records of twl_kv_shadow_build. A request's LAST page is always scored from its record, not from
+ * the planes: twl_kv_append (given meta_planes) folds a new token into the record at every step
+ * and writes the page's plane entries once, when the token completes the page. The plane entries
+ * of a last page may therefore be stale; every kernel here ignores them.
  * plane_slots (nullable, device, [batch]) names the slot of every batch position, so that a
  * request keeps its planes when its position in the batch changes (continuous batching: a request
  * leaves and the others move up); plane_num_slots is the number of slots the buffer holds, and
@@ -318,7 +322,8 @@ int twl_meta_planes_build(const void* meta, const int32_t* kv_page_indices,
  * here, the record form does). Scores are accumulated channel by channel in ascending order. */
 int twl_quest_page_scores_planes(const void* q, int q_dtype, const void* meta_planes,
                                  uint32_t plane_cap_pages, const int32_t* plane_slots,
-                                 uint32_t plane_num_slots, const int32_t* kv_page_indptr,
+                                 uint32_t plane_num_slots, const void* meta,
+                                 const int32_t* kv_page_indices, const int32_t* kv_page_indptr,
                                  uint32_t batch, uint32_t num_q_heads, uint32_t num_kv_heads,
                                  uint32_t max_pages_per_req, float* page_scores,
                                  uint32_t score_stride, void* stream);

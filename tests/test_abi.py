@@ -20,7 +20,7 @@ def test_header_symbols_are_exported(hip_lib):
     assert declared == set(_lib.EXPORTS)
     for name in declared:
         assert hasattr(hip_lib, name), name
-    assert hip_lib.twl_abi_version() == 4
+    assert hip_lib.twl_abi_version() == 5
 
 
 def test_header_compiles_as_c():
@@ -116,7 +116,7 @@ def test_c_level_validation_without_gpu(hip_lib):
     assert sep(sel_stride=3) == -2 and sep(idx_stride=63) == -2 and sep(p=2.0) == -2
     assert sep(hq=4, hkv=3) == -2
     assert sep(q=f + 4) == -4
-    assert sep(meta=0, planes=f, cap=16, budget=0) == -2  # planes alone pass the NULL check
+    assert sep(meta=0, planes=f, cap=16) == -1            # the records are needed with planes too
     assert sep(planes=f, cap=8) == -2 and sep(planes=f, cap=20) == -2   # cap < pages, cap % 8
     assert sep(planes=f, cap=16, slots=f, nslots=0) == -2               # slot table, no slots
     app = lambda **kw: L.twl_kv_append(
@@ -126,6 +126,7 @@ def test_c_level_validation_without_gpu(hip_lib):
     assert app(k=0) == -1 and app(last=0) == -1
     assert app(dt=2) == -3 and app(b=0) == -2 and app(ts=250) == -4 and app(k=f + 2) == -4
     assert app(planes=f, cap=12) == -2 and app(planes=f, cap=16, slots=f, nslots=0) == -2
+    assert app(planes=f, cap=16) == -1                    # planes are written from the record
     pb = lambda **kw: L.twl_meta_planes_build(kw.get("meta", f), f, f, 1, 1, kw.get("npg", 8),
                                               kw.get("planes", f), kw.get("cap", 8),
                                               kw.get("slots", 0), kw.get("nslots", 0), 0)

@@ -246,7 +246,7 @@ def test_row_kernel_with_plane_metadata(dev, N, budget, H, Hkv, dt):
     ps2 = torch.zeros((B, H, npg), dtype=torch.float32, device=dev)
     rc = _lib.lib().twl_quest_page_scores_planes(
         qd.data_ptr(), 0 if dt == torch.float16 else 1, cache.meta_planes.data_ptr(), cap, 0, 0,
-        cache.kv_page_indptr.data_ptr(), B, H, Hkv, npg, ps2.data_ptr(), npg,
+        cache.meta.data_ptr(), cache.kv_page_indices.data_ptr(), cache.kv_page_indptr.data_ptr(), B, H, Hkv, npg, ps2.data_ptr(), npg,
         torch.cuda.current_stream().cuda_stream)
     assert rc == 0
     assert torch.equal(ps2.view(torch.int32), Bv[5].view(torch.int32))

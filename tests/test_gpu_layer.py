@@ -197,9 +197,11 @@ def test_append_kernel_records_equal_bulk_build(dev, dt):
         cache.append(k[:, :, N0 + s].to(dev), v[:, :, N0 + s].to(dev), free)
     full = PagedKVCache.from_dense(k, v, dev, plane_pages=8)
     assert torch.equal(cache.kv_last_page_len.cpu(), full.kv_last_page_len.cpu())
-    npg_now = (N0 + steps + 15) // 16
-    assert torch.equal(cache.meta_planes.view(torch.int16)[..., :npg_now],
-                       full.meta_planes.view(torch.int16)[..., :npg_now])   # plane-layout metadata too
+    # plane-layout metadata too, for every COMPLETE page: the last page of a request is scored from
+    # its record, and its plane entries are written when its 16th token arrives
+    done = (N0 + steps) // 16
+    assert torch.equal(cache.meta_planes.view(torch.int16)[..., :done],
+                       full.meta_planes.view(torch.int16)[..., :done])
     ia, ib = cache.kv_page_indices.long(), full.kv_page_indices.long()
     assert ia.numel() == ib.numel()
     for name in ("k_cache", "v_cache", "k_int4", "meta"):

@@ -105,8 +105,8 @@ def lib() -> ctypes.CDLL:
     L.twl_kv_append.argtypes = [vp, vp, i32, u64, u64, vp, vp, u64, u64, u64, vp, vp, vp, u32, u32,
                                 vp, vp, vp, u32, vp, u32, vp]
     L.twl_meta_planes_build.argtypes = [vp, vp, vp, u32, u32, u32, vp, u32, vp, u32, vp]
-    L.twl_quest_page_scores_planes.argtypes = [vp, i32, vp, u32, vp, u32, vp, u32, u32, u32, u32, vp,
-                                               u32, vp]
+    L.twl_quest_page_scores_planes.argtypes = [vp, i32, vp, u32, vp, u32, vp, vp, vp, u32, u32, u32,
+                                               u32, vp, u32, vp]
     i64 = ctypes.c_int64
     L.twl_qk_int8_lse.argtypes = [vp, vp, vp, vp, vp, u32, u32, u32, u32, u32, u32, i64, i64, i64,
                                   i64, i64, i64, vp]

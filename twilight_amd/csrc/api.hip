@@ -15,7 +15,7 @@ extern "C" const char* twl_strerror(int status) {
   }
 }
 
-extern "C" int twl_abi_version(void) { return 4; }
+extern "C" int twl_abi_version(void) { return 5; }
 
 extern "C" int twl_device_count(void) {
   int n = 0;
@@ -87,7 +87,8 @@ extern "C" int twl_decode_layer(const twl_layer_args* a, void* stream) {
     } else if (a->meta_planes && a->num_q_heads == a->num_kv_heads &&
                a->plane_cap_pages >= a->max_pages_per_req) {
       rc = twl_quest_page_scores_planes(a->q, a->dtype, a->meta_planes, a->plane_cap_pages,
-                                        a->plane_slots, a->plane_num_slots, a->kv_page_indptr, a->batch, a->num_q_heads,
+                                        a->plane_slots, a->plane_num_slots, a->meta,
+                                        a->kv_page_indices, a->kv_page_indptr, a->batch, a->num_q_heads,
                                         a->num_kv_heads, a->max_pages_per_req, page_scores,
                                         ps_stride, stream);
       if (rc != TWL_OK) return rc;

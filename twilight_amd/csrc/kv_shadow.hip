@@ -115,7 +115,7 @@ __global__ __launch_bounds__(kShThreads) void kv_shadow_kernel(ShadowArgs a) {
 // last page (the host has made sure that page exists and, when it is a fresh page, has set the
 // length to 0), K and V rows are stored, the token's part of the INT4 record is quantised, the
 // page's min / max metadata is folded with the new row, and the length is advanced. One workgroup
-// per request; its four wavefronts share the kv heads.
+// per request; its wavefronts share the kv heads.
 struct AppendArgs {
   const void* k_new;
   const void* v_new;
@@ -135,8 +135,15 @@ struct AppendArgs {
   uint32_t plane_num_slots;
 };
 
+// 16 wavefronts per request: a kv head is a chain of two or three dependent memory round trips
+// (row in, records / runs in, results out), so heads run side by side rather than one after the
+// other (4 wavefronts: 55 us per call at 32 kv heads; one workgroup per request is kept because
+// the request's length is read by every wavefront and advanced once at the end)
+constexpr int kAppendThreads = 1024;
+constexpr int kAppendWaves = kAppendThreads / kWave;
+
 template <int DT>
-__global__ __launch_bounds__(kShThreads) void kv_append_kernel(AppendArgs a) {
+__global__ __launch_bounds__(kAppendThreads) void kv_append_kernel(AppendArgs a) {
   const uint32_t b = blockIdx.x;
   const int lane = lane_id();
   const int wave = threadIdx.x / kWave;
@@ -146,94 +153,94 @@ __global__ __launch_bounds__(kShThreads) void kv_append_kernel(AppendArgs a) {
   __syncthreads();  // every wave has read the length before it is advanced below
   if (n_pages <= 0 || slot < 0 || slot >= TWL_PAGE) return;  // nothing sane to do; length untouched
   const int page = a.kv_page_indices[pg_end - 1];
-  for (uint32_t kvh = wave; kvh < a.num_kv_heads; kvh += kShWaves) {
-    const size_t src_off = (size_t)b * a.new_batch_stride + (size_t)kvh * a.new_head_stride;
-    const size_t dst_off = (size_t)page * a.page_stride + (size_t)slot * a.token_stride +
-                           (size_t)kvh * a.head_stride;
-    // K and V rows: 2 channels per lane
-    const uint32_t kw = *((const uint32_t*)((const uint16_t*)a.k_new + src_off) + lane);
-    const uint32_t vw = *((const uint32_t*)((const uint16_t*)a.v_new + src_off) + lane);
-    *((uint32_t*)((uint16_t*)a.k_cache + dst_off) + lane) = kw;
-    *((uint32_t*)((uint16_t*)a.v_cache + dst_off) + lane) = vw;
-    if (a.k_int4) {
-      uint8_t* rec = a.k_int4 + ((size_t)page * a.num_kv_heads + kvh) * TWL_INT4_RECORD_BYTES;
-      if (slot == 0) {  // a fresh page: the other 15 tokens' parts read as "not written"
-        *(u32x4*)(rec + 16 * lane) = u32x4{0u, 0u, 0u, 0u};
-        *(uint32_t*)(rec + 1024 + 4 * lane) = 0u;
+  const bool use_planes = a.planes && n_pages <= (int)a.plane_cap;
+  const uint32_t pslot = use_planes ? plane_slot(a.plane_slots, a.plane_num_slots, b) : 0u;
+  constexpr int HU = 2;  // heads in flight per wavefront: their loads overlap
+  for (uint32_t kvh0 = wave; kvh0 < a.num_kv_heads; kvh0 += HU * kAppendWaves) {
+    uint32_t kw[HU], vw[HU], om[HU], ox[HU];
+    const int mc = lane >> 1, mo = (lane & 1) * 4;
+    // ---- every load first: the stores below may alias them as far as the compiler knows, and a
+    // load issued after a store waits for a memory round trip of its own -------------------------
+#pragma unroll
+    for (int u = 0; u < HU; ++u) {
+      const uint32_t kvh = kvh0 + u * kAppendWaves;
+      kw[u] = vw[u] = om[u] = ox[u] = 0u;
+      if (kvh < a.num_kv_heads) {
+        const size_t src_off = (size_t)b * a.new_batch_stride + (size_t)kvh * a.new_head_stride;
+        kw[u] = *((const uint32_t*)((const uint16_t*)a.k_new + src_off) + lane);  // 2 channels per lane
+        vw[u] = *((const uint32_t*)((const uint16_t*)a.v_new + src_off) + lane);
+        if (a.meta && slot > 0) {
+          const uint8_t* mrec = a.meta + ((size_t)page * a.num_kv_heads + kvh) * TWL_META_RECORD_BYTES;
+          om[u] = *(const uint32_t*)(mrec + 16 * mc + mo);
+          ox[u] = *(const uint32_t*)(mrec + 16 * mc + 8 + mo);
+        }
       }
-      if (lane < 4) {  // lane g quantises group g of the new row (same arithmetic as kv_shadow_kernel)
-        float x[32];
-        const uint16_t* src = (const uint16_t*)a.k_new + src_off + 32 * lane;
+    }
+    // ---- stores ------------------------------------------------------------------------------
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          u32x4 v = *(const u32x4*)(src + 8 * i);
-          const uint32_t ws[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            x[8 * i + 2 * j] = bits16_to_f32<DT>(ws[j] & 0xFFFFu);
-            x[8 * i + 2 * j + 1] = bits16_to_f32<DT>(ws[j] >> 16);
-          }
+    for (int u = 0; u < HU; ++u) {
+      const uint32_t kvh = kvh0 + u * kAppendWaves;
+      if (kvh >= a.num_kv_heads) continue;  // wave-uniform
+      const size_t dst_off = (size_t)page * a.page_stride + (size_t)slot * a.token_stride +
+                             (size_t)kvh * a.head_stride;
+      const float k0 = bits16_to_f32<DT>(kw[u] & 0xFFFFu), k1 = bits16_to_f32<DT>(kw[u] >> 16);
+      *((uint32_t*)((uint16_t*)a.k_cache + dst_off) + lane) = kw[u];
+      *((uint32_t*)((uint16_t*)a.v_cache + dst_off) + lane) = vw[u];
+      if (a.k_int4) {
+        uint8_t* rec = a.k_int4 + ((size_t)page * a.num_kv_heads + kvh) * TWL_INT4_RECORD_BYTES;
+        if (slot == 0) {  // a fresh page: the other 15 tokens' parts read as "not written"
+          *(u32x4*)(rec + 16 * lane) = u32x4{0u, 0u, 0u, 0u};
+          *(uint32_t*)(rec + 1024 + 4 * lane) = 0u;
         }
-        float mn = x[0], mx = x[0];
-#pragma unroll
-        for (int i = 1; i < 32; ++i) {
-          mn = fminf(mn, x[i]);
-          mx = fmaxf(mx, x[i]);
-        }
+        // The new row's 4 groups of 32 channels, 16 lanes per group, 2 channels per lane: the
+        // same arithmetic per element as kv_shadow_kernel (min / max are order-independent), two
+        // divisions per lane instead of 32 in a row on four lanes.
+        const float mn = row16_allreduce<OpMin>(fminf(k0, k1));
+        const float mx = row16_allreduce<OpMax>(fmaxf(k0, k1));
         const float range = fmaxf(mx - mn, 1e-9f);
         float sh = round_to<TWL_F16>(range / 15.0f);
         sh = fminf(fmaxf(sh, 6.103515625e-05f), 65504.0f);
         float zh = round_to<TWL_F16>(mn);
         zh = fminf(fmaxf(zh, -65504.0f), 65504.0f);
-        uint32_t w[4] = {0u, 0u, 0u, 0u};
-#pragma unroll
-        for (int i = 0; i < 32; ++i) {
-          float c = rintf((x[i] - zh) / sh);
-          c = fminf(fmaxf(c, 0.0f), 15.0f);
-          w[i >> 3] |= (uint32_t)c << (4 * (i & 7));
-        }
-        const int li = 4 * slot + lane;  // the record's (token, group) index
-        *(u32x4*)(rec + 16 * li) = u32x4{w[0], w[1], w[2], w[3]};
-        *(uint32_t*)(rec + 1024 + 4 * li) = f32_to_f16_bits(sh) | (f32_to_f16_bits(zh) << 16);
+        float c0 = rintf((k0 - zh) / sh), c1 = rintf((k1 - zh) / sh);
+        c0 = fminf(fmaxf(c0, 0.0f), 15.0f);
+        c1 = fminf(fmaxf(c1, 0.0f), 15.0f);
+        // channels 2r, 2r+1 (r = lane % 16) are byte r % 4 of dword r / 4 of the group's 16 bytes
+        int wv = (int)(((uint32_t)c0 | ((uint32_t)c1 << 4)) << (8 * (lane & 3)));
+        wv |= dpp<kDppXor1>(0, wv);
+        wv |= dpp<kDppXor2>(0, wv);
+        const int li = 4 * slot + (lane >> 4);  // the record's (token, group) index
+        if ((lane & 3) == 0) *(uint32_t*)(rec + 16 * li + 4 * ((lane & 15) >> 2)) = (uint32_t)wv;
+        if ((lane & 15) == 0)
+          *(uint32_t*)(rec + 1024 + 4 * li) = f32_to_f16_bits(sh) | (f32_to_f16_bits(zh) << 16);
       }
-    }
-    if (a.meta) {  // lane l folds channels 2l, 2l+1 into the page's min / max
-      uint8_t* rec = a.meta + ((size_t)page * a.num_kv_heads + kvh) * TWL_META_RECORD_BYTES;
-      const int c = lane >> 1, o = (lane & 1) * 4;
-      uint32_t* pmin = (uint32_t*)(rec + 16 * c + o);
-      uint32_t* pmax = (uint32_t*)(rec + 16 * c + 8 + o);
-      const float k0 = bits16_to_f32<DT>(kw & 0xFFFFu), k1 = bits16_to_f32<DT>(kw >> 16);
-      float mn0 = k0, mn1 = k1, mx0 = k0, mx1 = k1;
-      if (slot > 0) {
-        const uint32_t om = *pmin, ox = *pmax;
-        mn0 = fminf(mn0, bits16_to_f32<DT>(om & 0xFFFFu));
-        mn1 = fminf(mn1, bits16_to_f32<DT>(om >> 16));
-        mx0 = fmaxf(mx0, bits16_to_f32<DT>(ox & 0xFFFFu));
-        mx1 = fmaxf(mx1, bits16_to_f32<DT>(ox >> 16));
-      }
-      *pmin = f32_to_bits16<DT>(mn0) | (f32_to_bits16<DT>(mn1) << 16);
-      *pmax = f32_to_bits16<DT>(mx0) | (f32_to_bits16<DT>(mx1) << 16);
-    }
-    if (a.planes && n_pages <= (int)a.plane_cap) {
-      // the same fold in the plane layout: runs [d][min|max][logical page] of the request's slot
-      const uint32_t pslot = plane_slot(a.plane_slots, a.plane_num_slots, b);
-      uint16_t* pl = a.planes +
-                     ((size_t)pslot * a.num_kv_heads + kvh) * (TWL_HEAD_DIM * 2) * a.plane_cap +
-                     (n_pages - 1);
-#pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        const int d = 2 * lane + j;
-        const uint32_t kb = j ? (kw >> 16) : (kw & 0xFFFFu);
-        const float kv = bits16_to_f32<DT>(kb);
-        uint16_t* pmn = pl + (size_t)(2 * d) * a.plane_cap;
-        uint16_t* pmx = pl + (size_t)(2 * d + 1) * a.plane_cap;
-        float mn = kv, mx = kv;
+      if (a.meta) {  // lane l folds channels 2l, 2l+1 into the page's min / max
+        uint8_t* mrec = a.meta + ((size_t)page * a.num_kv_heads + kvh) * TWL_META_RECORD_BYTES;
+        float mn0 = k0, mn1 = k1, mx0 = k0, mx1 = k1;
         if (slot > 0) {
-          mn = fminf(mn, bits16_to_f32<DT>(*pmn));
-          mx = fmaxf(mx, bits16_to_f32<DT>(*pmx));
+          mn0 = fminf(mn0, bits16_to_f32<DT>(om[u] & 0xFFFFu));
+          mn1 = fminf(mn1, bits16_to_f32<DT>(om[u] >> 16));
+          mx0 = fmaxf(mx0, bits16_to_f32<DT>(ox[u] & 0xFFFFu));
+          mx1 = fmaxf(mx1, bits16_to_f32<DT>(ox[u] >> 16));
         }
-        *pmn = (uint16_t)f32_to_bits16<DT>(mn);
-        *pmx = (uint16_t)f32_to_bits16<DT>(mx);
+        const uint32_t bmn0 = f32_to_bits16<DT>(mn0), bmn1 = f32_to_bits16<DT>(mn1);
+        const uint32_t bmx0 = f32_to_bits16<DT>(mx0), bmx1 = f32_to_bits16<DT>(mx1);
+        *(uint32_t*)(mrec + 16 * mc + mo) = bmn0 | (bmn1 << 16);
+        *(uint32_t*)(mrec + 16 * mc + 8 + mo) = bmx0 | (bmx1 << 16);
+        if (use_planes && slot == TWL_PAGE - 1) {
+          // This token completes the page: its min / max go to the plane layout (runs
+          // [d][min|max][logical page] of the request's slot), 256 scattered 2-byte stores per
+          // head, once per 16 tokens. Until then the scoring passes take a request's last page
+          // from the record above, so the planes are not touched on the other 15 steps (folding
+          // them every step cost 8 of 15 us per call at 8 requests x 32 kv heads).
+          uint16_t* pl = a.planes +
+                         ((size_t)pslot * a.num_kv_heads + kvh) * (TWL_HEAD_DIM * 2) * a.plane_cap +
+                         (n_pages - 1);
+          pl[(size_t)(4 * lane + 0) * a.plane_cap] = (uint16_t)bmn0;
+          pl[(size_t)(4 * lane + 1) * a.plane_cap] = (uint16_t)bmx0;
+          pl[(size_t)(4 * lane + 2) * a.plane_cap] = (uint16_t)bmn1;
+          pl[(size_t)(4 * lane + 3) * a.plane_cap] = (uint16_t)bmx1;
+        }
       }
     }
   }
@@ -322,6 +329,7 @@ extern "C" int twl_kv_append(const void* k_new, const void* v_new, int kv_dtype,
     return TWL_EALIGN;
   if (meta_planes && (plane_cap_pages == 0 || (plane_cap_pages & 7u))) return TWL_EINVAL;
   if (meta_planes && plane_slots && plane_num_slots == 0) return TWL_EINVAL;
+  if (meta_planes && !meta) return TWL_ENULL;  // the planes are written from the folded record
   twl::AppendArgs a{};
   a.k_new = k_new; a.v_new = v_new; a.new_batch_stride = new_batch_stride;
   a.new_head_stride = new_head_stride; a.k_cache = k_cache; a.v_cache = v_cache;
@@ -332,10 +340,10 @@ extern "C" int twl_kv_append(const void* k_new, const void* v_new, int kv_dtype,
   a.planes = (uint16_t*)meta_planes; a.plane_cap = plane_cap_pages;
   a.plane_slots = plane_slots; a.plane_num_slots = plane_num_slots;
   if (kv_dtype == TWL_F16)
-    hipLaunchKernelGGL((twl::kv_append_kernel<TWL_F16>), dim3(batch), dim3(twl::kShThreads), 0,
+    hipLaunchKernelGGL((twl::kv_append_kernel<TWL_F16>), dim3(batch), dim3(twl::kAppendThreads), 0,
                        (hipStream_t)stream, a);
   else
-    hipLaunchKernelGGL((twl::kv_append_kernel<TWL_BF16>), dim3(batch), dim3(twl::kShThreads), 0,
+    hipLaunchKernelGGL((twl::kv_append_kernel<TWL_BF16>), dim3(batch), dim3(twl::kAppendThreads), 0,
                        (hipStream_t)stream, a);
   return hipGetLastError() == hipSuccess ? TWL_OK : TWL_ELAUNCH;
 }

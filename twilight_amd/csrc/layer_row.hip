@@ -103,6 +103,17 @@ __global__ __launch_bounds__(kRowThreads) void select_estimate_prune_kernel(RowA
     const uint16_t* pl =
         a.planes + ((size_t)slot * a.f.num_kv_heads + kvh) * (TWL_HEAD_DIM * 2) * a.plane_cap;
     constexpr int PL_PASSES = (SEL_VPT + 1) / 2;  // 16 waves x 128 pages = 2048 pages per pass
+    // The request's last page is scored from its metadata record: the appending side keeps the
+    // record current token by token and writes the plane entries once, when the page is full.
+    const int last_pg = n_score - 1;
+    float s_last = 0.0f;
+    if (wave == 0 && n_score > 0) {  // requested now, folded while the other pages stream
+      const uint32_t qw2 = *(const uint32_t*)(qrow + 2 * lane);
+      const int phys = a.f.kv_page_indices[pg_begin + last_pg];
+      s_last = record_page_score<QDT>(
+          a.meta + ((size_t)phys * a.f.num_kv_heads + kvh) * TWL_META_RECORD_BYTES,
+          bits16_to_f32<QDT>(qw2 & 0xFFFFu), bits16_to_f32<QDT>(qw2 >> 16));
+    }
 #pragma unroll
     for (int pass = 0; pass < PL_PASSES; ++pass) {
       const int w0 = (pass * kRowWaves + wave) * 128;  // first page of this wave's slice
@@ -120,14 +131,18 @@ __global__ __launch_bounds__(kRowThreads) void select_estimate_prune_kernel(RowA
           s0 = fmaf(qd, bits16_to_f32<QDT>(w & 0xFFFFu), s0);
           s1 = fmaf(qd, bits16_to_f32<QDT>(w >> 16), s1);
         }
-        if (pg0 < n_score) ps_lds[pg0] = s0;
-        if (pg0 + 1 < n_score) ps_lds[pg0 + 1] = s1;
+        if (pg0 < last_pg) ps_lds[pg0] = s0;
+        if (pg0 + 1 < last_pg) ps_lds[pg0 + 1] = s1;
         if (a.page_scores_out) {
           float* po = a.page_scores_out + (size_t)row * a.page_score_stride;
-          if (pg0 < n_score) po[pg0] = s0;
-          if (pg0 + 1 < n_score) po[pg0 + 1] = s1;
+          if (pg0 < last_pg) po[pg0] = s0;
+          if (pg0 + 1 < last_pg) po[pg0 + 1] = s1;
         }
       }
+    }
+    if (wave == 0 && lane == 0 && n_score > 0) {
+      ps_lds[last_pg] = s_last;
+      if (a.page_scores_out) a.page_scores_out[(size_t)row * a.page_score_stride + last_pg] = s_last;
     }
   } else {
     // page ids of all passes first: register r, lane l <-> pass 2r + l/32, page l%32 of the wave's
@@ -250,7 +265,7 @@ extern "C" int twl_select_estimate_prune(
     int32_t* count, float* page_scores_out, uint32_t page_score_stride, float* scores_out,
     uint32_t score_stride, int32_t* cand_count, const void* meta_planes,
     uint32_t plane_cap_pages, const int32_t* plane_slots, uint32_t plane_num_slots, void* stream) {
-  if (!q || (!meta && !meta_planes) || !k_int4 || !kv_page_indices || !kv_page_indptr || !kv_last_page_len ||
+  if (!q || !meta || !k_int4 || !kv_page_indices || !kv_page_indptr || !kv_last_page_len ||
       !sel_pages || !sel_count || !idx || !count)
     return TWL_ENULL;
   if (dtype != TWL_F16 && dtype != TWL_BF16) return TWL_EDTYPE;

@@ -95,6 +95,8 @@ struct PlaneScoreArgs {
   uint32_t cap;
   const int32_t* slots;  // nullable: slot of each batch position
   uint32_t num_slots;
+  const uint8_t* meta;             // records: a request's last page is scored from its record
+  const int32_t* kv_page_indices;
   const int32_t* kv_page_indptr;
   uint32_t num_q_heads, num_kv_heads;
   uint32_t max_pages;
@@ -142,8 +144,17 @@ __global__ __launch_bounds__(kPsThreads) void quest_score_planes_kernel(PlaneSco
     s1 = fmaf(qd, bits16_to_f32<DT>(w >> 16), s1);
   }
   float* po = a.page_scores + (size_t)row * a.score_stride;
-  if (pg0 < n_req) po[pg0] = s0;
-  if (pg0 + 1 < n_req) po[pg0 + 1] = s1;
+  const int last_pg = n_req - 1;  // scored from its record, by the wavefront that owns it
+  if (pg0 < last_pg) po[pg0] = s0;
+  if (pg0 + 1 < last_pg) po[pg0 + 1] = s1;
+  if (last_pg >= w0 && last_pg < w0 + 128) {  // wave-uniform
+    const uint32_t qw2 = *(const uint32_t*)(qrow + 2 * lane);
+    const int phys = a.kv_page_indices[a.kv_page_indptr[b] + last_pg];
+    const float s_last = record_page_score<DT>(
+        a.meta + ((size_t)phys * a.num_kv_heads + kvh) * TWL_META_RECORD_BYTES,
+        bits16_to_f32<DT>(qw2 & 0xFFFFu), bits16_to_f32<DT>(qw2 >> 16));
+    if (lane == 0) po[last_pg] = s_last;
+  }
 }
 
 }  // namespace twl
@@ -151,11 +162,13 @@ __global__ __launch_bounds__(kPsThreads) void quest_score_planes_kernel(PlaneSco
 extern "C" int twl_quest_page_scores_planes(const void* q, int q_dtype, const void* meta_planes,
                                             uint32_t plane_cap_pages,
                                             const int32_t* plane_slots, uint32_t plane_num_slots,
+                                            const void* meta, const int32_t* kv_page_indices,
                                             const int32_t* kv_page_indptr, uint32_t batch,
                                             uint32_t num_q_heads, uint32_t num_kv_heads,
                                             uint32_t max_pages_per_req, float* page_scores,
                                             uint32_t score_stride, void* stream) {
-  if (!q || !meta_planes || !kv_page_indptr || !page_scores) return TWL_ENULL;
+  if (!q || !meta_planes || !meta || !kv_page_indices || !kv_page_indptr || !page_scores)
+    return TWL_ENULL;
   if (q_dtype != TWL_F16 && q_dtype != TWL_BF16) return TWL_EDTYPE;
   if (batch == 0 || num_q_heads == 0 || num_kv_heads == 0 || num_q_heads % num_kv_heads != 0)
     return TWL_EINVAL;
@@ -164,11 +177,13 @@ extern "C" int twl_quest_page_scores_planes(const void* q, int q_dtype, const vo
   if (plane_cap_pages < max_pages_per_req || (plane_cap_pages & 7u)) return TWL_EINVAL;
   if (plane_slots && plane_num_slots == 0) return TWL_EINVAL;
   if ((uint64_t)batch * num_q_heads > 65535u) return TWL_EINVAL;
-  if ((((uintptr_t)q) & 1u) || (((uintptr_t)meta_planes) & 15u) || (((uintptr_t)page_scores) & 3u))
+  if ((((uintptr_t)q) & 3u) || (((uintptr_t)meta_planes) & 15u) || (((uintptr_t)meta) & 15u) ||
+      (((uintptr_t)page_scores) & 3u))
     return TWL_EALIGN;
   twl::PlaneScoreArgs a{};
   a.q = q; a.planes = (const uint16_t*)meta_planes; a.cap = plane_cap_pages;
   a.slots = plane_slots; a.num_slots = plane_num_slots;
+  a.meta = (const uint8_t*)meta; a.kv_page_indices = kv_page_indices;
   a.kv_page_indptr = kv_page_indptr; a.num_q_heads = num_q_heads; a.num_kv_heads = num_kv_heads;
   a.max_pages = max_pages_per_req; a.page_scores = page_scores; a.score_stride = score_stride;
   const dim3 grid((max_pages_per_req + twl::kPsPagesPerBlock - 1) / twl::kPsPagesPerBlock,

@@ -141,6 +141,21 @@ __device__ __forceinline__ int wave_inclusive_scan(int v) {
   return v;
 }
 
+// Quest score of ONE page from its 512-byte metadata record (chunks of min[4c..4c+3],
+// max[4c..4c+3]) by a whole wavefront: lane l takes channels 2l and 2l + 1 (q0, q1 = the query
+// there) and the sum is folded in a fixed order. The plane-layout scoring passes use it for a
+// request's LAST page, whose plane entries are only written when the page is complete.
+template <int DT>
+__device__ __forceinline__ float record_page_score(const uint8_t* rec, float q0, float q1) {
+  const int lane = lane_id();
+  const int c = lane >> 1, o = (lane & 1) * 4;
+  const uint32_t mn = *(const uint32_t*)(rec + 16 * c + o);
+  const uint32_t mx = *(const uint32_t*)(rec + 16 * c + 8 + o);
+  const float v0 = bits16_to_f32<DT>((q0 > 0.0f ? mx : mn) & 0xFFFFu);
+  const float v1 = bits16_to_f32<DT>((q1 > 0.0f ? mx : mn) >> 16);
+  return wave_allreduce<OpSum>(fmaf(q1, v1, q0 * v0));
+}
+
 // Slot of a request's plane-layout metadata: the request's position in the batch, or, with a slot
 // table, the entry of that position (clamped, so that a corrupt table cannot leave the buffer).
 __device__ __forceinline__ uint32_t plane_slot(const int32_t* slots, uint32_t num_slots, uint32_t b) {
