@@ -36,6 +36,8 @@ class PagedKVCache:
         self.kv_last_page_len: Optional[torch.Tensor] = None
         self.max_pages_per_req = 0
         self._seq_lens = None  # host copy, for append bookkeeping
+        self._room = 0         # appends that surely fit every request's last page
+        self._append_key = None
         # Quest metadata in plane layout [slots, Hkv, 128, 2, cap] (see enable_planes) and the
         # slot of every request of the batch (None: slot = position in the batch)
         self.meta_planes: Optional[torch.Tensor] = None
@@ -56,6 +58,8 @@ class PagedKVCache:
         ipl = ip.tolist()
         self._per_req = [ids[ipl[b]:ipl[b + 1]] for b in range(len(ipl) - 1)]
         self._last = kv_last_page_len.cpu().tolist()
+        self._room = PAGE - max(self._last) if self._last else 0
+        self._append_key = None
 
     @property
     def batch(self) -> int:
@@ -162,13 +166,15 @@ class PagedKVCache:
         B = self.batch
         per_req, last = self._per_req, self._last
         grew = False
-        for b in range(B):
-            if last[b] == PAGE:
-                if not free_pages:
-                    raise RuntimeError("PagedKVCache.append: no free page left")
-                per_req[b].append(int(free_pages.pop(0)))
-                last[b] = 0
-                grew = True
+        if self._room <= 0:  # some request may have filled its last page
+            for b in range(B):
+                if last[b] == PAGE:
+                    if not free_pages:
+                        raise RuntimeError("PagedKVCache.append: no free page left")
+                    per_req[b].append(int(free_pages.pop(0)))
+                    last[b] = 0
+                    grew = True
+            self._room = PAGE - max(last)
         if grew:  # a request took a new page: the CSR arrays change shape, lengths are re-sent
             flat = [p for r in per_req for p in r]
             ptr = [0]
@@ -182,14 +188,42 @@ class PagedKVCache:
                                    "(enable_planes with a larger cap_pages)")
             # same tensor object every step, so cached argument blocks of the layer stay valid
             self.kv_last_page_len.copy_(torch.tensor(last, dtype=torch.int32))
-        k_new = k_new.to(self.device, self.dtype)
-        v_new = v_new.to(self.device, self.dtype)
+        if k_new.device != self.device or k_new.dtype != self.dtype:
+            k_new = k_new.to(self.device, self.dtype)
+        if v_new.device != self.device or v_new.dtype != self.dtype:
+            v_new = v_new.to(self.device, self.dtype)
         if k_new.stride(-1) != 1 or v_new.stride() != k_new.stride():
             k_new, v_new = k_new.contiguous(), v_new.contiguous()
-        # one launch: rows, INT4 codes, min/max metadata, and the device-side lengths + 1
-        kv_append(k_new, v_new, self.k_cache, self.v_cache, self.kv_page_indices,
-                  self.kv_page_indptr, self.kv_last_page_len, self.k_int4, self.meta,
-                  self.meta_planes, self.plane_slots if self.meta_planes is not None else None)
+        # one launch: rows, INT4 codes, min/max metadata, and the device-side lengths + 1. The
+        # operands are checked (kv_append) when any of them changes; between such changes the
+        # call goes straight to the library with the checked shapes.
+        planes = self.meta_planes
+        slots = self.plane_slots if planes is not None else None
+        key = (tuple(k_new.shape), k_new.stride(), k_new.dtype, self.k_cache.data_ptr(),
+               self.v_cache.data_ptr(), self.kv_page_indices.data_ptr(),
+               self.kv_page_indptr.data_ptr(), self.kv_last_page_len.data_ptr(),
+               self.k_int4.data_ptr(), self.meta.data_ptr(),
+               0 if planes is None else planes.data_ptr(), 0 if slots is None else slots.data_ptr())
+        if key != self._append_key:
+            kv_append(k_new, v_new, self.k_cache, self.v_cache, self.kv_page_indices,
+                      self.kv_page_indptr, self.kv_last_page_len, self.k_int4, self.meta, planes, slots)
+            self._append_key = key
+        else:
+            ks = self.k_cache.stride()
+            with torch.cuda.device(self.device):
+                rc = _lib.lib().twl_kv_append(
+                    k_new.data_ptr(), v_new.data_ptr(), _lib.TWL_F16 if self.dtype == torch.float16
+                    else _lib.TWL_BF16, k_new.stride(0), k_new.stride(1), self.k_cache.data_ptr(),
+                    self.v_cache.data_ptr(), ks[0], ks[1], ks[2], self.kv_page_indices.data_ptr(),
+                    self.kv_page_indptr.data_ptr(), self.kv_last_page_len.data_ptr(), B,
+                    self.num_kv_heads, self.k_int4.data_ptr(), self.meta.data_ptr(),
+                    0 if planes is None else planes.data_ptr(),
+                    0 if planes is None else planes.size(4),
+                    0 if slots is None else slots.data_ptr(),
+                    0 if planes is None else planes.size(0),
+                    torch.cuda.current_stream(self.device).cuda_stream)
+            _lib.check(rc, "KvAppend")
+        self._room -= 1
         for b in range(B):
             last[b] += 1
             self._seq_lens[b] += 1
