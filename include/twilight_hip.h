@@ -72,7 +72,9 @@ enum twl_top_p_high {
 };
 
 const char* twl_strerror(int status);
-/* ABI version of this header; bumps when a signature changes. */
+/* ABI version of this header; bumps when a signature changes. twl_abi_version() returns the
+ * version the library was built with: a caller compares the two before anything else. */
+#define TWL_ABI_VERSION 5
 int twl_abi_version(void);
 /* Number of HIP devices visible, or a negative twl_status. */
 int twl_device_count(void);

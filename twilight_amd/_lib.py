@@ -14,6 +14,7 @@ from .build import LIB_PATH
 
 TWL_OK = 0
 TWL_F16, TWL_BF16, TWL_F32 = 0, 1, 2
+ABI_VERSION = 5  # TWL_ABI_VERSION of include/twilight_hip.h, checked when the library is loaded
 TWL_HIGH_FIRST, TWL_HIGH_MAX = 0, 1
 PAGE = 16
 HEAD_DIM = 128
@@ -74,6 +75,11 @@ def lib() -> ctypes.CDLL:
     L.twl_strerror.argtypes = [c_int]
     L.twl_strerror.restype = c_char_p
     L.twl_abi_version.argtypes = []
+    L.twl_abi_version.restype = c_int
+    if L.twl_abi_version() != ABI_VERSION:
+        raise RuntimeError(
+            f"{LIB_PATH} has ABI version {L.twl_abi_version()}, this package binds version "
+            f"{ABI_VERSION}: rebuild it with `python -m twilight_amd.build`")
     L.twl_device_count.argtypes = []
     L.twl_top_p_f32.argtypes = [vp, vp, vp, vp, vp, f32, u32, u32, u32, i32, vp, vp, vp]
     L.twl_top_p_f16.argtypes = [vp, i32, vp, vp, vp, vp, f32, u32, u32, u32, i32, vp, vp, vp]

@@ -15,7 +15,7 @@ extern "C" const char* twl_strerror(int status) {
   }
 }
 
-extern "C" int twl_abi_version(void) { return 5; }
+extern "C" int twl_abi_version(void) { return TWL_ABI_VERSION; }
 
 extern "C" int twl_device_count(void) {
   int n = 0;
