@@ -114,3 +114,53 @@ def test_patch_after_prefill_and_without_hf_cache_updates(dev):
     c, lc = run(True, False)
     assert torch.equal(a, b) and torch.equal(a, c)
     assert la == [95, 95, 95, 95] and lb == la and lc == [95, 95, 90, 90]
+
+
+def test_score_info_reports_kept_attention_mass(dev):
+    # p = 1 with a budget beyond the context keeps every token whose estimated probability is not
+    # zero: the kept share of the true attention mass is 1 up to the tokens the estimate flushed;
+    # at p = 0.9 with 64 of 300 tokens it lies strictly between 0 and 1 and equals a direct
+    # evaluation from the layer's own lists
+    model = _tiny_llama(layers=4, heads=4, kv_heads=2, dtype=torch.float16).to(dev)
+    ids = torch.randint(0, 97, (2, 300), generator=torch.Generator().manual_seed(6)).to(dev)
+    nxt = torch.randint(0, 97, (2, 3), generator=torch.Generator().manual_seed(7)).to(dev)
+    cfg = json.loads(json.dumps(CFG))
+    cfg["selector"]["token_budget"] = 4096
+    cfg["weight_pruner"]["threshold"] = 1.0
+    _, score = hf.enable_sparse_attention(model, cfg, enable_score_info=True)
+    _forced_decode(model, ids, nxt)
+    assert len(score._score_sum) == 3 and sorted(score._score_sum[0]) == [2, 3]
+    for q in score._score_sum:
+        for v in q.values():
+            assert v.shape == (8,) and float(v.min()) > 0.999 and float(v.max()) < 1.0001
+    assert score.get_total_avg_score() > 0.999
+    hf.disable_sparse_attention(model)
+
+    _, score = hf.enable_sparse_attention(model, CFG, enable_score_info=True)
+    _forced_decode(model, ids, nxt)
+    v = score._score_sum[-1][3].cpu()
+    assert float(v.min()) > 0.2 and float(v.max()) < 0.9999
+    # the function itself, on layer 3's cache: every token kept gives 1 ...
+    st = model.model.layers[3].self_attn._twilight_state
+    c, lay = st.cache, st.layer
+    B, H = lay.count.shape
+    n = st.seq_len
+    ptr = c.kv_page_indptr.tolist()
+    full = torch.arange(n, dtype=torch.int32, device=dev).expand(B, H, n).contiguous()
+    cnt_full = torch.full((B, H), n, dtype=torch.int32, device=dev)
+    q = torch.randn(B, H, 128, generator=torch.Generator().manual_seed(8)).to(dev, torch.float16)
+    ones = hf.kept_attention_mass(c, q, full, cnt_full, lay.sm_scale)
+    assert torch.allclose(ones, torch.ones_like(ones), atol=1e-5)
+    # ... and a hand-made list its closed form: mass of tokens {0, n-1} = (e^{s0} + e^{s_last}) / sum e^{s}
+    two = torch.zeros((B, H, 4), dtype=torch.int32, device=dev)
+    two[:, :, 1] = n - 1
+    got = hf.kept_attention_mass(c, q, two, torch.full((B, H), 2, dtype=torch.int32, device=dev),
+                                 lay.sm_scale).cpu()
+    for b in range(B):
+        pages = c.kv_page_indices[ptr[b]:ptr[b + 1]].long()
+        k = c.k_cache[pages].reshape(-1, c.num_kv_heads, 128)[:n].double().cpu()
+        for h in range(H):
+            s = (k[:, h // (H // c.num_kv_heads)] @ q[b, h].double().cpu()) * lay.sm_scale
+            want = float((s[0].exp() + s[-1].exp()) / s.exp().sum())
+            assert abs(float(got[b, h]) - want) < 1e-4
+    hf.disable_sparse_attention(model)

@@ -55,8 +55,24 @@ def test_config_validation():
     cfg["selector"]["chunk_size"] = 32
     with pytest.raises(RuntimeError):
         hf.enable_sparse_attention(m, cfg)
-    with pytest.raises(RuntimeError):
-        hf.enable_sparse_attention(m, CFG, enable_score_info=True)
+
+
+def test_score_info_accounting():
+    # queries split where the layer id does not follow the previous one; averages are over the
+    # per-layer MINIMUM over heads and skip layers 0 and 1 (twilight/pyimpl/state.py:96-132)
+    m = _tiny_llama()
+    info, score = hf.enable_sparse_attention(m, CFG, enable_budget_info=True, enable_score_info=True)
+    assert isinstance(score, hf.HistoryAccumulatedScoreInfo)
+    assert m.model.layers[3].self_attn._twilight_state.score_info is score
+    for query in range(2):
+        for lid in range(4):
+            score.update(lid, torch.tensor([[0.9 + 0.01 * lid, 0.95], [0.99, 0.97 - 0.1 * query]]))
+    assert len(score._min_sum) == 2 and sorted(score._min_sum[0]) == [0, 1, 2, 3]
+    assert score._score_sum[0][2].shape == (4,)
+    per_query = score.get_avg_score_per_query()
+    assert per_query[0] == pytest.approx((0.92 + 0.93) / 2, abs=1e-6)
+    assert per_query[1] == pytest.approx(0.87, abs=1e-6)
+    assert score.get_total_avg_score() == pytest.approx((0.925 + 0.87) / 2, abs=1e-6)
 
 
 def test_reference_config_file_shape_is_accepted():

@@ -86,13 +86,81 @@ class HistoryBudgetInfo:
             print(f"Layer {lid}: {v.tolist()} Head Average: {float(v.float().mean()):.2f}")
 
 
+class HistoryAccumulatedScoreInfo:
+    """Per query and layer: the share of the TRUE attention mass (softmax of q·K/sqrt(d) over the
+    whole context) that the kept tokens carry, per head, and its minimum over the heads. Same
+    accounting as twilight/pyimpl/state.py:82-132 (queries split on the layer id, averages skip
+    layers 0 and 1)."""
+
+    def __init__(self) -> None:
+        self.reset()
+
+    def reset(self) -> None:
+        self._score_sum: List[Dict[int, torch.Tensor]] = []
+        self._min_sum: List[Dict[int, float]] = []
+        self._last_layer_id = -999
+
+    def update(self, layer_id: int, score_sum: torch.Tensor) -> None:
+        """``score_sum``: kept attention mass per (batch, head), any shape; stored flattened."""
+        if layer_id != self._last_layer_id + 1:
+            self._score_sum.append({})
+            self._min_sum.append({})
+        flat = score_sum.detach().flatten().float().clone()
+        self._score_sum[-1][layer_id] = flat
+        self._min_sum[-1][layer_id] = float(flat.min())
+        self._last_layer_id = layer_id
+
+    def print_min_sum_single_query(self, query_index: int = -1) -> None:
+        for lid, v in self._min_sum[query_index].items():
+            print(f"Layer {lid}: {v:.2f}")
+
+    def print_score_sum_single_query(self, query_index: int = -1) -> None:
+        for lid, v in self._score_sum[query_index].items():
+            print(f"Layer {lid}: {v}")
+
+    def get_avg_score_per_query(self) -> List[float]:
+        out = []
+        for q in self._min_sum:
+            vals = [v for lid, v in q.items() if lid > 1]
+            out.append(sum(vals) / len(vals) if vals else float("nan"))
+        return out
+
+    def get_total_avg_score(self) -> float:
+        v = self.get_avg_score_per_query()
+        return sum(v) / len(v) if v else float("nan")
+
+
+def kept_attention_mass(cache: PagedKVCache, q: torch.Tensor, idx: torch.Tensor,
+                        count: torch.Tensor, sm_scale: float) -> torch.Tensor:
+    """Diagnostic, not part of the decode path: for every (request, q head) the sum over the kept
+    tokens ``idx[b, h, :count[b, h]]`` of softmax(q·K·sm_scale) taken over the request's WHOLE
+    context, [B, H] fp32. It reads all of K with plain tensor operations on the GPU, which is what
+    the decode path exists to avoid; the reference's statistic (state.py:96-110) costs the same
+    there, since its dense-masked attention has the full weights at hand."""
+    B, H, _ = q.shape
+    Hkv = cache.num_kv_heads
+    ptr = cache.kv_page_indptr.tolist()
+    last = cache.kv_last_page_len.tolist()
+    out = torch.zeros((B, H), dtype=torch.float32, device=q.device)
+    for b in range(B):
+        pages = cache.kv_page_indices[ptr[b]:ptr[b + 1]].long()
+        n = (len(pages) - 1) * PAGE + last[b]
+        k = cache.k_cache[pages].reshape(-1, Hkv, _lib.HEAD_DIM)[:n].float()      # [n, Hkv, D]
+        k = k.repeat_interleave(H // Hkv, dim=1)                                  # [n, H, D]
+        w = torch.softmax(torch.einsum("hd,nhd->hn", q[b].float(), k) * sm_scale, dim=-1)
+        keep = torch.arange(idx.shape[-1], device=q.device)[None, :] < count[b][:, None]
+        kept = torch.gather(w, 1, idx[b].long().clamp_(0, n - 1)) * keep
+        out[b] = kept.sum(-1)
+    return out
+
+
 class _LayerState:
     """What a patched attention module carries between calls."""
 
     def __init__(self, cfg: dict, reserve_tokens: int, budget_info: Optional[HistoryBudgetInfo],
-                 keep_hf_cache: bool):
+                 keep_hf_cache: bool, score_info: Optional[HistoryAccumulatedScoreInfo] = None):
         self.cfg, self.reserve_tokens, self.budget_info = cfg, reserve_tokens, budget_info
-        self.keep_hf_cache = keep_hf_cache
+        self.keep_hf_cache, self.score_info = keep_hf_cache, score_info
         self.cache: Optional[PagedKVCache] = None
         self.layer: Optional[TwilightDecodeLayer] = None
         self.free: List[int] = []
@@ -159,6 +227,9 @@ def _twilight_attention_forward(self, hidden_states, position_embeddings=None, a
     if st.budget_info is not None:
         st.budget_info.update(self.layer_idx, st.layer.count)
         st.budget_info.update_B0(self.layer_idx, min(st.layer.token_budget, st.seq_len))
+    if st.score_info is not None:
+        st.score_info.update(self.layer_idx, kept_attention_mass(
+            st.cache, q[:, :, 0], st.layer.idx, st.layer.count, st.layer.sm_scale))
     attn_output = self.o_proj(out.reshape(B, 1, -1))
     return attn_output, None
 
@@ -166,17 +237,18 @@ def _twilight_attention_forward(self, hidden_states, position_embeddings=None, a
 def enable_sparse_attention(model, sparse_config: Dict, enable_budget_info: bool = False,
                             enable_score_info: bool = False, reserve_tokens: int = 4096,
                             high: str = "max", keep_hf_cache: bool = True
-                            ) -> Tuple[Optional[HistoryBudgetInfo], None]:
+                            ) -> Tuple[Optional[HistoryBudgetInfo],
+                                       Optional[HistoryAccumulatedScoreInfo]]:
     """Patch every Llama / Mistral attention module of ``model`` (twilight/pyimpl/attention.py:
     351-418, 481-493). ``sparse_config`` is the reference's JSON template
     (benchmark/configs/config_quest_twi.json). ``reserve_tokens``: decode tokens per request the
     paged caches are sized for. ``keep_hf_cache=False`` stops patched layers from also appending
     decode tokens to the model's own cache (a whole-context copy per step with ``DynamicCache``);
     it needs ``skip_first_two_layers`` (layer 0 keeps the sequence length the model asks its cache
-    for) and a sequence that is only prefilled once. Returns ``(budget_info, None)``; the accumulated-score statistic
-    of the reference needs the dense attention weights, which this path never forms."""
-    if enable_score_info:
-        raise RuntimeError("enable_score_info needs dense attention weights; not available here")
+    for) and a sequence that is only prefilled once. Returns ``(budget_info, score_info)`` as the
+    reference does (attention.py:404-418). ``enable_score_info`` adds a dense pass over all of K
+    to every patched layer's decode step (:func:`kept_attention_mass`): a diagnostic, not for
+    timing runs."""
     for part in ("compressor",):
         t = sparse_config.get(part, {}).get("type", "none")
         if str(t).lower() not in ("none", ""):
@@ -189,6 +261,7 @@ def enable_sparse_attention(model, sparse_config: Dict, enable_budget_info: bool
     if not keep_hf_cache and skip == 0:
         raise RuntimeError("keep_hf_cache=False needs skip_first_two_layers")
     budget_info = HistoryBudgetInfo() if enable_budget_info else None
+    score_info = HistoryAccumulatedScoreInfo() if enable_score_info else None
     patched = 0
     for name, module in model.named_modules():
         if not all(hasattr(module, a) for a in ("q_proj", "k_proj", "v_proj", "o_proj", "layer_idx")):
@@ -199,13 +272,14 @@ def enable_sparse_attention(model, sparse_config: Dict, enable_budget_info: bool
             raise RuntimeError("enable_sparse_attention was already called on this model")
         if module.layer_idx < skip:
             continue
-        module._twilight_state = _LayerState(dict(cfg), reserve_tokens, budget_info, keep_hf_cache)
+        module._twilight_state = _LayerState(dict(cfg), reserve_tokens, budget_info, keep_hf_cache,
+                                              score_info)
         module._twilight_orig_forward = module.forward
         module.forward = types.MethodType(_twilight_attention_forward, module)
         patched += 1
     if patched == 0:
         raise RuntimeError("no attention module was patched")
-    return budget_info, None
+    return budget_info, score_info
 
 
 def disable_sparse_attention(model) -> None:
