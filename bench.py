@@ -232,6 +232,163 @@ def bench_ftka(args, dev) -> int:
     return 0
 
 
+def bench_llama3_model(args, dev) -> int:
+    """Whole-model decode at the Llama-3-8B shape: every layer of a random-initialised model
+    (GQA 32 / 8 heads, bf16), B requests with a synthetic context of N tokens already in the
+    caches, decode steps timed end to end — once dense (torch SDPA over a static KV cache) and once
+    with the Select-then-Prune path in layers 2.. (the first two layers stay dense, as the
+    reference's configuration has them, twilight/pyimpl/attention.py:199-201). Everything outside
+    the attention modules is the model's own eager PyTorch code in both runs."""
+    from transformers import DynamicCache, LlamaConfig, LlamaForCausalLM, StaticCache
+    from twilight_amd import hf
+    B, N, nl = args.batch, args.context, args.model_layers
+    steps, warmup = min(args.steps, 32), min(args.warmup, 4)
+    top_p = args.top_p if args.top_p != 0.95 else 0.9    # the configuration's p unless one is given
+    cfg = LlamaConfig(vocab_size=128256, hidden_size=4096, intermediate_size=14336,
+                      num_hidden_layers=nl, num_attention_heads=32, num_key_value_heads=8,
+                      head_dim=128, max_position_embeddings=N + 4096, rope_theta=500000.0,
+                      attn_implementation="sdpa")
+    torch.manual_seed(0)
+    old = torch.get_default_dtype()
+    torch.set_default_dtype(torch.bfloat16)
+    try:
+        with torch.device(dev):
+            model = LlamaForCausalLM(cfg).eval()
+    finally:
+        torch.set_default_dtype(old)
+    # A random-initialised model attends almost uniformly, which no trained model does: scale the
+    # query projection so that the softmax over the context is as peaked as the few hundred kept
+    # tokens per head that the reference reports; the kept count is part of the output.
+    with torch.no_grad():
+        for lay in model.model.layers:
+            lay.self_attn.q_proj.weight.mul_(args.q_gain)
+
+    def kv(layer):
+        g = torch.Generator(device=dev).manual_seed(1000 + layer)
+        k = torch.randn((B, 8, N, 128), generator=g, device=dev, dtype=torch.bfloat16)
+        v = torch.randn((B, 8, N, 128), generator=g, device=dev, dtype=torch.bfloat16)
+        return k, v
+
+    ids = torch.randint(0, cfg.vocab_size, (steps + warmup, B, 1),
+                        generator=torch.Generator().manual_seed(7)).to(dev)
+
+    def run(cache):
+        with torch.no_grad():
+            for s in range(warmup):
+                model(ids[s], past_key_values=cache, use_cache=True)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for s in range(warmup, warmup + steps):
+                out = model(ids[s], past_key_values=cache, use_cache=True)
+            torch.cuda.synchronize()
+            return (time.perf_counter() - t0) / steps, out.logits[:, -1].float()
+
+    reserve = steps + warmup + 16
+
+    def make_cache(kind, layers):
+        # "static": preallocated K / V, attention over the whole buffer under a mask;
+        # "dynamic": K / V grown by concatenation every step, attention without a mask
+        c = (StaticCache(config=cfg, max_cache_len=N + reserve) if kind == "static"
+             else DynamicCache(config=cfg))
+        for i in layers:
+            c.update(*kv(i), i)
+        return c
+
+    dense = {}
+    if not args.no_dense:
+        for kind in ("static", "dynamic"):
+            cache = make_cache(kind, range(nl))
+            t, _ = run(cache)
+            dense[kind] = t * 1e3
+            del cache
+            torch.cuda.empty_cache()
+
+    sparse_cfg = {"compressor": {"type": "none"},
+                  "selector": {"type": "quest", "token_budget": args.budget, "chunk_size": 16},
+                  "weight_estimator": {"type": "min_max_quant", "quant_bit": 4},
+                  "weight_pruner": {"type": "top_p", "threshold": top_p},
+                  "skip_first_two_layers": True, "use_estimated_weights_in_attn": False}
+    info, _ = hf.enable_sparse_attention(model, sparse_cfg, enable_budget_info=True,
+                                         reserve_tokens=2 * reserve + 16, keep_hf_cache=False)
+    patched = [hasattr(model.model.layers[i].self_attn, "_twilight_state") for i in range(nl)]
+    twi = {}
+    for kind in ("static", "dynamic"):
+        # the model's own cache serves the two dense layers; the patched ones page their K / V
+        cache = make_cache(kind, [i for i in range(nl) if not patched[i]])
+        for i in range(nl):
+            if patched[i]:
+                st = model.model.layers[i].self_attn._twilight_state
+                st.reset()
+                hf.fill_from_prefill(st, *kv(i), cfg.num_attention_heads)
+        info.reset()
+        t, logits = run(cache)
+        twi[kind] = t * 1e3
+        if kind == "static":
+            del cache
+            torch.cuda.empty_cache()
+    kept = info.get_total_avg_budget()
+    best = min(twi, key=twi.get)
+    twi_ms = twi[best]
+    dense_best = min(dense, key=dense.get) if dense else None
+    dense_ms = dense[dense_best] if dense else None
+    # GPU time of the decode-layer calls alone, by events around them in one more step
+    ev = []
+
+    def timed(lay):
+        def call(q):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            o = lay(q)
+            e1.record()
+            ev.append((e0, e1))
+            return o
+        return call
+
+    for i in range(nl):
+        st = getattr(model.model.layers[i].self_attn, "_twilight_state", None)
+        if st is not None:
+            st.layer = _Timed(st.layer, timed(st.layer))
+    with torch.no_grad():
+        model(ids[0], past_key_values=cache, use_cache=True)
+    torch.cuda.synchronize()
+    layer_us = sum(a.elapsed_time(b) for a, b in ev) * 1e3 / max(len(ev), 1)
+    print(json.dumps({
+        "metric": "tokens/s, whole-model decode with Twilight applied", "value": round(B / twi_ms * 1e3, 1),
+        "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": round(twi_ms, 3), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"random-init Llama-3-8B shape, {nl} layers, GQA 32/8, bf16, B={B}, "
+                               f"context {N} (synthetic K/V), budget {args.budget}, p={top_p}, "
+                               f"layers 0-1 dense, q_proj x{args.q_gain}"},
+        "model_cache": best,
+        "ms_per_step_by_model_cache": {k: round(v, 3) for k, v in twi.items()},
+        "dense": None if dense_ms is None else {
+            "ms_per_step": round(dense_ms, 3), "tokens_per_s": round(B / dense_ms * 1e3, 1),
+            "model_cache": dense_best,
+            "ms_per_step_by_model_cache": {k: round(v, 3) for k, v in dense.items()},
+            "what": "same model and context, every layer through the model's own attention "
+                    "(torch SDPA) over the transformers cache class named"},
+        "speedup_vs_dense": None if dense_ms is None else round(dense_ms / twi_ms, 2),
+        "kept_tokens_per_head_mean": round(kept, 1),
+        "twilight_layer_us": round(layer_us, 1),
+        "finite_logits": bool(torch.isfinite(logits).all()),
+    }))
+    return 0
+
+
+class _Timed:
+    """Stands in for a decode layer object: calls go through ``fn``, attributes to the layer."""
+
+    def __init__(self, layer, fn):
+        self._layer, self._fn = layer, fn
+
+    def __call__(self, q):
+        return self._fn(q)
+
+    def __getattr__(self, name):
+        return getattr(self._layer, name)
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -241,12 +398,18 @@ def main() -> int:
     ap.add_argument("--context", type=int, default=32768)
     ap.add_argument("--budget", type=int, default=8192)
     ap.add_argument("--top-p", type=float, default=0.95)
-    ap.add_argument("--workload", choices=["longchat", "llama3", "topp", "ftka"], default="longchat",
+    ap.add_argument("--workload", choices=["longchat", "llama3", "llama3-model", "topp", "ftka"],
+                    default="longchat",
                     help="longchat: 32 MHA heads fp16 (the headline workload); llama3: GQA 32/8 "
                          "bf16, with a dense-decode baseline (the same attention kernel over "
                          "every token); topp: the pruner kernel alone on [8,32,8192] scores; "
                          "ftka: the NHD GEMV call shapes of the reference's bench_gemv.py and the "
-                         "Double-Sparse label ops")
+                         "Double-Sparse label ops; llama3-model: whole-model decode of a "
+                         "random-initialised Llama-3-8B shape, dense against Twilight, tokens/s")
+    ap.add_argument("--model-layers", type=int, default=32, help="llama3-model: number of layers")
+    ap.add_argument("--q-gain", type=float, default=3.0,
+                    help="llama3-model: factor on the random q_proj weights (peakedness of attention)")
+    ap.add_argument("--no-dense", action="store_true", help="llama3-model: skip the dense run")
     ap.add_argument("--layers", type=int, default=4,
                     help="independent layer caches visited round-robin (cold-cache steps)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -279,6 +442,8 @@ def main() -> int:
         return bench_topp(args, L, dev)
     if args.workload == "ftka":
         return bench_ftka(args, dev)
+    if args.workload == "llama3-model":
+        return bench_llama3_model(args, dev)
     llama = args.workload == "llama3"
     B, H, Hkv, N, D = args.batch, 32, (8 if llama else 32), args.context, 128
     npg = N // 16

@@ -170,9 +170,11 @@ class _LayerState:
         self.cache, self.layer, self.free, self.seq_len = None, None, [], 0
 
 
-def _fill_from_prefill(st: _LayerState, k: torch.Tensor, v: torch.Tensor, num_q_heads: int) -> None:
+def fill_from_prefill(st: _LayerState, k: torch.Tensor, v: torch.Tensor, num_q_heads: int) -> None:
     """Page the prefill K / V [B, Hkv, N, 128] of a layer and size everything for
-    ``reserve_tokens`` more tokens per request."""
+    ``reserve_tokens`` more tokens per request. The first decode step of a patched module calls
+    this on what the model's cache holds; a caller that has the K / V of a context from elsewhere
+    may call it on ``module._twilight_state`` itself and decode from there."""
     B, _, N, _ = k.shape
     npg = (N + PAGE - 1) // PAGE
     spare_per_req = (st.reserve_tokens + PAGE - 1) // PAGE + 1
@@ -211,7 +213,7 @@ def _twilight_attention_forward(self, hidden_states, position_embeddings=None, a
             raise RuntimeError("decode step without prefilled K / V of this layer on a GPU (the "
                                "path has no CPU implementation and needs use_cache=True)")
         n = st.seq_len if st.seq_len > 0 else past_key_values.get_seq_length(self.layer_idx)
-        _fill_from_prefill(st, keys[:, :, :n], lay.values[:, :, :n], self.config.num_attention_heads)
+        fill_from_prefill(st, keys[:, :, :n], lay.values[:, :, :n], self.config.num_attention_heads)
     B = hidden_states.shape[0]
     hidden_shape = (B, 1, -1, self.head_dim)
     q = self.q_proj(hidden_states).view(hidden_shape).transpose(1, 2)
