@@ -272,14 +272,17 @@ def bench_llama3_model(args, dev) -> int:
     ids = torch.randint(0, cfg.vocab_size, (steps + warmup, B, 1),
                         generator=torch.Generator().manual_seed(7)).to(dev)
 
-    def run(cache):
+    def run(cache, positions=False):
+        # positions: pass position_ids explicitly (needed when nothing updates the model's cache)
+        def pos(s):
+            return {"position_ids": torch.full((B, 1), N + s, device=dev)} if positions else {}
         with torch.no_grad():
             for s in range(warmup):
-                model(ids[s], past_key_values=cache, use_cache=True)
+                model(ids[s], past_key_values=cache, use_cache=True, **pos(s))
             torch.cuda.synchronize()
             t0 = time.perf_counter()
             for s in range(warmup, warmup + steps):
-                out = model(ids[s], past_key_values=cache, use_cache=True)
+                out = model(ids[s], past_key_values=cache, use_cache=True, **pos(s))
             torch.cuda.synchronize()
             return (time.perf_counter() - t0) / steps, out.logits[:, -1].float()
 
@@ -308,25 +311,25 @@ def bench_llama3_model(args, dev) -> int:
                   "weight_estimator": {"type": "min_max_quant", "quant_bit": 4},
                   "weight_pruner": {"type": "top_p", "threshold": top_p},
                   "skip_first_two_layers": True, "use_estimated_weights_in_attn": False}
-    info, _ = hf.enable_sparse_attention(model, sparse_cfg, enable_budget_info=True,
-                                         reserve_tokens=2 * reserve + 16, keep_hf_cache=False)
-    patched = [hasattr(model.model.layers[i].self_attn, "_twilight_state") for i in range(nl)]
     twi = {}
-    for kind in ("static", "dynamic"):
-        # the model's own cache serves the two dense layers; the patched ones page their K / V
-        cache = make_cache(kind, [i for i in range(nl) if not patched[i]])
+    for mode in ("model", "paged"):
+        # "model": the two dense layers run the model's own attention over a DynamicCache;
+        # "paged": they run twl_group_attn over paged K / V and the model's cache stays empty
+        info, _ = hf.enable_sparse_attention(model, sparse_cfg, enable_budget_info=True,
+                                             reserve_tokens=reserve + 16, keep_hf_cache=False,
+                                             dense_layers=mode)
+        states = [getattr(model.model.layers[i].self_attn, "_twilight_state", None) for i in range(nl)]
+        cache = make_cache("dynamic", [i for i in range(nl) if states[i] is None])
         for i in range(nl):
-            if patched[i]:
-                st = model.model.layers[i].self_attn._twilight_state
-                st.reset()
-                hf.fill_from_prefill(st, *kv(i), cfg.num_attention_heads)
-        info.reset()
-        t, logits = run(cache)
-        twi[kind] = t * 1e3
-        if kind == "static":
-            del cache
+            if states[i] is not None:
+                hf.fill_from_prefill(states[i], *kv(i), cfg.num_attention_heads)
+        t, logits = run(cache, positions=True)
+        twi[mode] = t * 1e3
+        kept = info.get_total_avg_budget()
+        if mode == "model":
+            hf.disable_sparse_attention(model)
+            del cache, states
             torch.cuda.empty_cache()
-    kept = info.get_total_avg_budget()
     best = min(twi, key=twi.get)
     twi_ms = twi[best]
     dense_best = min(dense, key=dense.get) if dense else None
@@ -346,10 +349,11 @@ def bench_llama3_model(args, dev) -> int:
 
     for i in range(nl):
         st = getattr(model.model.layers[i].self_attn, "_twilight_state", None)
-        if st is not None:
+        if st is not None and not st.dense:
             st.layer = _Timed(st.layer, timed(st.layer))
     with torch.no_grad():
-        model(ids[0], past_key_values=cache, use_cache=True)
+        model(ids[0], past_key_values=cache, use_cache=True,
+              position_ids=torch.full((B, 1), N + steps + warmup, device=dev))
     torch.cuda.synchronize()
     layer_us = sum(a.elapsed_time(b) for a, b in ev) * 1e3 / max(len(ev), 1)
     print(json.dumps({
@@ -360,8 +364,10 @@ def bench_llama3_model(args, dev) -> int:
         "config": {"workload": f"random-init Llama-3-8B shape, {nl} layers, GQA 32/8, bf16, B={B}, "
                                f"context {N} (synthetic K/V), budget {args.budget}, p={top_p}, "
                                f"layers 0-1 dense, q_proj x{args.q_gain}"},
-        "model_cache": best,
-        "ms_per_step_by_model_cache": {k: round(v, 3) for k, v in twi.items()},
+        "dense_layers_what": "how layers 0-1 decode: 'model' = the model's own attention (torch "
+                             "SDPA) over a DynamicCache, 'paged' = twl_group_attn over paged K/V",
+        "dense_layers": best,
+        "ms_per_step_by_dense_layers": {k: round(v, 3) for k, v in twi.items()},
         "dense": None if dense_ms is None else {
             "ms_per_step": round(dense_ms, 3), "tokens_per_s": round(B / dense_ms * 1e3, 1),
             "model_cache": dense_best,
@@ -662,6 +668,21 @@ def main() -> int:
                          "used densely: K/V are fetched per q head, 4x the bytes counted here, "
                          "which count K/V once per kv head)"}
         del full_idx, ws
+        # the group kernel: K / V of a token fetched once for the 4 q heads of its kv head
+        gws = torch.empty(int(L.twl_group_attn_workspace_bytes(B, H, Hkv, N, 0)), dtype=torch.uint8,
+                          device=dev)
+        fn = rotating(lambda l, c, q: lambda: L.twl_group_attn(
+            p(q), p(outd), qcode, p(c.k_cache), p(c.v_cache), *c.k_cache.stride()[:3], 0, 0, 0, N,
+            p(c.kv_page_indices), p(c.kv_page_indptr), p(c.kv_last_page_len), B, H, Hkv, sm, 0,
+            p(gws), gws.numel(), stream))
+        us = _time_calls(fn, 40, nl)
+        dense["group_attn_us"] = round(us, 2)
+        dense["group_attn_GBps"] = round(nbytes / us / 1e3, 1)
+        dense["group_attn_frac_of_hbm_peak"] = round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)
+        dense["group_attn_what"] = ("twl_group_attn over every token (dense paged decode, K/V read "
+                                    "once per kv head, two launches: partial results + merge), "
+                                    "cold caches")
+        del gws
         # torch's own dense decode attention over contiguous K/V of one layer (GQA-aware)
         try:
             c0 = layers[0].cache

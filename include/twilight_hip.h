@@ -74,7 +74,7 @@ enum twl_top_p_high {
 const char* twl_strerror(int status);
 /* ABI version of this header; bumps when a signature changes. twl_abi_version() returns the
  * version the library was built with: a caller compares the two before anything else. */
-#define TWL_ABI_VERSION 5
+#define TWL_ABI_VERSION 6
 int twl_abi_version(void);
 /* Number of HIP devices visible, or a negative twl_status. */
 int twl_device_count(void);
@@ -240,6 +240,44 @@ int twl_sparse_attn(const void* q, void* out, int dtype, const void* k_cache, co
                     const int32_t* kv_page_indices, const int32_t* kv_page_indptr, uint32_t batch,
                     uint32_t num_q_heads, uint32_t num_kv_heads, float sm_scale, float* lse_out,
                     void* workspace, uint64_t workspace_bytes, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Paged decode attention with ONE token list per (request, kv head), shared by the kv head's
+ * G = num_q_heads / num_kv_heads query heads (G in {1, 2, 4, 8}): K and V of a token are fetched
+ * once for the group.
+ * Replaces: the same masked softmax.V of twilight/pyimpl/attention.py:188-190,299-306, (a) over
+ * every token of the request (group_idx == NULL; kv_last_page_len gives the length): the dense
+ * decode of the layers a configuration leaves dense (attention.py:199-201, config default :413)
+ * and the dense baseline; (b) over group_idx int32 [batch, num_kv_heads, idx_stride] ascending
+ * token positions with group_count int32 [batch, num_kv_heads], e.g. the union of the group's
+ * survivor sets (twl_group_union): the "top-p per kv-head group" reading of GQA, where the
+ * reference itself repeats K / V per q head (attention.py:124-126).
+ * max_tokens: upper bound of the request lengths (dense form: tokens of a request beyond it are
+ * not attended to; ignored with a list, whose bound is idx_stride). out [batch, num_q_heads, 128] in dtype, lse_out (nullable) float
+ * [batch, num_q_heads]; an empty list gives a zero row and lse -inf. workspace: at least
+ * twl_group_attn_workspace_bytes(...) bytes, 16-byte aligned, no initial contents required; two
+ * calls that share it must not overlap in time. The softmax weights stay in fp32 (they are not
+ * rounded to dtype before the V product as attention.py:302-304 does; the difference is below
+ * the rounding of the output).
+ * ------------------------------------------------------------------------------------------- */
+uint64_t twl_group_attn_workspace_bytes(uint32_t batch, uint32_t num_q_heads,
+                                        uint32_t num_kv_heads, uint32_t max_tokens, int with_list);
+int twl_group_attn(const void* q, void* out, int dtype, const void* k_cache, const void* v_cache,
+                   uint64_t page_stride, uint64_t token_stride, uint64_t head_stride,
+                   const int32_t* group_idx, uint32_t idx_stride, const int32_t* group_count,
+                   uint32_t max_tokens, const int32_t* kv_page_indices,
+                   const int32_t* kv_page_indptr, const int32_t* kv_last_page_len, uint32_t batch,
+                   uint32_t num_q_heads, uint32_t num_kv_heads, float sm_scale, float* lse_out,
+                   void* workspace, uint64_t workspace_bytes, void* stream);
+/* Union of the survivor lists of each kv head's q heads (mask OR over the group; the per-head
+ * lists are those of twl_top_p_* / twl_decode_layer: idx int32 [batch, num_q_heads, idx_stride],
+ * count int32 [batch, num_q_heads]). Token positions must be < max_tokens (<= 262144). Output:
+ * group_idx int32 [batch, num_kv_heads, group_stride] ascending, group_count int32
+ * [batch, num_kv_heads]; a union longer than group_stride is cut to its first group_stride
+ * positions (group_stride >= min(max_tokens, G * idx_stride) never cuts). */
+int twl_group_union(const int32_t* idx, uint32_t idx_stride, const int32_t* count, uint32_t batch,
+                    uint32_t num_q_heads, uint32_t num_kv_heads, uint32_t max_tokens,
+                    int32_t* group_idx, uint32_t group_stride, int32_t* group_count, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Quest page selector: page score + top-k pages per row.
@@ -418,6 +456,17 @@ typedef struct twl_layer_args {
    * way; with 0, `scores` and `page_scores` are guaranteed filled only when keep_scores != 0. */
   int split_estimator;
   int keep_scores;
+  /* Group attention (optional; group_idx == NULL: every q head attends over its own survivor
+   * list, as the reference's repeated K / V does, attention.py:124-126). With group_idx the q
+   * heads of a kv head attend over the UNION of their survivor lists (twl_group_union, then
+   * twl_group_attn): group_idx int32 [batch, num_kv_heads, group_idx_stride] and group_count
+   * int32 [batch, num_kv_heads] receive the unions; group_idx_stride >= min(16 *
+   * max_pages_per_req, G * 16 * k) never cuts one. group_workspace: at least
+   * twl_group_attn_workspace_bytes(batch, num_q_heads, num_kv_heads, group_idx_stride, 1) bytes.
+   * Needs 16 * max_pages_per_req <= 262144 and G in {1, 2, 4, 8}. */
+  int32_t* group_idx; uint32_t group_idx_stride;
+  int32_t* group_count;
+  void* group_workspace; uint64_t group_workspace_bytes;
 } twl_layer_args;
 
 int twl_decode_layer(const twl_layer_args* args, void* stream);

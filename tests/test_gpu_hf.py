@@ -164,3 +164,35 @@ def test_score_info_reports_kept_attention_mass(dev):
             want = float((s[0].exp() + s[-1].exp()) / s.exp().sum())
             assert abs(float(got[b, h]) - want) < 1e-4
     hf.disable_sparse_attention(model)
+
+
+def test_paged_dense_layers_reproduce_dense_decode(dev):
+    # dense_layers="paged": layers 0-1 decode from paged K / V through the group attention kernel;
+    # with p = 1 and a budget beyond the context the whole model must reproduce dense decoding.
+    # With keep_hf_cache=False nothing updates the model's cache, so positions are passed in.
+    model = _tiny_llama(layers=4, heads=4, kv_heads=2, dtype=torch.float16).to(dev)
+    ids = torch.randint(0, 97, (2, 150), generator=torch.Generator().manual_seed(9)).to(dev)
+    ref_logits, toks = _decode(model, ids, 20)            # crosses a page boundary
+    cfg = json.loads(json.dumps(CFG))
+    cfg["selector"]["token_budget"] = 4096
+    cfg["weight_pruner"]["threshold"] = 1.0
+    for keep in (True, False):
+        hf.enable_sparse_attention(model, cfg, reserve_tokens=64, dense_layers="paged",
+                                   keep_hf_cache=keep)
+        states = [l.self_attn._twilight_state for l in model.model.layers]
+        assert [s.dense for s in states] == [True, True, False, False]
+        logits = []
+        with torch.no_grad():
+            out = model(ids, use_cache=True)
+            past = out.past_key_values
+            for s in range(toks.shape[1]):
+                pos = torch.full((2, 1), 150 + s, device=dev)
+                out = model(toks[:, s:s + 1], past_key_values=past, use_cache=True, position_ids=pos)
+                past = out.past_key_values
+                logits.append(out.logits[:, -1].float())
+        got = torch.stack(logits)
+        assert torch.allclose(got, ref_logits, rtol=2e-2, atol=2e-2), (keep, (got - ref_logits).abs().max())
+        assert past.get_seq_length(0) == (170 if keep else 150)
+        hf.disable_sparse_attention(model)
+    with pytest.raises(RuntimeError):
+        hf.enable_sparse_attention(model, cfg, dense_layers="flash")

@@ -393,3 +393,44 @@ def test_plane_slot_table(dev):
         slotted.set_plane_slots(torch.tensor([4, 4], dtype=torch.int32))   # one slot, two requests
     with pytest.raises(RuntimeError):
         slotted.set_plane_slots(torch.tensor([4, 5], dtype=torch.int32))   # outside the buffer
+
+
+@pytest.mark.parametrize("B,H,Hkv,N,budget,dt,planes", [
+    (2, 8, 2, 1200, 512, torch.float16, False),          # three launches, G = 4
+    (4, 32, 8, 2048, 1024, torch.bfloat16, True),        # Llama-3 grouping, one-launch kernel
+    (1, 4, 4, 700, 256, torch.float16, False)])          # G = 1: the union is the head's own list
+def test_layer_group_union_attention(dev, B, H, Hkv, N, budget, dt, planes):
+    # group_union: the q heads of a kv head attend over the union of their survivor lists. The
+    # per-head lists are the pruner's (unchanged); the union and the attention over it are checked
+    # against the oracle's masked attention with the OR of the group's masks
+    p, G = 0.9, H // Hkv
+    q, k, v = synth.heavy_hitter_qkv(B, H, N, n_heavy=12, mass=0.6, seed=N, dtype=dt)
+    kk, vv = k[:, ::G].contiguous(), v[:, ::G].contiguous()
+    npg = (N + 15) // 16
+    cache = PagedKVCache.from_dense(kk.to(dt), vv.to(dt), dev,
+                                    page_perm=torch.randperm(B * npg, generator=torch.Generator().manual_seed(1)),
+                                    plane_pages=npg if planes else None)
+    qd = q[:, :, 0].to(dt).to(dev)
+    plain = TwilightDecodeLayer(cache, H, token_budget=budget, top_p=p)
+    out_plain = plain(qd).clone()
+    layer = TwilightDecodeLayer(cache, H, token_budget=budget, top_p=p, group_union=True)
+    out = layer(qd).cpu().float()
+    rows = B * H
+    assert torch.equal(layer.count, plain.count)
+    idx = layer.idx.cpu().numpy().reshape(rows, -1)
+    cnt = layer.count.cpu().numpy().reshape(rows)
+    own = _lists_to_mask(idx, cnt, N)                                        # [rows, N]
+    union = own.reshape(B, Hkv, G, N).any(2)                                 # [B, Hkv, N]
+    gidx = layer.group_idx.cpu().numpy().reshape(B * Hkv, -1)
+    gcnt = layer.group_count.cpu().numpy().reshape(B * Hkv)
+    assert np.array_equal(_lists_to_mask(gidx, gcnt, N), union.reshape(B * Hkv, N))
+    assert np.array_equal(gcnt, union.reshape(B * Hkv, N).sum(-1))
+    for r in range(B * Hkv):
+        assert np.all(np.diff(gidx[r, :gcnt[r]]) > 0)                        # ascending, distinct
+    umask = torch.from_numpy(np.repeat(union, G, axis=1)).reshape(B, H, 1, N)
+    krep, vrep = kk.repeat_interleave(G, dim=1), vv.repeat_interleave(G, dim=1)
+    ref = P.masked_attention(q, krep, vrep, umask)[:, :, 0]
+    tol = 1e-3 if dt == torch.float16 else 8e-3
+    assert torch.allclose(out, ref, rtol=tol, atol=tol)
+    if G == 1:
+        assert torch.allclose(out, out_plain.cpu().float(), rtol=tol, atol=tol)

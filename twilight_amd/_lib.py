@@ -14,7 +14,7 @@ from .build import LIB_PATH
 
 TWL_OK = 0
 TWL_F16, TWL_BF16, TWL_F32 = 0, 1, 2
-ABI_VERSION = 5  # TWL_ABI_VERSION of include/twilight_hip.h, checked when the library is loaded
+ABI_VERSION = 6  # TWL_ABI_VERSION of include/twilight_hip.h, checked when the library is loaded
 TWL_HIGH_FIRST, TWL_HIGH_MAX = 0, 1
 PAGE = 16
 HEAD_DIM = 128
@@ -27,7 +27,8 @@ EXPORTS = (
     "twl_strerror", "twl_abi_version", "twl_device_count", "twl_top_p_f32", "twl_top_p_f16",
     "twl_softmax_top_p_f32", "twl_gemv_top_p", "twl_select_estimate_prune", "twl_gemv_int4", "twl_gemv_int4_nhd",
     "twl_gemv_int8_nhd", "twl_gemv_f16_nhd", "twl_gemv_f16_single", "twl_sparse_attn",
-    "twl_sparse_attn_workspace_bytes", "twl_quest_select",
+    "twl_sparse_attn_workspace_bytes", "twl_group_attn", "twl_group_attn_workspace_bytes",
+    "twl_group_union", "twl_quest_select",
     "twl_quest_page_scores", "twl_quest_topk_pages", "twl_kv_shadow_build", "twl_kv_append", "twl_meta_planes_build", "twl_quest_page_scores_planes", "twl_dequant_int4",
     "twl_decode_layer", "twl_get_label_tensor", "twl_bgemv_int8", "twl_qk_int8_lse",
 )
@@ -55,6 +56,9 @@ class LayerArgs(ctypes.Structure):
         ("attn_workspace", c_void_p), ("attn_workspace_bytes", c_uint64),
         ("out", c_void_p),
         ("split_estimator", c_int), ("keep_scores", c_int),
+        ("group_idx", c_void_p), ("group_idx_stride", c_uint32),
+        ("group_count", c_void_p),
+        ("group_workspace", c_void_p), ("group_workspace_bytes", c_uint64),
     ]
 
 
@@ -99,6 +103,10 @@ def lib() -> ctypes.CDLL:
     L.twl_sparse_attn.argtypes = [vp, vp, i32, vp, vp, u64, u64, u64, vp, u32, vp, vp, vp, u32, u32,
                                   u32, f32, vp, vp, u64, vp]
     L.twl_sparse_attn_workspace_bytes.argtypes = [u32, u32]
+    L.twl_group_attn_workspace_bytes.argtypes = [u32, u32, u32, u32, i32]
+    L.twl_group_attn.argtypes = [vp, vp, i32, vp, vp, u64, u64, u64, vp, u32, vp, u32, vp, vp, vp,
+                                 u32, u32, u32, f32, vp, vp, u64, vp]
+    L.twl_group_union.argtypes = [vp, u32, vp, u32, u32, u32, u32, vp, u32, vp, vp]
     L.twl_quest_select.argtypes = [vp, i32, vp, vp, vp, u32, u32, u32, u32, u32, vp, u32, vp, vp,
                                    u32, vp]
     L.twl_quest_page_scores.argtypes = [vp, i32, vp, vp, vp, u32, u32, u32, u32, vp, u32, vp]
@@ -117,9 +125,11 @@ def lib() -> ctypes.CDLL:
     L.twl_qk_int8_lse.argtypes = [vp, vp, vp, vp, vp, u32, u32, u32, u32, u32, u32, i64, i64, i64,
                                   i64, i64, i64, vp]
     for name in EXPORTS:
-        if name not in ("twl_strerror", "twl_sparse_attn_workspace_bytes"):
+        if name not in ("twl_strerror", "twl_sparse_attn_workspace_bytes",
+                        "twl_group_attn_workspace_bytes"):
             getattr(L, name).restype = c_int
     L.twl_sparse_attn_workspace_bytes.restype = c_uint64
+    L.twl_group_attn_workspace_bytes.restype = c_uint64
     _lib = L
     return L
 

@@ -32,6 +32,7 @@ extern "C" int twl_decode_layer(const twl_layer_args* a, void* stream) {
   if (!a->sel_pages || !a->sel_count || !a->scores || !a->cand_count || !a->idx || !a->count ||
       !a->out)
     return TWL_ENULL;
+  if (a->group_idx && (!a->group_count || !a->group_workspace)) return TWL_ENULL;
   if (a->batch == 0 || a->num_q_heads == 0) return TWL_EINVAL;
   const uint32_t rows = a->batch * a->num_q_heads;
   uint32_t k = (a->token_budget / TWL_PAGE ? a->token_budget / TWL_PAGE : 1) +
@@ -125,7 +126,20 @@ extern "C" int twl_decode_layer(const twl_layer_args* a, void* stream) {
       if (rc != TWL_OK) return rc;
     }
   }
-  // 4. exact attention over the survivors
+  // 4. exact attention over the survivors: per q head, or per kv head over the group's union
+  if (a->group_idx) {
+    if (!a->group_count || !a->group_workspace) return TWL_ENULL;
+    rc = twl_group_union(a->idx, a->idx_stride, a->count, a->batch, a->num_q_heads,
+                         a->num_kv_heads, a->max_pages_per_req * TWL_PAGE, a->group_idx,
+                         a->group_idx_stride, a->group_count, stream);
+    if (rc != TWL_OK) return rc;
+    return twl_group_attn(a->q, a->out, a->dtype, a->k_cache, a->v_cache, a->page_stride,
+                          a->token_stride, a->head_stride, a->group_idx, a->group_idx_stride,
+                          a->group_count, 0, a->kv_page_indices, a->kv_page_indptr,
+                          a->kv_last_page_len, a->batch, a->num_q_heads, a->num_kv_heads,
+                          a->sm_scale, nullptr, a->group_workspace, a->group_workspace_bytes,
+                          stream);
+  }
   return twl_sparse_attn(a->q, a->out, a->dtype, a->k_cache, a->v_cache, a->page_stride,
                          a->token_stride, a->head_stride, a->idx, a->idx_stride, a->count,
                          a->kv_page_indices, a->kv_page_indptr, a->batch, a->num_q_heads,

@@ -21,6 +21,7 @@ import torch
 
 from . import _lib
 from .cache import PagedKVCache
+from .kernel.attention import group_attention_workspace_bytes, group_paged_decode_attention
 from .layer import TwilightDecodeLayer, parse_sparse_config
 
 PAGE = _lib.PAGE
@@ -158,9 +159,13 @@ class _LayerState:
     """What a patched attention module carries between calls."""
 
     def __init__(self, cfg: dict, reserve_tokens: int, budget_info: Optional[HistoryBudgetInfo],
-                 keep_hf_cache: bool, score_info: Optional[HistoryAccumulatedScoreInfo] = None):
+                 keep_hf_cache: bool, score_info: Optional[HistoryAccumulatedScoreInfo] = None,
+                 dense: bool = False):
         self.cfg, self.reserve_tokens, self.budget_info = cfg, reserve_tokens, budget_info
         self.keep_hf_cache, self.score_info = keep_hf_cache, score_info
+        self.dense = dense        # a layer the configuration leaves dense, served from paged K / V
+        self.workspace: Optional[torch.Tensor] = None
+        self.max_tokens = 0
         self.cache: Optional[PagedKVCache] = None
         self.layer: Optional[TwilightDecodeLayer] = None
         self.free: List[int] = []
@@ -168,6 +173,7 @@ class _LayerState:
 
     def reset(self) -> None:
         self.cache, self.layer, self.free, self.seq_len = None, None, [], 0
+        self.workspace = None
 
 
 def fill_from_prefill(st: _LayerState, k: torch.Tensor, v: torch.Tensor, num_q_heads: int) -> None:
@@ -182,10 +188,15 @@ def fill_from_prefill(st: _LayerState, k: torch.Tensor, v: torch.Tensor, num_q_h
     # it (with GQA it is used at the batch sizes where that launch runs, the records otherwise)
     planes = npg + spare_per_req
     st.cache = PagedKVCache.from_dense(k, v, k.device, spare_pages=B * spare_per_req,
-                                       plane_pages=planes)
+                                       plane_pages=None if st.dense else planes)
     st.free = list(range(B * npg, B * (npg + spare_per_req)))
-    st.layer = TwilightDecodeLayer(st.cache, num_q_heads, reserve_pages=npg + spare_per_req, **st.cfg)
     st.seq_len = N
+    if st.dense:
+        st.max_tokens = (npg + spare_per_req) * PAGE
+        st.workspace = torch.empty(group_attention_workspace_bytes(
+            B, num_q_heads, k.shape[1], st.max_tokens, False), dtype=torch.uint8, device=k.device)
+        return
+    st.layer = TwilightDecodeLayer(st.cache, num_q_heads, reserve_pages=npg + spare_per_req, **st.cfg)
 
 
 def _twilight_attention_forward(self, hidden_states, position_embeddings=None, attention_mask=None,
@@ -225,6 +236,13 @@ def _twilight_attention_forward(self, hidden_states, position_embeddings=None, a
         past_key_values.update(k, v, self.layer_idx)  # keeps the model's own cache consistent
     st.cache.append(k[:, :, 0], v[:, :, 0], st.free)
     st.seq_len += 1
+    if st.dense:
+        c = st.cache
+        out = group_paged_decode_attention(
+            q[:, :, 0].contiguous(), c.k_cache, c.v_cache, c.kv_page_indices, c.kv_page_indptr,
+            c.kv_last_page_len, max_tokens=st.max_tokens, sm_scale=getattr(self, "scaling", None),
+            workspace=st.workspace)
+        return self.o_proj(out.reshape(B, 1, -1)), None
     out = st.layer(q[:, :, 0].contiguous())           # [B, H, 128]
     if st.budget_info is not None:
         st.budget_info.update(self.layer_idx, st.layer.count)
@@ -238,8 +256,8 @@ def _twilight_attention_forward(self, hidden_states, position_embeddings=None, a
 
 def enable_sparse_attention(model, sparse_config: Dict, enable_budget_info: bool = False,
                             enable_score_info: bool = False, reserve_tokens: int = 4096,
-                            high: str = "max", keep_hf_cache: bool = True
-                            ) -> Tuple[Optional[HistoryBudgetInfo],
+                            high: str = "max", keep_hf_cache: bool = True,
+                            dense_layers: str = "model") -> Tuple[Optional[HistoryBudgetInfo],
                                        Optional[HistoryAccumulatedScoreInfo]]:
     """Patch every Llama / Mistral attention module of ``model`` (twilight/pyimpl/attention.py:
     351-418, 481-493). ``sparse_config`` is the reference's JSON template
@@ -248,7 +266,11 @@ def enable_sparse_attention(model, sparse_config: Dict, enable_budget_info: bool
     decode tokens to the model's own cache (a whole-context copy per step with ``DynamicCache``);
     it needs ``skip_first_two_layers`` (layer 0 keeps the sequence length the model asks its cache
     for) and a sequence that is only prefilled once. Returns ``(budget_info, score_info)`` as the
-    reference does (attention.py:404-418). ``enable_score_info`` adds a dense pass over all of K
+    reference does (attention.py:404-418). ``dense_layers``: how the layers the configuration
+    leaves dense (``skip_first_two_layers``) decode — "model": through the model's own attention
+    and cache, as in the reference; "paged": from paged K / V through the group attention kernel
+    (K / V read once per kv head). With "paged" and ``keep_hf_cache=False`` nothing updates the
+    model's cache at decode time, so the caller passes ``position_ids`` to the model itself. ``enable_score_info`` adds a dense pass over all of K
     to every patched layer's decode step (:func:`kept_attention_mass`): a diagnostic, not for
     timing runs."""
     for part in ("compressor",):
@@ -260,6 +282,8 @@ def enable_sparse_attention(model, sparse_config: Dict, enable_budget_info: bool
     cfg = parse_sparse_config(sparse_config)
     cfg["high"] = high
     skip = 2 if sparse_config.get("skip_first_two_layers", True) else 0
+    if dense_layers not in ("model", "paged"):
+        raise RuntimeError(f"dense_layers must be 'model' or 'paged', got {dense_layers!r}")
     if not keep_hf_cache and skip == 0:
         raise RuntimeError("keep_hf_cache=False needs skip_first_two_layers")
     budget_info = HistoryBudgetInfo() if enable_budget_info else None
@@ -272,10 +296,12 @@ def enable_sparse_attention(model, sparse_config: Dict, enable_budget_info: bool
             raise RuntimeError(f"{name}: head_dim must be {_lib.HEAD_DIM}")
         if hasattr(module, "_twilight_state"):
             raise RuntimeError("enable_sparse_attention was already called on this model")
-        if module.layer_idx < skip:
+        dense = module.layer_idx < skip
+        if dense and dense_layers == "model":
             continue
-        module._twilight_state = _LayerState(dict(cfg), reserve_tokens, budget_info, keep_hf_cache,
-                                              score_info)
+        module._twilight_state = _LayerState(dict(cfg), reserve_tokens,
+                                             None if dense else budget_info, keep_hf_cache,
+                                             None if dense else score_info, dense=dense)
         module._twilight_orig_forward = module.forward
         module.forward = types.MethodType(_twilight_attention_forward, module)
         patched += 1

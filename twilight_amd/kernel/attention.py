@@ -93,3 +93,125 @@ def sparse_paged_decode_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cach
             B, H, Hkv, scale, ptr(lse), ptr(workspace), workspace.numel(), stream_of(q))
     _lib.check(rc, "SparsePagedDecodeAttention")
     return (out, lse) if return_lse else out
+
+
+def group_attention_workspace_bytes(batch: int, num_q_heads: int, num_kv_heads: int,
+                                    max_tokens: int, with_list: bool) -> int:
+    """Bytes of scratch :func:`group_paged_decode_attention` needs (``max_tokens``: the longest
+    request, or the stride of the group lists)."""
+    return int(_lib.lib().twl_group_attn_workspace_bytes(batch, num_q_heads, num_kv_heads,
+                                                         max_tokens, int(with_list)))
+
+
+def group_paged_decode_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                                 kv_page_indices: torch.Tensor, kv_page_indptr: torch.Tensor,
+                                 kv_last_page_len: Optional[torch.Tensor] = None,
+                                 max_tokens: Optional[int] = None,
+                                 group_idx: Optional[torch.Tensor] = None,
+                                 group_count: Optional[torch.Tensor] = None,
+                                 sm_scale: Optional[float] = None, return_lse: bool = False,
+                                 out: Optional[torch.Tensor] = None,
+                                 workspace: Optional[torch.Tensor] = None):
+    """Softmax attention of one decode token in which the q heads of a kv head share one token
+    list, so K / V are read once per kv head (twilight/pyimpl/attention.py:188-190,299-306 over the
+    listed tokens; the reference repeats K / V per q head, attention.py:124-126).
+
+    Without ``group_idx``: dense decode over every token of each request (``kv_last_page_len``
+    int32 [B] and ``max_tokens`` >= the longest request are needed) — what the reference runs in
+    the layers its configuration leaves dense (attention.py:199-201). With ``group_idx`` int32
+    [B,Hkv,S] (ascending token positions) and ``group_count`` int32 [B,Hkv]: attention of every q
+    head over its group's list, e.g. the union from :func:`group_union_lists`. ``q`` [B,H,128]
+    fp16/bf16 with H/Hkv in {1,2,4,8}; returns ``out`` [B,H,128] (and ``lse`` fp32 [B,H])."""
+    check_input(q, "q")
+    check_dim(3, q, "q")
+    B, H, D = q.shape
+    if D != _lib.HEAD_DIM:
+        raise RuntimeError(f"head_dim must be {_lib.HEAD_DIM}, got {D}")
+    ks = _cache_strides(k_cache, "k_cache")
+    vs = _cache_strides(v_cache, "v_cache")
+    if ks != vs or k_cache.shape != v_cache.shape:
+        raise RuntimeError("k_cache and v_cache must share shape and strides")
+    if k_cache.dtype != q.dtype or v_cache.dtype != q.dtype:
+        raise RuntimeError("q, k_cache and v_cache must share one dtype (float16 or bfloat16)")
+    Hkv = k_cache.size(2)
+    if H % Hkv != 0 or H // Hkv not in (1, 2, 4, 8):
+        raise RuntimeError(f"num_q_heads {H} must be 1, 2, 4 or 8 times num_kv_heads {Hkv}")
+    others = [("k_cache", k_cache), ("v_cache", v_cache), ("kv_page_indices", kv_page_indices),
+              ("kv_page_indptr", kv_page_indptr)]
+    for name, t in others[2:]:
+        check_input(t, name); check_dtype(t, torch.int32, name)
+    if kv_page_indptr.numel() != B + 1:
+        raise RuntimeError("kv_page_indptr must have B+1 elements")
+    with_list = group_idx is not None
+    if with_list:
+        if group_count is None:
+            raise RuntimeError("group_count is needed with group_idx")
+        check_input(group_idx, "group_idx"); check_dtype(group_idx, torch.int32, "group_idx")
+        check_dim(3, group_idx, "group_idx")
+        check_input(group_count, "group_count"); check_dtype(group_count, torch.int32, "group_count")
+        if group_idx.size(0) != B or group_idx.size(1) != Hkv or group_count.numel() != B * Hkv:
+            raise RuntimeError("group_idx must be [B,Hkv,S] and group_count [B,Hkv]")
+        others += [("group_idx", group_idx), ("group_count", group_count)]
+        bound = group_idx.size(2)
+    else:
+        if kv_last_page_len is None or max_tokens is None:
+            raise RuntimeError("dense decode needs kv_last_page_len and max_tokens")
+        check_input(kv_last_page_len, "kv_last_page_len")
+        check_dtype(kv_last_page_len, torch.int32, "kv_last_page_len")
+        if kv_last_page_len.numel() != B:
+            raise RuntimeError("kv_last_page_len must have B elements")
+        others.append(("kv_last_page_len", kv_last_page_len))
+        bound = int(max_tokens)
+        if bound <= 0:
+            raise RuntimeError("max_tokens must be positive")
+    check_same_device(q, *others)
+    dev = q.device
+    with torch.cuda.device(dev):
+        if out is None:
+            out = torch.empty_like(q)
+        else:
+            check_input(out, "out")
+            if out.shape != q.shape or out.dtype != q.dtype:
+                raise RuntimeError("out must match q")
+        lse = torch.empty((B, H), dtype=torch.float32, device=dev) if return_lse else None
+        scale = 1.0 / math.sqrt(D) if sm_scale is None else float(sm_scale)
+        need = group_attention_workspace_bytes(B, H, Hkv, bound, with_list)
+        if workspace is None:
+            workspace = torch.empty(need, dtype=torch.uint8, device=dev)
+        else:
+            check_input(workspace, "workspace"); check_dtype(workspace, torch.uint8, "workspace")
+            if workspace.numel() < need or workspace.device != dev:
+                raise RuntimeError(f"workspace must hold {need} bytes on {dev}")
+        rc = _lib.lib().twl_group_attn(
+            ptr(q), ptr(out), dtype_code(q.dtype, "q"), ptr(k_cache), ptr(v_cache), ks[0], ks[1],
+            ks[2], ptr(group_idx), group_idx.size(2) if with_list else 0, ptr(group_count), bound,
+            ptr(kv_page_indices), ptr(kv_page_indptr), ptr(kv_last_page_len), B, H, Hkv, scale,
+            ptr(lse), ptr(workspace), workspace.numel(), stream_of(q))
+    _lib.check(rc, "GroupPagedDecodeAttention")
+    return (out, lse) if return_lse else out
+
+
+def group_union_lists(idx: torch.Tensor, count: torch.Tensor, num_kv_heads: int, max_tokens: int,
+                      group_stride: Optional[int] = None):
+    """Union of the survivor lists of each kv head's q heads: ``idx`` int32 [B,H,S] ascending,
+    ``count`` int32 [B,H] -> ``(group_idx int32 [B,Hkv,group_stride] ascending, group_count int32
+    [B,Hkv])``. Token positions must be < ``max_tokens`` (<= 262144). The default
+    ``group_stride`` = min(max_tokens, (H/Hkv)·S) holds every possible union."""
+    check_input(idx, "idx"); check_dtype(idx, torch.int32, "idx"); check_dim(3, idx, "idx")
+    check_input(count, "count"); check_dtype(count, torch.int32, "count")
+    B, H, S = idx.shape
+    if count.numel() != B * H:
+        raise RuntimeError("count must be [B,H]")
+    if num_kv_heads <= 0 or H % num_kv_heads != 0:
+        raise RuntimeError(f"num_q_heads {H} must be a multiple of num_kv_heads {num_kv_heads}")
+    check_same_device(idx, ("count", count))
+    if group_stride is None:
+        group_stride = min(int(max_tokens), (H // num_kv_heads) * S)
+    dev = idx.device
+    with torch.cuda.device(dev):
+        gidx = torch.empty((B, num_kv_heads, group_stride), dtype=torch.int32, device=dev)
+        gcnt = torch.empty((B, num_kv_heads), dtype=torch.int32, device=dev)
+        rc = _lib.lib().twl_group_union(ptr(idx), S, ptr(count), B, H, num_kv_heads, int(max_tokens),
+                                        ptr(gidx), group_stride, ptr(gcnt), stream_of(idx))
+    _lib.check(rc, "GroupUnionLists")
+    return gidx, gcnt

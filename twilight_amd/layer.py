@@ -46,7 +46,7 @@ class TwilightDecodeLayer:
     def __init__(self, cache: PagedKVCache, num_q_heads: int, token_budget: int = 8192,
                  top_p: float = 0.85, high: str = "max", sm_scale: Optional[float] = None,
                  fused_estimator: bool = True, keep_scores: bool = False,
-                 reserve_pages: int = 0):
+                 reserve_pages: int = 0, group_union: bool = False):
         if num_q_heads % cache.num_kv_heads != 0:
             raise RuntimeError("num_q_heads must be a multiple of the cache's kv heads")
         if not (0.0 < top_p <= 1.0):
@@ -63,6 +63,12 @@ class TwilightDecodeLayer:
         # work buffers are sized for requests of up to reserve_pages pages, so a context that grows
         # during decode does not reallocate them every time a request takes a new page
         self.reserve_pages = int(reserve_pages)
+        # group_union: the q heads of a kv head attend over the union of their survivor lists
+        # (``group_idx`` / ``group_count``) instead of each over its own; ``count`` / ``idx`` still
+        # hold the per-head results of the pruner
+        self.group_union = bool(group_union)
+        if self.group_union and num_q_heads // cache.num_kv_heads not in (1, 2, 4, 8):
+            raise RuntimeError("group_union needs 1, 2, 4 or 8 q heads per kv head")
         self._alloc()
 
     @classmethod
@@ -88,6 +94,14 @@ class TwilightDecodeLayer:
         self.out = torch.zeros((B, H, _lib.HEAD_DIM), dtype=c.dtype, device=dev)
         ws = int(_lib.lib().twl_sparse_attn_workspace_bytes(B * H, M))
         self.attn_workspace = torch.zeros(ws, dtype=torch.uint8, device=dev)
+        self.group_idx = self.group_count = self.group_workspace = None
+        if self.group_union:
+            Hkv = c.num_kv_heads
+            gs = min(cap * _lib.PAGE, (H // Hkv) * M)
+            self.group_idx = torch.zeros((B, Hkv, gs), dtype=i32, device=dev)
+            self.group_count = torch.zeros((B, Hkv), dtype=i32, device=dev)
+            gws = int(_lib.lib().twl_group_attn_workspace_bytes(B, H, Hkv, gs, 1))
+            self.group_workspace = torch.empty(gws, dtype=torch.uint8, device=dev)
         self._shape = (B, cap)
         self._args, self._args_key = None, None
 
@@ -125,6 +139,11 @@ class TwilightDecodeLayer:
         a.out = ptr(self.out)
         a.split_estimator = 0 if self.fused_estimator else 1
         a.keep_scores = 1 if self.keep_scores else 0
+        if self.group_union:
+            a.group_idx, a.group_idx_stride = ptr(self.group_idx), self.group_idx.size(2)
+            a.group_count = ptr(self.group_count)
+            a.group_workspace = ptr(self.group_workspace)
+            a.group_workspace_bytes = self.group_workspace.numel()
         return a
 
     def forward(self, q: torch.Tensor) -> torch.Tensor:
