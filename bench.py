@@ -425,6 +425,8 @@ def main() -> int:
                     help="run the INT4 GEMV and the softmax + top-p as two launches instead of one")
     ap.add_argument("--no-planes", action="store_true",
                     help="keep the Quest metadata in the 512-byte record layout only")
+    ap.add_argument("--group-union", action="store_true",
+                    help="attention over the union of each kv head's survivor lists (GQA)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel breakdown")
     args = ap.parse_args()
@@ -478,7 +480,8 @@ def main() -> int:
         if not args.no_planes:
             cache.enable_planes()      # metadata also in plane layout: the row kernel reads half
         layers.append(TwilightDecodeLayer(cache, H, token_budget=args.budget, top_p=args.top_p,
-                                          high="max", fused_estimator=not args.split_estimator))
+                                          high="max", fused_estimator=not args.split_estimator,
+                                          group_union=args.group_union))
         qs.append(q)
     torch.cuda.synchronize()
     nl = len(layers)

@@ -271,7 +271,8 @@ int twl_group_attn(const void* q, void* out, int dtype, const void* k_cache, con
                    void* workspace, uint64_t workspace_bytes, void* stream);
 /* Union of the survivor lists of each kv head's q heads (mask OR over the group; the per-head
  * lists are those of twl_top_p_* / twl_decode_layer: idx int32 [batch, num_q_heads, idx_stride],
- * count int32 [batch, num_q_heads]). Token positions must be < max_tokens (<= 262144). Output:
+ * count int32 [batch, num_q_heads]; at most 8 q heads per kv head). Token positions must be
+ * < max_tokens (<= 262144). Output:
  * group_idx int32 [batch, num_kv_heads, group_stride] ascending, group_count int32
  * [batch, num_kv_heads]; a union longer than group_stride is cut to its first group_stride
  * positions (group_stride >= min(max_tokens, G * idx_stride) never cuts). */

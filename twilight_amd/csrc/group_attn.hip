@@ -97,11 +97,13 @@ __global__ __launch_bounds__(kGrpThreads) void group_attn_partial_kernel(GroupAt
   const int gid = tx >> 4, sub = tx & 15;
   const uint32_t kvh = hblk * hb + (gid & (hb - 1));
   const int tsel = gid >> a.hb_log2;
-  const int j0 = blockIdx.x * a.chunk;
   // with a list a workgroup serves one kv head (hb == 1), without one every head has the same
   // length: n is uniform over the workgroup
   const int n = group_list_len(a, b, kvh);
-  if (j0 >= n) return;
+  // dense form: one chunk per workgroup; with lists (mostly far shorter than their stride) the
+  // grid holds a few chunks per kv head and a workgroup walks the chunks of a long list
+  for (uint32_t ch = blockIdx.x; (int)(ch * a.chunk) < n; ch += gridDim.x) {
+  const int j0 = ch * a.chunk;
   const int cn = min((int)a.chunk, n - j0);
 
   // ---- resolve the chunk's token addresses once --------------------------------------------
@@ -194,7 +196,7 @@ __global__ __launch_bounds__(kGrpThreads) void group_attn_partial_kernel(GroupAt
 
   // ---- leave the lane group's partial result -------------------------------------------------
   float* part = a.partials +
-                ((((size_t)b * a.num_kv_heads + kvh) * a.max_chunks + blockIdx.x) * ts + tsel) *
+                ((((size_t)b * a.num_kv_heads + kvh) * a.max_chunks + ch) * ts + tsel) *
                     (size_t)(G * kGrpPartial);
 #pragma unroll
   for (int g = 0; g < G; ++g) {
@@ -206,6 +208,8 @@ __global__ __launch_bounds__(kGrpThreads) void group_attn_partial_kernel(GroupAt
     f32x4* dst = (f32x4*)(pg + 4 + 8 * sub);
     dst[0] = f32x4{acc[g][0], acc[g][1], acc[g][2], acc[g][3]};
     dst[1] = f32x4{acc[g][4], acc[g][5], acc[g][6], acc[g][7]};
+  }
+  __syncthreads();   // slot_id is rewritten by the next chunk
   }
 }
 
@@ -294,7 +298,8 @@ __global__ __launch_bounds__(kMergeThreads) void group_attn_merge_kernel(GroupAt
 template <int DT>
 static int launch_group_attn(const GroupAttnArgs& a, hipStream_t stream) {
   const uint32_t G = a.num_q_heads / a.num_kv_heads;
-  dim3 grid(a.max_chunks, a.batch * (a.num_kv_heads >> a.hb_log2));
+  dim3 grid(a.idx ? (a.max_chunks < 16u ? a.max_chunks : 16u) : a.max_chunks,
+            a.batch * (a.num_kv_heads >> a.hb_log2));
   dim3 block(kGrpThreads);
   switch (G) {
     case 1: hipLaunchKernelGGL((group_attn_partial_kernel<DT, 1>), grid, block, 0, stream, a); break;
@@ -323,26 +328,32 @@ struct GroupUnionArgs {
   int32_t* group_count;    // [batch, kv heads]
 };
 
-constexpr int kUnionThreads = 256;
+constexpr int kUnionThreads = 1024;
+constexpr int kUnionWaves = kUnionThreads / kWave;
 
 __global__ __launch_bounds__(kUnionThreads) void group_union_kernel(GroupUnionArgs a) {
   extern __shared__ uint32_t bits[];   // ceil(max_tokens / 32) words
-  __shared__ int wave_tot[kUnionThreads / kWave];
+  __shared__ int wave_tot[kUnionWaves];
   __shared__ int running;
   const int tx = threadIdx.x;
   const uint32_t b = blockIdx.x / a.num_kv_heads, kvh = blockIdx.x - b * a.num_kv_heads;
   const uint32_t G = a.num_q_heads / a.num_kv_heads;
   const int words = (int)((a.max_tokens + 31) / 32);
+  const size_t row0 = (size_t)b * a.num_q_heads + kvh * G;
+  // the G lists as one run of items: item t belongs to list g with cum[g] <= t < cum[g + 1]
+  int cum[9];
+  cum[0] = 0;
+  for (uint32_t g = 0; g < 8; ++g)
+    cum[g + 1] = cum[g] + (g < G ? min(max(a.count[row0 + g], 0), (int)a.idx_stride) : 0);
   for (int w = tx; w < words; w += kUnionThreads) bits[w] = 0;
   if (tx == 0) running = 0;
   __syncthreads();
-  for (uint32_t g = 0; g < G; ++g) {
-    const size_t row = (size_t)b * a.num_q_heads + kvh * G + g;
-    const int n = min(max(a.count[row], 0), (int)a.idx_stride);
-    for (int i = tx; i < n; i += kUnionThreads) {
-      const int tok = a.idx[row * a.idx_stride + i];
-      if (tok >= 0 && (uint32_t)tok < a.max_tokens) atomicOr(&bits[tok >> 5], 1u << (tok & 31));
-    }
+  for (int t = tx; t < cum[8]; t += kUnionThreads) {
+    int g = 0;
+#pragma unroll
+    for (int x = 1; x < 8; ++x) g += (t >= cum[x]) ? 1 : 0;
+    const int tok = a.idx[(row0 + g) * a.idx_stride + (t - cum[g])];
+    if (tok >= 0 && (uint32_t)tok < a.max_tokens) atomicOr(&bits[tok >> 5], 1u << (tok & 31));
   }
   __syncthreads();
   int32_t* dst = a.group_idx + (size_t)blockIdx.x * a.group_stride;
@@ -356,7 +367,7 @@ __global__ __launch_bounds__(kUnionThreads) void group_union_kernel(GroupUnionAr
     __syncthreads();
     int before = running;
 #pragma unroll
-    for (int wv = 0; wv < kUnionThreads / kWave; ++wv) before += (wv < wave) ? wave_tot[wv] : 0;
+    for (int wv = 0; wv < kUnionWaves; ++wv) before += (wv < wave) ? wave_tot[wv] : 0;
     int pos = before + incl - c;
     while (v) {
       const int bit = __builtin_ctz(v);
@@ -436,6 +447,7 @@ extern "C" int twl_group_union(const int32_t* idx, uint32_t idx_stride, const in
   if (batch == 0 || num_q_heads == 0 || num_kv_heads == 0 || num_q_heads % num_kv_heads != 0 ||
       idx_stride == 0 || group_stride == 0)
     return TWL_EINVAL;
+  if (num_q_heads / num_kv_heads > 8) return TWL_EINVAL;
   if (max_tokens == 0 || max_tokens > 256u * 1024u) return TWL_EINVAL;   // 32 KB bitmap in LDS
   if ((uint64_t)batch * num_kv_heads > 0x7FFFFFFFull) return TWL_EINVAL;
   twl::GroupUnionArgs a{};
