@@ -311,22 +311,34 @@ def bench_llama3_model(args, dev) -> int:
                   "weight_estimator": {"type": "min_max_quant", "quant_bit": 4},
                   "weight_pruner": {"type": "top_p", "threshold": top_p},
                   "skip_first_two_layers": True, "use_estimated_weights_in_attn": False}
+    def run_graphed():
+        step = hf.GraphedDecodeStep(model)
+        for s in range(warmup):              # the first call records the step
+            step(ids[s])
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for s in range(warmup, warmup + steps):
+            logits = step(ids[s])
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / steps, logits[:, -1].float()
+
     twi = {}
-    for mode in ("model", "paged"):
+    for mode in ("model", "paged", "paged+graph"):
         # "model": the two dense layers run the model's own attention over a DynamicCache;
-        # "paged": they run twl_group_attn over paged K / V and the model's cache stays empty
+        # "paged": they run twl_group_attn over paged K / V and the model's cache stays empty;
+        # "paged+graph": the same step recorded once into a HIP graph and replayed
         info, _ = hf.enable_sparse_attention(model, sparse_cfg, enable_budget_info=True,
                                              reserve_tokens=reserve + 16, keep_hf_cache=False,
-                                             dense_layers=mode)
+                                             dense_layers="model" if mode == "model" else "paged")
         states = [getattr(model.model.layers[i].self_attn, "_twilight_state", None) for i in range(nl)]
         cache = make_cache("dynamic", [i for i in range(nl) if states[i] is None])
         for i in range(nl):
             if states[i] is not None:
                 hf.fill_from_prefill(states[i], *kv(i), cfg.num_attention_heads)
-        t, logits = run(cache, positions=True)
+        t, logits = run_graphed() if mode == "paged+graph" else run(cache, positions=True)
         twi[mode] = t * 1e3
         kept = info.get_total_avg_budget()
-        if mode == "model":
+        if mode != "paged+graph":
             hf.disable_sparse_attention(model)
             del cache, states
             torch.cuda.empty_cache()
@@ -365,7 +377,8 @@ def bench_llama3_model(args, dev) -> int:
                                f"context {N} (synthetic K/V), budget {args.budget}, p={top_p}, "
                                f"layers 0-1 dense, q_proj x{args.q_gain}"},
         "dense_layers_what": "how layers 0-1 decode: 'model' = the model's own attention (torch "
-                             "SDPA) over a DynamicCache, 'paged' = twl_group_attn over paged K/V",
+                             "SDPA) over a DynamicCache, 'paged' = twl_group_attn over paged K/V, "
+                             "'paged+graph' = that step recorded into one HIP graph and replayed",
         "dense_layers": best,
         "ms_per_step_by_dense_layers": {k: round(v, 3) for k, v in twi.items()},
         "dense": None if dense_ms is None else {

@@ -209,6 +209,11 @@ def test_one_launch_row_kernel_equals_three_launches(dev, N, lens, budget, H, Hk
     (11200, 16384, 2, 2, torch.float16),     # every page
     (40000, 4096, 2, 2, torch.float16),      # 2500 pages per request (four scoring passes)
     (32768, 8192, 2, 2, torch.float16),      # the benchmark's row shape
+    (32768 + 32, 8192, 2, 2, torch.float16),   # 2050 pages: the 2 beyond 2048 come from records
+    (32768 + 250, 8192, 4, 2, torch.bfloat16), # 2064 pages, the last one partial, GQA
+    (34816, 8192, 2, 2, torch.float16),      # 2176 pages: a tail of 128 pages from records
+    (34832, 8192, 2, 2, torch.float16),      # 2177 pages: a second plane pass, last page from its record
+    (65536 + 48, 8192, 2, 2, torch.float16), # 4099 pages: three pages beyond two plane passes
     (1600, 320, 16, 4, torch.float16),       # GQA 4:1, 32 rows: a group's rows share an XCD
     (1000, 100, 4, 2, torch.bfloat16),       # GQA 2:1, 8 rows: rows in launch order
 ])

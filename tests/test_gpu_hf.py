@@ -196,3 +196,51 @@ def test_paged_dense_layers_reproduce_dense_decode(dev):
         hf.disable_sparse_attention(model)
     with pytest.raises(RuntimeError):
         hf.enable_sparse_attention(model, cfg, dense_layers="flash")
+
+
+def test_graphed_decode_step_equals_eager_decode(dev):
+    # the whole decode step recorded once into a HIP graph and replayed: same logits as the eager
+    # patched model at every step, across page boundaries (tokens 160 and 176) and with the
+    # budget statistics still collected
+    model = _tiny_llama(layers=4, heads=4, kv_heads=2, dtype=torch.float16).to(dev)
+    ids = torch.randint(0, 97, (2, 150), generator=torch.Generator().manual_seed(11)).to(dev)
+    toks = torch.randint(0, 97, (2, 30), generator=torch.Generator().manual_seed(12)).to(dev)
+
+    def eager():
+        hf.enable_sparse_attention(model, CFG, reserve_tokens=64, dense_layers="paged",
+                                   keep_hf_cache=False)
+        logits = []
+        with torch.no_grad():
+            past = model(ids, use_cache=True).past_key_values
+            for s in range(toks.shape[1]):
+                pos = torch.full((2, 1), 150 + s, device=dev)
+                out = model(toks[:, s:s + 1], past_key_values=past, use_cache=True, position_ids=pos)
+                logits.append(out.logits[:, -1].float().clone())
+        hf.disable_sparse_attention(model)
+        return torch.stack(logits)
+
+    want = eager()
+    info, _ = hf.enable_sparse_attention(model, CFG, reserve_tokens=64, dense_layers="paged",
+                                         keep_hf_cache=False, enable_budget_info=True)
+    got = []
+    with torch.no_grad():
+        past = model(ids, use_cache=True).past_key_values
+        pos = torch.full((2, 1), 150, device=dev)     # first decode step eagerly: pages the prefill
+        out = model(toks[:, :1], past_key_values=past, use_cache=True, position_ids=pos)
+        got.append(out.logits[:, -1].float().clone())
+        step = hf.GraphedDecodeStep(model)
+        for s in range(1, toks.shape[1]):
+            got.append(step(toks[:, s:s + 1])[:, -1].float().clone())
+            torch.cuda.synchronize()                  # eager work and syncs between the replays
+    got = torch.stack(got)
+    assert torch.equal(got, want), (got - want).abs().max()
+    st = model.model.layers[3].self_attn._twilight_state
+    assert st.seq_len == 180 and st.cache._seq_lens == [180, 180]
+    assert st.cache.kv_last_page_len.cpu().tolist() == [4, 4]
+    assert len(info._budget_num) == 30 and sorted(info._budget_num[-1]) == [2, 3]
+    hf.disable_sparse_attention(model)
+    # the recording needs paged dense layers and an untouched model cache
+    hf.enable_sparse_attention(model, CFG)
+    with pytest.raises(RuntimeError):
+        hf.GraphedDecodeStep(model)
+    hf.disable_sparse_attention(model)

@@ -38,6 +38,7 @@ class PagedKVCache:
         self._seq_lens = None  # host copy, for append bookkeeping
         self._room = 0         # appends that surely fit every request's last page
         self._append_key = None
+        self._table_cap = 0    # pages per request of a fixed-address page table (0: not fixed)
         # Quest metadata in plane layout [slots, Hkv, 128, 2, cap] (see enable_planes) and the
         # slot of every request of the batch (None: slot = position in the batch)
         self.meta_planes: Optional[torch.Tensor] = None
@@ -59,6 +60,26 @@ class PagedKVCache:
         self._per_req = [ids[ipl[b]:ipl[b + 1]] for b in range(len(ipl) - 1)]
         self._last = kv_last_page_len.cpu().tolist()
         self._room = PAGE - max(self._last) if self._last else 0
+        self._append_key = None
+        self._table_cap = 0
+
+    def reserve_page_table(self, cap_pages: int) -> None:
+        """Fix the addresses of the page table for requests of up to ``cap_pages`` pages: from
+        here on ``append`` rewrites ``kv_page_indices`` / ``kv_page_indptr`` in place when a
+        request takes a new page, and ``max_pages_per_req`` stays at ``cap_pages`` (the kernels
+        take it as an upper bound; the pages a request really has come from the table). A decode
+        step whose launches were recorded into a HIP graph therefore stays valid while the
+        requests grow."""
+        if cap_pages < self.max_pages_per_req:
+            raise RuntimeError(f"cap_pages {cap_pages} is below the longest request "
+                               f"({self.max_pages_per_req} pages)")
+        if self.meta_planes is not None and cap_pages > self.meta_planes.size(4):
+            raise RuntimeError("reserve_page_table: the plane buffer is smaller than cap_pages")
+        buf = torch.zeros(self.batch * cap_pages, dtype=torch.int32, device=self.device)
+        buf[:self.kv_page_indices.numel()] = self.kv_page_indices
+        self.kv_page_indices = buf
+        self._table_cap = int(cap_pages)
+        self.max_pages_per_req = int(cap_pages)
         self._append_key = None
 
     @property
@@ -84,7 +105,9 @@ class PagedKVCache:
         if self.kv_page_indptr is None:
             raise RuntimeError("enable_planes needs a page table (set_page_table)")
         cap = max(int(cap_pages or 0), self.max_pages_per_req, 8)
-        cap = (cap + 7) // 8 * 8
+        # the library needs a multiple of 8; a multiple of 128 pages keeps every run 256-byte
+        # aligned, so that a wavefront's 256-byte load touches two cache lines, not three
+        cap = (cap + 127) // 128 * 128
         n = max(int(num_slots or 0), self.batch)
         self.meta_planes = torch.zeros((n, self.num_kv_heads, HEAD_DIM, 2, cap),
                                        dtype=self.dtype, device=self.device)
@@ -162,7 +185,15 @@ class PagedKVCache:
         """Decode append of one token per request: ``k_new`` / ``v_new`` [B, Hkv, 128]. Extends the
         page table when a request's last page is full (taking ids from ``free_pages``; host-side
         bookkeeping only, nothing is read back from the device), then one kernel writes the token
-        and updates the shadow records and the lengths."""
+        and updates the shadow records and the lengths. The two halves are also callable on their
+        own: :meth:`advance_host` every step before a recorded step is replayed,
+        :meth:`append_device` inside the recorded step."""
+        self.advance_host(free_pages)
+        self.append_device(k_new, v_new)
+
+    def advance_host(self, free_pages: Optional[list] = None) -> None:
+        """Host half of :meth:`append`: make room for one more token per request (a new page from
+        ``free_pages`` where the last one is full) and count the token."""
         B = self.batch
         per_req, last = self._per_req, self._last
         grew = False
@@ -180,14 +211,30 @@ class PagedKVCache:
             ptr = [0]
             for r in per_req:
                 ptr.append(ptr[-1] + len(r))
-            self.kv_page_indices = torch.tensor(flat, dtype=torch.int32, device=self.device)
-            self.kv_page_indptr = torch.tensor(ptr, dtype=torch.int32, device=self.device)
-            self.max_pages_per_req = max(len(r) for r in per_req)
+            if self._table_cap:
+                if max(len(r) for r in per_req) > self._table_cap:
+                    raise RuntimeError("PagedKVCache.append: request outgrew reserve_page_table")
+                self.kv_page_indices[:len(flat)].copy_(torch.tensor(flat, dtype=torch.int32))
+                self.kv_page_indptr.copy_(torch.tensor(ptr, dtype=torch.int32))
+            else:
+                self.kv_page_indices = torch.tensor(flat, dtype=torch.int32, device=self.device)
+                self.kv_page_indptr = torch.tensor(ptr, dtype=torch.int32, device=self.device)
+                self.max_pages_per_req = max(len(r) for r in per_req)
             if self.meta_planes is not None and self.max_pages_per_req > self.meta_planes.size(4):
                 raise RuntimeError("PagedKVCache.append: request outgrew the plane buffer "
                                    "(enable_planes with a larger cap_pages)")
             # same tensor object every step, so cached argument blocks of the layer stay valid
             self.kv_last_page_len.copy_(torch.tensor(last, dtype=torch.int32))
+        self._room -= 1
+        for b in range(B):
+            last[b] += 1
+            self._seq_lens[b] += 1
+
+    def append_device(self, k_new: torch.Tensor, v_new: torch.Tensor) -> None:
+        """Device half of :meth:`append`: one launch writes the token of every request at the
+        position the device-side lengths give (and adds one to them), its INT4 codes and the
+        min/max fold. :meth:`advance_host` must have made room for it."""
+        B = self.batch
         if k_new.device != self.device or k_new.dtype != self.dtype:
             k_new = k_new.to(self.device, self.dtype)
         if v_new.device != self.device or v_new.dtype != self.dtype:
@@ -223,7 +270,3 @@ class PagedKVCache:
                     0 if planes is None else planes.size(0),
                     torch.cuda.current_stream(self.device).cuda_stream)
             _lib.check(rc, "KvAppend")
-        self._room -= 1
-        for b in range(B):
-            last[b] += 1
-            self._seq_lens[b] += 1

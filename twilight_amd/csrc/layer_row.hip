@@ -103,21 +103,23 @@ __global__ __launch_bounds__(kRowThreads) void select_estimate_prune_kernel(RowA
     const uint16_t* pl =
         a.planes + ((size_t)slot * a.f.num_kv_heads + kvh) * (TWL_HEAD_DIM * 2) * a.plane_cap;
     constexpr int PL_PASSES = (SEL_VPT + 1) / 2;  // 16 waves x 128 pages = 2048 pages per pass
-    // The request's last page is scored from its metadata record: the appending side keeps the
-    // record current token by token and writes the plane entries once, when the page is full.
-    const int last_pg = n_score - 1;
-    float s_last = 0.0f;
-    if (wave == 0 && n_score > 0) {  // requested now, folded while the other pages stream
-      const uint32_t qw2 = *(const uint32_t*)(qrow + 2 * lane);
-      const int phys = a.f.kv_page_indices[pg_begin + last_pg];
-      s_last = record_page_score<QDT>(
-          a.meta + ((size_t)phys * a.f.num_kv_heads + kvh) * TWL_META_RECORD_BYTES,
-          bits16_to_f32<QDT>(qw2 & 0xFFFFu), bits16_to_f32<QDT>(qw2 >> 16));
-    }
+    // The request's last pages are scored from their metadata records (plane_scored_pages): the
+    // appending side keeps the record of the last page current token by token and writes its
+    // plane entries once, when the page is full.
+    const int np = plane_scored_pages(n_score);
+    // tail pages np + wave, np + wave + 16, ... of this wavefront (at most 8): their records are
+    // requested now and folded after the plane passes
+    const int tail = n_score - np - wave;              // wave-uniform
+    const int tail_cnt = tail > 0 ? min((tail + kRowWaves - 1) / kRowWaves, 8) : 0;
+    RecordBatch8 rb;
+    if (tail_cnt > 0)
+      record_pages_load8(rb, a.meta + (size_t)kvh * TWL_META_RECORD_BYTES,
+                         (size_t)a.f.num_kv_heads * TWL_META_RECORD_BYTES,
+                         a.f.kv_page_indices + pg_begin, np + wave, kRowWaves, tail_cnt);
 #pragma unroll
     for (int pass = 0; pass < PL_PASSES; ++pass) {
       const int w0 = (pass * kRowWaves + wave) * 128;  // first page of this wave's slice
-      if (w0 < n_score) {                                // wave-uniform
+      if (w0 < np) {                                     // wave-uniform
         const int pg0 = w0 + 2 * lane;                 // this lane's two pages
         const int pgc = min(pg0, (int)a.plane_cap - 2);  // loads stay inside the run
         float s0 = 0.0f, s1 = 0.0f;
@@ -131,18 +133,29 @@ __global__ __launch_bounds__(kRowThreads) void select_estimate_prune_kernel(RowA
           s0 = fmaf(qd, bits16_to_f32<QDT>(w & 0xFFFFu), s0);
           s1 = fmaf(qd, bits16_to_f32<QDT>(w >> 16), s1);
         }
-        if (pg0 < last_pg) ps_lds[pg0] = s0;
-        if (pg0 + 1 < last_pg) ps_lds[pg0 + 1] = s1;
+        if (pg0 < np) ps_lds[pg0] = s0;
+        if (pg0 + 1 < np) ps_lds[pg0 + 1] = s1;
         if (a.page_scores_out) {
           float* po = a.page_scores_out + (size_t)row * a.page_score_stride;
-          if (pg0 < last_pg) po[pg0] = s0;
-          if (pg0 + 1 < last_pg) po[pg0 + 1] = s1;
+          if (pg0 < np) po[pg0] = s0;
+          if (pg0 + 1 < np) po[pg0 + 1] = s1;
         }
       }
     }
-    if (wave == 0 && lane == 0 && n_score > 0) {
-      ps_lds[last_pg] = s_last;
-      if (a.page_scores_out) a.page_scores_out[(size_t)row * a.page_score_stride + last_pg] = s_last;
+    if (tail_cnt > 0) {
+      const uint32_t qw2 = *(const uint32_t*)(qrow + 2 * lane);
+      float sc[8];
+      record_pages_fold8<QDT>(rb, bits16_to_f32<QDT>(qw2 & 0xFFFFu), bits16_to_f32<QDT>(qw2 >> 16), sc);
+      if (lane == 0) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          if (i < tail_cnt) {
+            const int pg = np + wave + i * kRowWaves;
+            ps_lds[pg] = sc[i];
+            if (a.page_scores_out) a.page_scores_out[(size_t)row * a.page_score_stride + pg] = sc[i];
+          }
+        }
+      }
     }
   } else {
     // page ids of all passes first: register r, lane l <-> pass 2r + l/32, page l%32 of the wave's
@@ -303,14 +316,17 @@ extern "C" int twl_select_estimate_prune(
   a.plane_slots = plane_slots; a.plane_num_slots = plane_num_slots;
   const uint32_t rows = batch * num_q_heads;
   hipStream_t s = (hipStream_t)stream;
-  const bool small = max_pages_per_req <= 2048;
+  // page scores per thread of the selection: 2 up to 2048 pages (32k tokens), 4 up to 4096, else 8
+  const int vpt = max_pages_per_req <= 2048 ? 2 : (max_pages_per_req <= 4096 ? 4 : 8);
 #define TWL_ROW_LAUNCH(DT)                                              \
   do {                                                                  \
     if (meta_planes) {                                                  \
-      if (small) twl::launch_row<DT, 2, true>(a, rows, s);              \
+      if (vpt == 2) twl::launch_row<DT, 2, true>(a, rows, s);           \
+      else if (vpt == 4) twl::launch_row<DT, 4, true>(a, rows, s);      \
       else twl::launch_row<DT, 8, true>(a, rows, s);                    \
     } else {                                                            \
-      if (small) twl::launch_row<DT, 2, false>(a, rows, s);             \
+      if (vpt == 2) twl::launch_row<DT, 2, false>(a, rows, s);          \
+      else if (vpt == 4) twl::launch_row<DT, 4, false>(a, rows, s);     \
       else twl::launch_row<DT, 8, false>(a, rows, s);                   \
     }                                                                   \
   } while (0)

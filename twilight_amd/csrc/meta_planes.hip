@@ -124,8 +124,35 @@ __global__ __launch_bounds__(kPsThreads) void quest_score_planes_kernel(PlaneSco
   const int n_req = min(max(a.kv_page_indptr[b + 1] - a.kv_page_indptr[b], 0),
                         min((int)a.max_pages, (int)a.cap));
   const int w0 = blockIdx.x * kPsPagesPerBlock + wave * 128;
-  if (w0 >= n_req) return;
   const uint16_t* qrow = (const uint16_t*)a.q + (size_t)row * TWL_HEAD_DIM;
+  float* po = a.page_scores + (size_t)row * a.score_stride;
+  // pages from np on are scored from their records (plane_scored_pages), by the wavefronts of the
+  // workgroup whose slice begins at np (np is a multiple of that slice whenever more than the
+  // last page is left) or by the wavefront that owns the last page
+  const int np = plane_scored_pages(n_req);
+  if (n_req - np > 1) {
+    if ((int)(blockIdx.x * kPsPagesPerBlock) == np) {   // workgroup-uniform
+      constexpr int kWaves = kPsThreads / kWave;
+      const uint32_t qw2 = *(const uint32_t*)(qrow + 2 * lane);
+      const float q0 = bits16_to_f32<DT>(qw2 & 0xFFFFu), q1 = bits16_to_f32<DT>(qw2 >> 16);
+      for (int first = np + wave; first < n_req; first += 8 * kWaves) {
+        const int cnt = min((n_req - first + kWaves - 1) / kWaves, 8);
+        RecordBatch8 rb;
+        record_pages_load8(rb, a.meta + (size_t)kvh * TWL_META_RECORD_BYTES,
+                           (size_t)a.num_kv_heads * TWL_META_RECORD_BYTES,
+                           a.kv_page_indices + a.kv_page_indptr[b], first, kWaves, cnt);
+        float sc[8];
+        record_pages_fold8<DT>(rb, q0, q1, sc);
+        if (lane == 0) {
+#pragma unroll
+          for (int i = 0; i < 8; ++i)
+            if (i < cnt) po[first + i * kWaves] = sc[i];
+        }
+      }
+      return;
+    }
+  }
+  if (w0 >= n_req || (n_req - np > 1 && w0 >= np)) return;
   const float q_lo = bits16_to_f32<DT>(qrow[lane]);
   const float q_hi = bits16_to_f32<DT>(qrow[64 + lane]);
   const uint32_t slot = plane_slot(a.slots, a.num_slots, b);
@@ -143,11 +170,10 @@ __global__ __launch_bounds__(kPsThreads) void quest_score_planes_kernel(PlaneSco
     s0 = fmaf(qd, bits16_to_f32<DT>(w & 0xFFFFu), s0);
     s1 = fmaf(qd, bits16_to_f32<DT>(w >> 16), s1);
   }
-  float* po = a.page_scores + (size_t)row * a.score_stride;
   const int last_pg = n_req - 1;  // scored from its record, by the wavefront that owns it
-  if (pg0 < last_pg) po[pg0] = s0;
-  if (pg0 + 1 < last_pg) po[pg0 + 1] = s1;
-  if (last_pg >= w0 && last_pg < w0 + 128) {  // wave-uniform
+  if (pg0 < np) po[pg0] = s0;
+  if (pg0 + 1 < np) po[pg0 + 1] = s1;
+  if (np == last_pg && last_pg >= w0 && last_pg < w0 + 128) {  // wave-uniform
     const uint32_t qw2 = *(const uint32_t*)(qrow + 2 * lane);
     const int phys = a.kv_page_indices[a.kv_page_indptr[b] + last_pg];
     const float s_last = record_page_score<DT>(

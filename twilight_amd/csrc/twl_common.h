@@ -156,6 +156,50 @@ __device__ __forceinline__ float record_page_score(const uint8_t* rec, float q0,
   return wave_allreduce<OpSum>(fmaf(q1, v1, q0 * v0));
 }
 
+// Up to 8 pages at once, same arithmetic per page, in two steps so that a caller can put other
+// work between the loads and the folds: page i of the batch is logical page first + i * step of
+// the table `pages` (i < count <= 8; the other slots repeat page 0 of the batch). rec0 points at
+// the kv head's record of physical page 0, `stride` = bytes from one physical page's record to
+// the next one's.
+struct RecordBatch8 {
+  uint32_t mn[8], mx[8];
+};
+__device__ __forceinline__ void record_pages_load8(RecordBatch8& r, const uint8_t* rec0,
+                                                   size_t stride, const int32_t* pages, int first,
+                                                   int step, int count) {
+  const int lane = lane_id();
+  const int c = lane >> 1, o = (lane & 1) * 4;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int phys = pages[first + (i < count ? i : 0) * step];
+    const uint8_t* rec = rec0 + (size_t)phys * stride;
+    r.mn[i] = *(const uint32_t*)(rec + 16 * c + o);
+    r.mx[i] = *(const uint32_t*)(rec + 16 * c + 8 + o);
+  }
+}
+template <int DT>
+__device__ __forceinline__ void record_pages_fold8(const RecordBatch8& r, float q0, float q1,
+                                                   float* out) {
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const float v0 = bits16_to_f32<DT>((q0 > 0.0f ? r.mx[i] : r.mn[i]) & 0xFFFFu);
+    const float v1 = bits16_to_f32<DT>((q1 > 0.0f ? r.mx[i] : r.mn[i]) >> 16);
+    out[i] = wave_allreduce<OpSum>(fmaf(q1, v1, q0 * v0));
+  }
+}
+
+// The plane-layout scoring passes read a request's first plane_scored_pages(n) pages from the
+// planes and the rest from the metadata records: always the last page (its plane entries are only
+// written when it is complete), and a whole tail of up to kPlaneTailMax pages beyond the last
+// multiple of kPlaneBlock, so that a request a little longer than a multiple of what one pass of
+// a workgroup covers does not pay a whole pass for a handful of pages.
+constexpr int kPlaneBlock = 2048, kPlaneTailMax = 128;
+__host__ __device__ __forceinline__ int plane_scored_pages(int n) {
+  if (n <= 0) return 0;
+  const int full = ((n - 1) / kPlaneBlock) * kPlaneBlock;
+  return (n - full <= kPlaneTailMax) ? full : n - 1;
+}
+
 // Slot of a request's plane-layout metadata: the request's position in the batch, or, with a slot
 // table, the entry of that position (clamped, so that a corrupt table cannot leave the buffer).
 __device__ __forceinline__ uint32_t plane_slot(const int32_t* slots, uint32_t num_slots, uint32_t b) {

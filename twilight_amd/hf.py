@@ -164,6 +164,7 @@ class _LayerState:
         self.cfg, self.reserve_tokens, self.budget_info = cfg, reserve_tokens, budget_info
         self.keep_hf_cache, self.score_info = keep_hf_cache, score_info
         self.dense = dense        # a layer the configuration leaves dense, served from paged K / V
+        self.recorded = False     # the decode step is recorded / replayed by GraphedDecodeStep
         self.workspace: Optional[torch.Tensor] = None
         self.max_tokens = 0
         self.cache: Optional[PagedKVCache] = None
@@ -234,8 +235,11 @@ def _twilight_attention_forward(self, hidden_states, position_embeddings=None, a
     q, k = apply_rotary_pos_emb(q, k, cos, sin)
     if st.keep_hf_cache:
         past_key_values.update(k, v, self.layer_idx)  # keeps the model's own cache consistent
-    st.cache.append(k[:, :, 0], v[:, :, 0], st.free)
-    st.seq_len += 1
+    if st.recorded:   # GraphedDecodeStep has done the host half for this step
+        st.cache.append_device(k[:, :, 0], v[:, :, 0])
+    else:
+        st.cache.append(k[:, :, 0], v[:, :, 0], st.free)
+        st.seq_len += 1
     if st.dense:
         c = st.cache
         out = group_paged_decode_attention(
@@ -244,10 +248,10 @@ def _twilight_attention_forward(self, hidden_states, position_embeddings=None, a
             workspace=st.workspace)
         return self.o_proj(out.reshape(B, 1, -1)), None
     out = st.layer(q[:, :, 0].contiguous())           # [B, H, 128]
-    if st.budget_info is not None:
+    if st.budget_info is not None and not st.recorded:
         st.budget_info.update(self.layer_idx, st.layer.count)
         st.budget_info.update_B0(self.layer_idx, min(st.layer.token_budget, st.seq_len))
-    if st.score_info is not None:
+    if st.score_info is not None and not st.recorded:
         st.score_info.update(self.layer_idx, kept_attention_mass(
             st.cache, q[:, :, 0], st.layer.idx, st.layer.count, st.layer.sm_scale))
     attn_output = self.o_proj(out.reshape(B, 1, -1))
@@ -308,6 +312,87 @@ def enable_sparse_attention(model, sparse_config: Dict, enable_budget_info: bool
     if patched == 0:
         raise RuntimeError("no attention module was patched")
     return budget_info, score_info
+
+
+class GraphedDecodeStep:
+    """Decode steps of a patched model replayed from ONE recorded HIP graph.
+
+    The model's eager decode step issues about a thousand small launches; at the speeds of this
+    path the host cannot keep up with the GPU. Here the step is recorded once
+    (``torch.cuda.graph``: the model's own kernels and the library's launches alike, all on the
+    capture stream) and replayed; per step the host only advances the page tables
+    (:meth:`PagedKVCache.advance_host`), writes the token ids and positions into fixed buffers and
+    launches the graph. Page tables have fixed addresses (:meth:`PagedKVCache.reserve_page_table`),
+    so the recording stays valid while the requests grow, up to ``reserve_tokens`` more tokens.
+
+    Needs ``enable_sparse_attention(..., dense_layers="paged", keep_hf_cache=False)`` (nothing may
+    touch the model's own cache inside the recording) and that every patched layer holds its paged
+    K / V: run the first decode step after a prefill eagerly, or call :func:`fill_from_prefill`.
+    Budget statistics are updated after every replay; the accumulated-score diagnostic is not
+    available."""
+
+    def __init__(self, model):
+        self.model = model
+        self.states: List[Tuple[int, _LayerState]] = []
+        for _, module in model.named_modules():
+            if all(hasattr(module, a) for a in ("q_proj", "k_proj", "v_proj", "o_proj", "layer_idx")):
+                st = getattr(module, "_twilight_state", None)
+                if st is None:
+                    raise RuntimeError("GraphedDecodeStep needs dense_layers='paged': attention "
+                                       f"layer {module.layer_idx} is not patched")
+                if st.keep_hf_cache:
+                    raise RuntimeError("GraphedDecodeStep needs keep_hf_cache=False")
+                if st.score_info is not None:
+                    raise RuntimeError("GraphedDecodeStep cannot record the score diagnostic")
+                self.states.append((module.layer_idx, st))
+        if not self.states:
+            raise RuntimeError("no patched attention module")
+        self.states.sort(key=lambda t: t[0])
+        self.graph: Optional[torch.cuda.CUDAGraph] = None
+        self.ids = self.pos = self.logits = self.past = None
+
+    def _prepare(self, input_ids: torch.Tensor) -> None:
+        from transformers import DynamicCache
+        for lid, st in self.states:
+            if st.cache is None:
+                raise RuntimeError(f"layer {lid} has no paged K / V yet: run the first decode step "
+                                   "after a prefill eagerly")
+            cap = (st.max_tokens // PAGE) if st.dense else st.layer.reserve_pages
+            st.cache.reserve_page_table(max(cap, st.cache.max_pages_per_req))
+        self.ids = input_ids.clone()
+        self.pos = torch.zeros_like(self.ids)
+        self.past = DynamicCache(config=self.model.config)   # stays empty: nothing updates it
+
+    def __call__(self, input_ids: torch.Tensor) -> torch.Tensor:
+        """``input_ids`` [B, 1] -> logits [B, 1, vocab] (the same buffer every call)."""
+        if self.ids is None:
+            self._prepare(input_ids)
+        seq = self.states[0][1].seq_len
+        if any(st.seq_len != seq for _, st in self.states):
+            raise RuntimeError("the patched layers disagree on the sequence length")
+        for _, st in self.states:
+            st.cache.advance_host(st.free)
+            st.seq_len += 1
+            st.recorded = True
+        try:
+            self.ids.copy_(input_ids)
+            self.pos.fill_(seq)
+            if self.graph is None:
+                graph = torch.cuda.CUDAGraph()
+                with torch.no_grad(), torch.cuda.graph(graph):
+                    out = self.model(self.ids, past_key_values=self.past, use_cache=True,
+                                     position_ids=self.pos)
+                self.graph, self.logits = graph, out.logits
+            # recording does not execute: the step itself is the replay, the first time too
+            self.graph.replay()
+        finally:
+            for _, st in self.states:
+                st.recorded = False
+        for lid, st in self.states:
+            if st.budget_info is not None and not st.dense:
+                st.budget_info.update(lid, st.layer.count)
+                st.budget_info.update_B0(lid, min(st.layer.token_budget, st.seq_len))
+        return self.logits
 
 
 def disable_sparse_attention(model) -> None:
