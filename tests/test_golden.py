@@ -1,0 +1,109 @@
+"""The known-answer vectors of tests/golden/known_answers.json (written by
+tests/golden/make_fixtures.py from the closed forms the reference states, without running the
+reference or the oracle) against the oracle on the CPU and against the HIP path through the C ABI."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import native
+from oracle import pyimpl_port as P
+
+with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "known_answers.json")) as f:
+    KA = json.load(f)
+
+
+def test_fixture_file_is_what_the_generator_writes():
+    import importlib.util
+    spec = importlib.util.spec_from_file_location(
+        "make_fixtures", os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "make_fixtures.py"))
+    m = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(m)
+    assert m.int4_quant() == KA["int4_quant"] and m.top_p_figure() == KA["top_p_figure"]
+    assert m.top_p_trace() == KA["top_p_trace"] and m.gemv_constant() == KA["gemv_constant"]
+
+
+def test_oracle_quantiser_on_the_reference_vector():
+    k = KA["int4_quant"]
+    out = P.min_max_quant_ref(torch.tensor(k["x"]), 4)                      # quantize.py:4-13
+    np.testing.assert_allclose(out.numpy(), np.array(k["dequant"], np.float32), rtol=0, atol=3e-6)
+    codes, scale, zero = native.int4_quant(np.array(k["x"], np.float32)[None], group=15)
+    assert codes[0].tolist() == k["codes"]
+    assert scale[0, 0] == np.float16(k["scale"]) and zero[0, 0] == np.float16(k["min"])
+
+
+def test_oracle_top_p_on_the_figure_and_the_hand_trace():
+    fig = KA["top_p_figure"]
+    w = np.array([fig["weights"]], np.float32)
+    for mode in (native.HIGH_FIRST, native.HIGH_MAX):
+        mask, _, _ = native.top_p_mask_f32(w, fig["p"], mode)
+        assert np.nonzero(mask[0])[0].tolist() == fig["keep"]
+    tr = KA["top_p_trace"]
+    mask, low, iters = native.top_p_mask_f32(np.array([tr["probs"]], np.float32), tr["p"], native.HIGH_FIRST)
+    assert mask[0].tolist() == tr["mask"] and iters[0] == tr["iterations"] and low[0] == np.float32(tr["low"])
+
+
+def test_oracle_estimator_on_the_constant_inputs():
+    c = KA["gemv_constant"]
+    deq = native.int4_dequant(np.full((1, c["head_dim"]), c["nibble"], np.uint8),
+                              np.full((1, 4), c["scale"], np.float16), np.full((1, 4), c["zero"], np.float16))
+    q = torch.full((1, 1, 1, c["head_dim"]), c["q"])
+    assert float(P.estimator_scores(q, torch.from_numpy(deq)[None, None], sm_scale=1.0)) == c["raw_score"]
+
+
+@pytest.mark.gpu
+def test_hip_top_p_on_the_figure_and_the_hand_trace(dev):
+    import twilight_amd.kernel as K
+    fig = KA["top_p_figure"]
+    w = torch.tensor(fig["weights"], dtype=torch.float32, device=dev).reshape(1, 1, 1, -1)
+    mask = K.top_p_fp32_return_mask(w, fig["p"])
+    assert torch.nonzero(mask[0, 0, 0]).flatten().tolist() == fig["keep"]
+    idx, count = K.top_p_select(w, fig["p"])
+    assert idx[0, 0, :int(count[0, 0])].tolist() == fig["keep"]
+    tr = KA["top_p_trace"]                                  # token 0 is the maximum: both bounds agree
+    pr = torch.tensor(tr["probs"], dtype=torch.float32, device=dev).reshape(1, 1, 1, -1)
+    assert K.top_p_fp32_return_mask(pr, tr["p"])[0, 0, 0].int().tolist() == tr["mask"]
+
+
+@pytest.mark.gpu
+def test_hip_quantiser_on_the_reference_vector(dev):
+    import twilight_amd.kernel as K
+    k = KA["int4_quant"]
+    # one page, one kv head; token 0's first quantisation group holds the vector twice and its
+    # first two values once more (same minimum and maximum), everything else is zero
+    x = torch.tensor(k["x"] + k["x"] + k["x"][:2], dtype=torch.float16)
+    page = torch.zeros((1, 16, 1, 128), dtype=torch.float16)
+    page[0, 0, 0, :32] = x
+    page = page.to(dev)
+    rec = torch.zeros((1, 1, 1280), dtype=torch.uint8, device=dev)
+    K.kv_shadow_build(page, rec, None)
+    nib = rec[0, 0, :16].cpu().numpy()                      # token 0, elements 0..31
+    codes = np.stack([nib & 15, nib >> 4], axis=-1).reshape(-1)
+    assert codes[:15].tolist() == k["codes"] and codes[15:30].tolist() == k["codes"]
+    sz = rec[0, 0, 1024:1028].cpu().numpy().view(np.float16)
+    assert sz[0] == np.float16(k["scale"]) and sz[1] == np.float16(k["min"])
+    deq = K.dequant_int4(rec)[0, 0, 0, :15].cpu().numpy()
+    # storage form: fp16 scale and zero, one fp32 rounding of code * scale + zero
+    want = np.array(k["codes"], np.float32) * np.float32(sz[0]) + np.float32(sz[1])
+    assert np.array_equal(deq, want)
+    np.testing.assert_allclose(deq, np.array(k["dequant"], np.float32), atol=0.5 * 2 ** -9 * 16)
+
+
+@pytest.mark.gpu
+def test_hip_estimator_on_the_constant_inputs(dev):
+    import twilight_amd.kernel as K
+    from twilight_amd import synth
+    c = KA["gemv_constant"]
+    H, pages = 2, 3
+    rec = np.zeros((pages, H, 1280), np.uint8)
+    rec[:, :, :1024] = c["nibble"] | (c["nibble"] << 4)
+    sz = np.tile(np.array([c["scale"], c["zero"]], np.float16), 64)
+    rec[:, :, 1024:] = sz.view(np.uint8)
+    ids, indptr, last = synth.identity_page_table(1, pages, 16, dev)
+    q = torch.full((1, H, 128), c["q"], dtype=torch.float16, device=dev)
+    scores, cnt = K.sparse_gemv_int4(q, torch.from_numpy(rec).to(dev), ids, indptr, last,
+                                     max_pages=pages, sm_scale=1.0)
+    assert int(cnt.min()) == pages * 16
+    assert torch.all(scores[:, :, :pages * 16] == c["raw_score"])
