@@ -511,6 +511,22 @@ def main() -> int:
     for i in range(nl):                      # leave every layer's buffers as a whole step does
         layers[i].forward(qs[i])
     torch.cuda.synchronize()
+    # the same steps recorded once into a HIP graph (one step of each rotated layer) and replayed,
+    # as a serving loop that records its decode step would run them (reported beside `value`)
+    graph_us = None
+    if args.steps >= nl:
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for i in range(nl):
+                layers[i].forward(qs[i])
+        reps = max(args.steps // nl, 1)
+        g.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            g.replay()
+        torch.cuda.synchronize()
+        graph_us = (time.perf_counter() - t0) * 1e6 / (reps * nl)
     counts = torch.stack([l.count for l in layers]).float()
     n_bar = float(counts.mean())
     n_max = int(counts.max())
@@ -735,6 +751,7 @@ def main() -> int:
                    "batch": B, "context": N, "budget": args.budget, "top_p": args.top_p,
                    "layers_rotated": nl, "survivors_mean": round(n_bar, 1),
                    "survivors_max": n_max},
+        "us_per_step_graph_replay": None if graph_us is None else round(graph_us, 2),
         "layer_bytes": layer_bytes,
         "layer_frac_of_hbm_peak": (round(layer_bytes / wall_us / 1e3 / HBM_PEAK_GBS, 4)
                                    if layer_bytes else None),

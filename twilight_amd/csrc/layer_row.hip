@@ -145,7 +145,7 @@ __global__ __launch_bounds__(kRowThreads) void select_estimate_prune_kernel(RowA
     if (tail_cnt > 0) {
       const uint32_t qw2 = *(const uint32_t*)(qrow + 2 * lane);
       float sc[8];
-      record_pages_fold8<QDT>(rb, bits16_to_f32<QDT>(qw2 & 0xFFFFu), bits16_to_f32<QDT>(qw2 >> 16), sc);
+      record_pages_fold8<QDT>(rb, tail_cnt, bits16_to_f32<QDT>(qw2 & 0xFFFFu), bits16_to_f32<QDT>(qw2 >> 16), sc);
       if (lane == 0) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) {

@@ -142,7 +142,7 @@ __global__ __launch_bounds__(kPsThreads) void quest_score_planes_kernel(PlaneSco
                            (size_t)a.num_kv_heads * TWL_META_RECORD_BYTES,
                            a.kv_page_indices + a.kv_page_indptr[b], first, kWaves, cnt);
         float sc[8];
-        record_pages_fold8<DT>(rb, q0, q1, sc);
+        record_pages_fold8<DT>(rb, cnt, q0, q1, sc);
         if (lane == 0) {
 #pragma unroll
           for (int i = 0; i < 8; ++i)

@@ -158,7 +158,7 @@ __device__ __forceinline__ float record_page_score(const uint8_t* rec, float q0,
 
 // Up to 8 pages at once, same arithmetic per page, in two steps so that a caller can put other
 // work between the loads and the folds: page i of the batch is logical page first + i * step of
-// the table `pages` (i < count <= 8; the other slots repeat page 0 of the batch). rec0 points at
+// the table `pages` (i < count <= 8; the other slots stay untouched). rec0 points at
 // the kv head's record of physical page 0, `stride` = bytes from one physical page's record to
 // the next one's.
 struct RecordBatch8 {
@@ -171,20 +171,24 @@ __device__ __forceinline__ void record_pages_load8(RecordBatch8& r, const uint8_
   const int c = lane >> 1, o = (lane & 1) * 4;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    const int phys = pages[first + (i < count ? i : 0) * step];
-    const uint8_t* rec = rec0 + (size_t)phys * stride;
-    r.mn[i] = *(const uint32_t*)(rec + 16 * c + o);
-    r.mx[i] = *(const uint32_t*)(rec + 16 * c + 8 + o);
+    if (i < count) {   // wave-uniform
+      const int phys = pages[first + i * step];
+      const uint8_t* rec = rec0 + (size_t)phys * stride;
+      r.mn[i] = *(const uint32_t*)(rec + 16 * c + o);
+      r.mx[i] = *(const uint32_t*)(rec + 16 * c + 8 + o);
+    }
   }
 }
 template <int DT>
-__device__ __forceinline__ void record_pages_fold8(const RecordBatch8& r, float q0, float q1,
-                                                   float* out) {
+__device__ __forceinline__ void record_pages_fold8(const RecordBatch8& r, int count, float q0,
+                                                   float q1, float* out) {
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    const float v0 = bits16_to_f32<DT>((q0 > 0.0f ? r.mx[i] : r.mn[i]) & 0xFFFFu);
-    const float v1 = bits16_to_f32<DT>((q1 > 0.0f ? r.mx[i] : r.mn[i]) >> 16);
-    out[i] = wave_allreduce<OpSum>(fmaf(q1, v1, q0 * v0));
+    if (i < count) {   // wave-uniform
+      const float v0 = bits16_to_f32<DT>((q0 > 0.0f ? r.mx[i] : r.mn[i]) & 0xFFFFu);
+      const float v1 = bits16_to_f32<DT>((q1 > 0.0f ? r.mx[i] : r.mn[i]) >> 16);
+      out[i] = wave_allreduce<OpSum>(fmaf(q1, v1, q0 * v0));
+    }
   }
 }
 
