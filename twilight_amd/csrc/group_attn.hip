@@ -103,113 +103,113 @@ __global__ __launch_bounds__(kGrpThreads) void group_attn_partial_kernel(GroupAt
   // dense form: one chunk per workgroup; with lists (mostly far shorter than their stride) the
   // grid holds a few chunks per kv head and a workgroup walks the chunks of a long list
   for (uint32_t ch = blockIdx.x; (int)(ch * a.chunk) < n; ch += gridDim.x) {
-  const int j0 = ch * a.chunk;
-  const int cn = min((int)a.chunk, n - j0);
+    const int j0 = ch * a.chunk;
+    const int cn = min((int)a.chunk, n - j0);
 
-  // ---- resolve the chunk's token addresses once --------------------------------------------
-  const int pbase = a.kv_page_indptr[b];
-  for (int i = tx; i < cn; i += kGrpThreads) {
-    const int tok = a.idx ? a.idx[((size_t)b * a.num_kv_heads + kvh) * a.idx_stride + j0 + i] : j0 + i;
-    slot_id[i] = a.kv_page_indices[pbase + (tok >> 4)] * TWL_PAGE + (tok & 15);
-  }
-  float qf[G][8];
-#pragma unroll
-  for (int g = 0; g < G; ++g) {
-    const u32x4 v = *(const u32x4*)((const uint16_t*)a.q +
-                                    ((size_t)b * a.num_q_heads + kvh * G + g) * TWL_HEAD_DIM + 8 * sub);
-    grp_unpack8<DT>(v, qf[g]);
-#pragma unroll
-    for (int d = 0; d < 8; ++d) qf[g][d] *= a.scale_log2;
-  }
-  __syncthreads();
-
-  const size_t head_off = (size_t)kvh * a.head_stride + 8 * sub;
-  const uint16_t* kc = (const uint16_t*)a.k_cache;
-  const uint16_t* vc = (const uint16_t*)a.v_cache;
-  float m[G], l[G], acc[G][8];
-#pragma unroll
-  for (int g = 0; g < G; ++g) {
-    m[g] = kGrpNoMax;
-    l[g] = 0.0f;
-#pragma unroll
-    for (int d = 0; d < 8; ++d) acc[g][d] = 0.0f;
-  }
-
-  const int steps = (cn + (int)ts - 1) / (int)ts;   // list positions tsel + ts * s, s < steps
-  for (int s0 = 0; s0 < steps; s0 += kGrpUnroll) {
-    u32x4 kreg[kGrpUnroll], vreg[kGrpUnroll];
-    bool valid[kGrpUnroll];
-    size_t off[kGrpUnroll];
-#pragma unroll
-    for (int u = 0; u < kGrpUnroll; ++u) {
-      const int t = tsel + (int)ts * (s0 + u);
-      valid[u] = t < cn;
-      const int sid = slot_id[min(t, cn - 1)];
-      off[u] = (size_t)(sid >> 4) * a.page_stride + (size_t)(sid & 15) * a.token_stride + head_off;
-      kreg[u] = __builtin_nontemporal_load((const u32x4*)(kc + off[u]));
+    // ---- resolve the chunk's token addresses once --------------------------------------------
+    const int pbase = a.kv_page_indptr[b];
+    for (int i = tx; i < cn; i += kGrpThreads) {
+      const int tok = a.idx ? a.idx[((size_t)b * a.num_kv_heads + kvh) * a.idx_stride + j0 + i] : j0 + i;
+      slot_id[i] = a.kv_page_indices[pbase + (tok >> 4)] * TWL_PAGE + (tok & 15);
     }
-#pragma unroll
-    for (int u = 0; u < kGrpUnroll; ++u)
-      vreg[u] = __builtin_nontemporal_load((const u32x4*)(vc + off[u]));
-
-    float sc[kGrpUnroll][G];
-#pragma unroll
-    for (int u = 0; u < kGrpUnroll; ++u) {
-      float kf[8];
-      grp_unpack8<DT>(kreg[u], kf);
-#pragma unroll
-      for (int g = 0; g < G; ++g) {
-        float d0 = 0.0f;
-#pragma unroll
-        for (int d = 0; d < 8; ++d) d0 = fmaf(qf[g][d], kf[d], d0);
-        d0 = row16_allreduce<OpSum>(d0);
-        sc[u][g] = valid[u] ? d0 : -__builtin_inff();
-      }
-    }
+    float qf[G][8];
 #pragma unroll
     for (int g = 0; g < G; ++g) {
-      float mn = m[g];
+      const u32x4 v = *(const u32x4*)((const uint16_t*)a.q +
+                                      ((size_t)b * a.num_q_heads + kvh * G + g) * TWL_HEAD_DIM + 8 * sub);
+      grp_unpack8<DT>(v, qf[g]);
 #pragma unroll
-      for (int u = 0; u < kGrpUnroll; ++u) mn = fmaxf(mn, sc[u][g]);
-      const float f = __builtin_amdgcn_exp2f(m[g] - mn);
-      m[g] = mn;
-      float ps = 0.0f;
+      for (int d = 0; d < 8; ++d) qf[g][d] *= a.scale_log2;
+    }
+    __syncthreads();
+
+    const size_t head_off = (size_t)kvh * a.head_stride + 8 * sub;
+    const uint16_t* kc = (const uint16_t*)a.k_cache;
+    const uint16_t* vc = (const uint16_t*)a.v_cache;
+    float m[G], l[G], acc[G][8];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      m[g] = kGrpNoMax;
+      l[g] = 0.0f;
+#pragma unroll
+      for (int d = 0; d < 8; ++d) acc[g][d] = 0.0f;
+    }
+
+    const int steps = (cn + (int)ts - 1) / (int)ts;   // list positions tsel + ts * s, s < steps
+    for (int s0 = 0; s0 < steps; s0 += kGrpUnroll) {
+      u32x4 kreg[kGrpUnroll], vreg[kGrpUnroll];
+      bool valid[kGrpUnroll];
+      size_t off[kGrpUnroll];
 #pragma unroll
       for (int u = 0; u < kGrpUnroll; ++u) {
-        sc[u][g] = __builtin_amdgcn_exp2f(sc[u][g] - mn);   // now the weight
-        ps += sc[u][g];
+        const int t = tsel + (int)ts * (s0 + u);
+        valid[u] = t < cn;
+        const int sid = slot_id[min(t, cn - 1)];
+        off[u] = (size_t)(sid >> 4) * a.page_stride + (size_t)(sid & 15) * a.token_stride + head_off;
+        kreg[u] = __builtin_nontemporal_load((const u32x4*)(kc + off[u]));
       }
-      l[g] = fmaf(l[g], f, ps);
 #pragma unroll
-      for (int d = 0; d < 8; ++d) acc[g][d] *= f;
-    }
-#pragma unroll
-    for (int u = 0; u < kGrpUnroll; ++u) {
-      float vf[8];
-      grp_unpack8<DT>(vreg[u], vf);
-#pragma unroll
-      for (int g = 0; g < G; ++g)
-#pragma unroll
-        for (int d = 0; d < 8; ++d) acc[g][d] = fmaf(sc[u][g], vf[d], acc[g][d]);
-    }
-  }
+      for (int u = 0; u < kGrpUnroll; ++u)
+        vreg[u] = __builtin_nontemporal_load((const u32x4*)(vc + off[u]));
 
-  // ---- leave the lane group's partial result -------------------------------------------------
-  float* part = a.partials +
-                ((((size_t)b * a.num_kv_heads + kvh) * a.max_chunks + ch) * ts + tsel) *
-                    (size_t)(G * kGrpPartial);
+      float sc[kGrpUnroll][G];
 #pragma unroll
-  for (int g = 0; g < G; ++g) {
-    float* pg = part + g * kGrpPartial;
-    if (sub == 0) {
-      pg[0] = m[g];
-      pg[1] = l[g];
+      for (int u = 0; u < kGrpUnroll; ++u) {
+        float kf[8];
+        grp_unpack8<DT>(kreg[u], kf);
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+          float d0 = 0.0f;
+#pragma unroll
+          for (int d = 0; d < 8; ++d) d0 = fmaf(qf[g][d], kf[d], d0);
+          d0 = row16_allreduce<OpSum>(d0);
+          sc[u][g] = valid[u] ? d0 : -__builtin_inff();
+        }
+      }
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        float mn = m[g];
+#pragma unroll
+        for (int u = 0; u < kGrpUnroll; ++u) mn = fmaxf(mn, sc[u][g]);
+        const float f = __builtin_amdgcn_exp2f(m[g] - mn);
+        m[g] = mn;
+        float ps = 0.0f;
+#pragma unroll
+        for (int u = 0; u < kGrpUnroll; ++u) {
+          sc[u][g] = __builtin_amdgcn_exp2f(sc[u][g] - mn);   // now the weight
+          ps += sc[u][g];
+        }
+        l[g] = fmaf(l[g], f, ps);
+#pragma unroll
+        for (int d = 0; d < 8; ++d) acc[g][d] *= f;
+      }
+#pragma unroll
+      for (int u = 0; u < kGrpUnroll; ++u) {
+        float vf[8];
+        grp_unpack8<DT>(vreg[u], vf);
+#pragma unroll
+        for (int g = 0; g < G; ++g)
+#pragma unroll
+          for (int d = 0; d < 8; ++d) acc[g][d] = fmaf(sc[u][g], vf[d], acc[g][d]);
+      }
     }
-    f32x4* dst = (f32x4*)(pg + 4 + 8 * sub);
-    dst[0] = f32x4{acc[g][0], acc[g][1], acc[g][2], acc[g][3]};
-    dst[1] = f32x4{acc[g][4], acc[g][5], acc[g][6], acc[g][7]};
-  }
-  __syncthreads();   // slot_id is rewritten by the next chunk
+
+    // ---- leave the lane group's partial result -------------------------------------------------
+    float* part = a.partials +
+                  ((((size_t)b * a.num_kv_heads + kvh) * a.max_chunks + ch) * ts + tsel) *
+                      (size_t)(G * kGrpPartial);
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      float* pg = part + g * kGrpPartial;
+      if (sub == 0) {
+        pg[0] = m[g];
+        pg[1] = l[g];
+      }
+      f32x4* dst = (f32x4*)(pg + 4 + 8 * sub);
+      dst[0] = f32x4{acc[g][0], acc[g][1], acc[g][2], acc[g][3]};
+      dst[1] = f32x4{acc[g][4], acc[g][5], acc[g][6], acc[g][7]};
+    }
+    __syncthreads();   // slot_id is rewritten by the next chunk
   }
 }
 
