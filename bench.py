@@ -243,7 +243,7 @@ def bench_llama3_model(args, dev) -> int:
     from twilight_amd import hf
     B, N, nl = args.batch, args.context, args.model_layers
     steps, warmup = min(args.steps, 32), min(args.warmup, 4)
-    top_p = args.top_p if args.top_p != 0.95 else 0.9    # the configuration's p unless one is given
+    top_p = args.top_p
     cfg = LlamaConfig(vocab_size=128256, hidden_size=4096, intermediate_size=14336,
                       num_hidden_layers=nl, num_attention_heads=32, num_key_value_heads=8,
                       head_dim=128, max_position_embeddings=N + 4096, rope_theta=500000.0,
@@ -416,7 +416,8 @@ def main() -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=32768)
     ap.add_argument("--budget", type=int, default=8192)
-    ap.add_argument("--top-p", type=float, default=0.95)
+    ap.add_argument("--top-p", type=float, default=None,
+                    help="pruning threshold (default 0.95; 0.9 for the Llama-3 workloads)")
     ap.add_argument("--workload", choices=["longchat", "llama3", "llama3-model", "topp", "ftka"],
                     default="longchat",
                     help="longchat: 32 MHA heads fp16 (the headline workload); llama3: GQA 32/8 "
@@ -443,6 +444,8 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel breakdown")
     args = ap.parse_args()
+    if args.top_p is None:
+        args.top_p = 0.9 if args.workload in ("llama3", "llama3-model") else 0.95
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU part (every (batch, head) "
               "row is independent); run with --gpus 1", file=sys.stderr)

@@ -66,16 +66,6 @@ inline GroupPlan group_plan(uint32_t batch, uint32_t num_kv_heads, uint32_t max_
   return p;
 }
 
-template <int DT>
-__device__ __forceinline__ void grp_unpack8(const u32x4& v, float* f) {
-  const uint32_t ws[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    f[2 * j] = bits16_to_f32<DT>(ws[j] & 0xFFFFu);
-    f[2 * j + 1] = bits16_to_f32<DT>(ws[j] >> 16);
-  }
-}
-
 // tokens of request b / list length of (b, kvh)
 __device__ __forceinline__ int group_list_len(const GroupAttnArgs& a, uint32_t b, uint32_t kvh) {
   if (a.idx) return min(max(a.count[b * a.num_kv_heads + kvh], 0), (int)a.idx_stride);
@@ -117,7 +107,7 @@ __global__ __launch_bounds__(kGrpThreads) void group_attn_partial_kernel(GroupAt
     for (int g = 0; g < G; ++g) {
       const u32x4 v = *(const u32x4*)((const uint16_t*)a.q +
                                       ((size_t)b * a.num_q_heads + kvh * G + g) * TWL_HEAD_DIM + 8 * sub);
-      grp_unpack8<DT>(v, qf[g]);
+      unpack8<DT>(v, qf[g]);
 #pragma unroll
       for (int d = 0; d < 8; ++d) qf[g][d] *= a.scale_log2;
     }
@@ -156,7 +146,7 @@ __global__ __launch_bounds__(kGrpThreads) void group_attn_partial_kernel(GroupAt
 #pragma unroll
       for (int u = 0; u < kGrpUnroll; ++u) {
         float kf[8];
-        grp_unpack8<DT>(kreg[u], kf);
+        unpack8<DT>(kreg[u], kf);
 #pragma unroll
         for (int g = 0; g < G; ++g) {
           float d0 = 0.0f;
@@ -186,7 +176,7 @@ __global__ __launch_bounds__(kGrpThreads) void group_attn_partial_kernel(GroupAt
 #pragma unroll
       for (int u = 0; u < kGrpUnroll; ++u) {
         float vf[8];
-        grp_unpack8<DT>(vreg[u], vf);
+        unpack8<DT>(vreg[u], vf);
 #pragma unroll
         for (int g = 0; g < G; ++g)
 #pragma unroll

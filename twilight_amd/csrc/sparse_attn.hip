@@ -48,16 +48,6 @@ constexpr int kAttnChunk = 128;                        // survivors per workgrou
 constexpr int kAttnSteps = kAttnChunk / (4 * kAttnWaves);  // 8 tokens per lane-group
 constexpr int kAttnPartial = TWL_HEAD_DIM + 2;         // m, l, acc[128]
 
-template <int DT>
-__device__ __forceinline__ void unpack8(const u32x4& v, float* f) {
-  const uint32_t ws[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    f[2 * j] = bits16_to_f32<DT>(ws[j] & 0xFFFFu);
-    f[2 * j + 1] = bits16_to_f32<DT>(ws[j] >> 16);
-  }
-}
-
 struct AttnSmem {
   int slot_id[kAttnChunk];      // physical token slot = page * 16 + slot
   float w[kAttnChunk];          // logits, then weights

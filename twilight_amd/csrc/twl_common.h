@@ -54,6 +54,17 @@ __device__ __forceinline__ float round_to(float f) {
   return f;
 }
 
+// eight 16-bit values of a 16-byte load, widened to fp32 (element order = memory order)
+template <int DT>
+__device__ __forceinline__ void unpack8(const u32x4& v, float* f) {
+  const uint32_t ws[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    f[2 * j] = bits16_to_f32<DT>(ws[j] & 0xFFFFu);
+    f[2 * j + 1] = bits16_to_f32<DT>(ws[j] >> 16);
+  }
+}
+
 // ---- DPP data movement -----------------------------------------------------------------------
 // Lanes disabled by ROW_MASK / out-of-range sources receive `old`.
 template <int CTRL, int ROW_MASK = 0xF>
