@@ -323,7 +323,8 @@ def bench_llama3_model(args, dev) -> int:
         return (time.perf_counter() - t0) / steps, logits[:, -1].float()
 
     twi = {}
-    for mode in ("model", "paged", "paged+graph"):
+    modes = ("model", "paged", "paged+graph") if args.model_mode == "all" else (args.model_mode,)
+    for mode in modes:
         # "model": the two dense layers run the model's own attention over a DynamicCache;
         # "paged": they run twl_group_attn over paged K / V and the model's cache stays empty;
         # "paged+graph": the same step recorded once into a HIP graph and replayed
@@ -338,7 +339,7 @@ def bench_llama3_model(args, dev) -> int:
         t, logits = run_graphed() if mode == "paged+graph" else run(cache, positions=True)
         twi[mode] = t * 1e3
         kept = info.get_total_avg_budget()
-        if mode != "paged+graph":
+        if mode != modes[-1]:
             hf.disable_sparse_attention(model)
             del cache, states
             torch.cuda.empty_cache()
@@ -430,6 +431,8 @@ def main() -> int:
     ap.add_argument("--q-gain", type=float, default=3.0,
                     help="llama3-model: factor on the random q_proj weights (peakedness of attention)")
     ap.add_argument("--no-dense", action="store_true", help="llama3-model: skip the dense run")
+    ap.add_argument("--model-mode", choices=["all", "model", "paged", "paged+graph"], default="all",
+                    help="llama3-model: which of the patched runs to time (see dense_layers_what)")
     ap.add_argument("--layers", type=int, default=4,
                     help="independent layer caches visited round-robin (cold-cache steps)")
     ap.add_argument("--calibrate-copy", action="store_true",

@@ -350,6 +350,7 @@ class GraphedDecodeStep:
         self.states.sort(key=lambda t: t[0])
         self.graph: Optional[torch.cuda.CUDAGraph] = None
         self.ids = self.pos = self.logits = self.past = None
+        self._warm = False
 
     def _prepare(self, input_ids: torch.Tensor) -> None:
         from transformers import DynamicCache
@@ -364,7 +365,8 @@ class GraphedDecodeStep:
         self.past = DynamicCache(config=self.model.config)   # stays empty: nothing updates it
 
     def __call__(self, input_ids: torch.Tensor) -> torch.Tensor:
-        """``input_ids`` [B, 1] -> logits [B, 1, vocab] (the same buffer every call)."""
+        """``input_ids`` [B, 1] -> logits [B, 1, vocab] (from the second call on the same buffer
+        every call; the first call runs the step eagerly, the second records it)."""
         if self.ids is None:
             self._prepare(input_ids)
         seq = self.states[0][1].seq_len
@@ -377,14 +379,22 @@ class GraphedDecodeStep:
         try:
             self.ids.copy_(input_ids)
             self.pos.fill_(seq)
-            if self.graph is None:
-                graph = torch.cuda.CUDAGraph()
-                with torch.no_grad(), torch.cuda.graph(graph):
-                    out = self.model(self.ids, past_key_values=self.past, use_cache=True,
-                                     position_ids=self.pos)
-                self.graph, self.logits = graph, out.logits
-            # recording does not execute: the step itself is the replay, the first time too
-            self.graph.replay()
+            if not self._warm:
+                # the first step runs eagerly, with the same shapes and buffers: libraries that
+                # set themselves up on first use (GEMM workspaces) must not do so while recording
+                with torch.no_grad():
+                    self.logits = self.model(self.ids, past_key_values=self.past, use_cache=True,
+                                             position_ids=self.pos).logits
+                self._warm = True
+            else:
+                if self.graph is None:
+                    graph = torch.cuda.CUDAGraph()
+                    with torch.no_grad(), torch.cuda.graph(graph):
+                        out = self.model(self.ids, past_key_values=self.past, use_cache=True,
+                                         position_ids=self.pos)
+                    self.graph, self.logits = graph, out.logits
+                # recording does not execute: the step itself is the replay, the first time too
+                self.graph.replay()
         finally:
             for _, st in self.states:
                 st.recorded = False
