@@ -79,7 +79,7 @@ enum twl_top_p_high {
 const char* twl_strerror(int status);
 /* ABI version of this header; bumps when a signature changes. twl_abi_version() returns the
  * version the library was built with: a caller compares the two before anything else. */
-#define TWL_ABI_VERSION 6
+#define TWL_ABI_VERSION 7
 int twl_abi_version(void);
 /* Number of HIP devices visible, or a negative twl_status. */
 int twl_device_count(void);
@@ -310,6 +310,18 @@ int twl_quest_topk_pages(const float* page_scores, uint32_t score_stride,
                          const int32_t* kv_page_indptr, uint32_t batch, uint32_t num_q_heads,
                          uint32_t token_budget, uint32_t max_pages_per_req, int32_t* sel_pages,
                          uint32_t sel_stride, int32_t* sel_count, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Rotary position embedding of one decode token, in place: q [batch, num_q_heads, 128] and
+ * k [batch, num_kv_heads, 128] in dtype, cos / sin [batch, 128] in dtype (the values of the
+ * request's position).
+ * Replaces: apply_rotary_pos_emb as called at twilight/pyimpl/attention.py:118-123 (half-split
+ * convention: out = x * cos + rotate_half(x) * sin, rotate_half(x) = (-x[64:], x[:64])), with
+ * the roundings of its chain of element-wise tensor operations (each product and the sum rounded
+ * to dtype), so the result is bit-identical to the unfused form; one launch instead of about ten.
+ * ------------------------------------------------------------------------------------------- */
+int twl_rope_qk(void* q, void* k, const void* cos, const void* sin, int dtype, uint32_t batch,
+                uint32_t num_q_heads, uint32_t num_kv_heads, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * KV-append side: build the INT4 shadow and the Quest metadata of whole pages from the paged K.

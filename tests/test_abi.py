@@ -20,7 +20,7 @@ def test_header_symbols_are_exported(hip_lib):
     assert declared == set(_lib.EXPORTS)
     for name in declared:
         assert hasattr(hip_lib, name), name
-    assert hip_lib.twl_abi_version() == int(re.search(r"#define TWL_ABI_VERSION (\d+)", hdr).group(1)) == 6
+    assert hip_lib.twl_abi_version() == int(re.search(r"#define TWL_ABI_VERSION (\d+)", hdr).group(1)) == 7
 
 
 def test_header_compiles_as_c():

@@ -244,3 +244,25 @@ def test_graphed_decode_step_equals_eager_decode(dev):
     with pytest.raises(RuntimeError):
         hf.GraphedDecodeStep(model)
     hf.disable_sparse_attention(model)
+
+
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
+def test_fused_rotary_embedding_equals_the_tensor_form(dev, dt):
+    # one launch, in place, bit-identical to apply_rotary_pos_emb on tensors of the same dtype
+    # (twilight/pyimpl/attention.py:118-123 calls that function)
+    import twilight_amd.kernel as K
+    from transformers.models.llama.modeling_llama import apply_rotary_pos_emb
+    B, H, Hkv = 3, 8, 2
+    g = torch.Generator().manual_seed(13)
+    q = (torch.randn((B, H, 1, 128), generator=g) * 3).to(dt).to(dev)
+    k = (torch.randn((B, Hkv, 1, 128), generator=g) * 3).to(dt).to(dev)
+    pos = torch.tensor([[5.0], [1234.0], [32767.0]])
+    inv = 1.0 / (500000.0 ** (torch.arange(0, 128, 2).float() / 128))
+    ang = torch.cat([pos * inv, pos * inv], dim=-1)                       # [B, 128]
+    cos, sin = ang.cos().to(dt).to(dev), ang.sin().to(dt).to(dev)
+    want_q, want_k = apply_rotary_pos_emb(q, k, cos[:, None], sin[:, None])
+    q3, k3 = q[:, :, 0].contiguous(), k[:, :, 0].contiguous()
+    K.rope_qk_(q3, k3, cos, sin)
+    assert torch.equal(q3, want_q[:, :, 0]) and torch.equal(k3, want_k[:, :, 0])
+    with pytest.raises(RuntimeError):
+        K.rope_qk_(q3, k3, cos.float(), sin.float())

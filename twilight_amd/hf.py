@@ -21,7 +21,8 @@ import torch
 
 from . import _lib
 from .cache import PagedKVCache
-from .kernel.attention import group_attention_workspace_bytes, group_paged_decode_attention
+from .kernel.attention import (group_attention_workspace_bytes, group_paged_decode_attention,
+                               rope_qk_)
 from .layer import TwilightDecodeLayer, parse_sparse_config
 
 PAGE = _lib.PAGE
@@ -204,7 +205,6 @@ def _twilight_attention_forward(self, hidden_states, position_embeddings=None, a
                                 past_key_values=None, **kwargs):
     """Replacement of ``LlamaAttention.forward``: the module's own forward for prefill, the
     Select-then-Prune layer for decode (twilight/pyimpl/attention.py:59-306 split the same way)."""
-    from transformers.models.llama.modeling_llama import apply_rotary_pos_emb
     st: _LayerState = self._twilight_state
     q_len = hidden_states.shape[1]
     if q_len > 1 or past_key_values is None:
@@ -227,12 +227,17 @@ def _twilight_attention_forward(self, hidden_states, position_embeddings=None, a
         n = st.seq_len if st.seq_len > 0 else past_key_values.get_seq_length(self.layer_idx)
         fill_from_prefill(st, keys[:, :, :n], lay.values[:, :, :n], self.config.num_attention_heads)
     B = hidden_states.shape[0]
-    hidden_shape = (B, 1, -1, self.head_dim)
-    q = self.q_proj(hidden_states).view(hidden_shape).transpose(1, 2)
-    k = self.k_proj(hidden_states).view(hidden_shape).transpose(1, 2)
-    v = self.v_proj(hidden_states).view(hidden_shape).transpose(1, 2)
+    # one token per request: the projections are already [B, heads, 128]; the rotary embedding
+    # is one launch, in place, with the roundings of the model's own chain of tensor operations
+    q = self.q_proj(hidden_states).view(B, -1, self.head_dim)
+    k = self.k_proj(hidden_states).view(B, -1, self.head_dim)
+    v = self.v_proj(hidden_states).view(B, -1, self.head_dim)
     cos, sin = position_embeddings
-    q, k = apply_rotary_pos_emb(q, k, cos, sin)
+    cos, sin = cos[:, 0].expand(B, -1).contiguous(), sin[:, 0].expand(B, -1).contiguous()
+    if cos.dtype != q.dtype:
+        cos, sin = cos.to(q.dtype), sin.to(q.dtype)
+    rope_qk_(q, k, cos, sin)
+    q, k, v = q.unsqueeze(2), k.unsqueeze(2), v.unsqueeze(2)      # [B, heads, 1, 128] views
     if st.keep_hf_cache:
         past_key_values.update(k, v, self.layer_idx)  # keeps the model's own cache consistent
     if st.recorded:   # GraphedDecodeStep has done the host half for this step

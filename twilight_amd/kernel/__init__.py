@@ -12,7 +12,7 @@ from .gemv import (batched_sparse_gemv, batched_sparse_gemv_int4_k, batched_spar
                    single_sparse_gemv, sparse_gemv_int4, sparse_gemv_int4_top_p,
                    quest_gemv_int4_top_p)
 from .attention import (attention_workspace_bytes, group_attention_workspace_bytes,
-                        group_paged_decode_attention, group_union_lists,
+                        group_paged_decode_attention, group_union_lists, rope_qk_,
                         sparse_paged_decode_attention)
 from .quest import quest_num_pages, quest_select
 from .kv_shadow import dequant_int4, kv_append, kv_shadow_build, meta_planes_build
@@ -24,7 +24,7 @@ __all__ = [
     "single_sparse_gemv", "sparse_gemv_int4", "sparse_gemv_int4_top_p", "quest_gemv_int4_top_p",
     "sparse_paged_decode_attention",
     "attention_workspace_bytes", "group_paged_decode_attention", "group_union_lists",
-    "group_attention_workspace_bytes",
+    "group_attention_workspace_bytes", "rope_qk_",
     "quest_num_pages", "quest_select", "dequant_int4", "kv_shadow_build", "kv_append", "meta_planes_build",
     "get_label_tensor", "bgemv_int8", "qk_int8_per_block",
 ]

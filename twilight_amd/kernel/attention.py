@@ -215,3 +215,24 @@ def group_union_lists(idx: torch.Tensor, count: torch.Tensor, num_kv_heads: int,
                                         ptr(gidx), group_stride, ptr(gcnt), stream_of(idx))
     _lib.check(rc, "GroupUnionLists")
     return gidx, gcnt
+
+
+def rope_qk_(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> None:
+    """Rotary position embedding of one decode token in place: ``q`` [B,H,128], ``k`` [B,Hkv,128],
+    ``cos`` / ``sin`` [B,128], all contiguous in one dtype (fp16 / bf16). Same values, bit for bit,
+    as ``apply_rotary_pos_emb`` on tensors of that dtype (twilight/pyimpl/attention.py:118-123)."""
+    for name, t in (("q", q), ("k", k), ("cos", cos), ("sin", sin)):
+        check_input(t, name)
+        if t.dtype != q.dtype:
+            raise RuntimeError("q, k, cos and sin must share one dtype")
+    check_dim(3, q, "q"); check_dim(3, k, "k"); check_dim(2, cos, "cos"); check_dim(2, sin, "sin")
+    B, H, D = q.shape
+    if D != _lib.HEAD_DIM or k.size(2) != D or k.size(0) != B:
+        raise RuntimeError("q must be [B,H,128] and k [B,Hkv,128]")
+    if tuple(cos.shape) != (B, D) or tuple(sin.shape) != (B, D):
+        raise RuntimeError("cos and sin must be [B,128]")
+    check_same_device(q, ("k", k), ("cos", cos), ("sin", sin))
+    with torch.cuda.device(q.device):
+        rc = _lib.lib().twl_rope_qk(ptr(q), ptr(k), ptr(cos), ptr(sin), dtype_code(q.dtype, "q"), B, H,
+                                    k.size(1), stream_of(q))
+    _lib.check(rc, "RopeQK")
