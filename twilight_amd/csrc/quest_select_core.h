@@ -15,7 +15,7 @@ __device__ __forceinline__ int quest_budget_pages(uint32_t token_budget) {
 
 struct SelSmem {
   int hist[4][256];  // one histogram per radix pass (at most 4 x 8 bits), zeroed by select_smem_init
-  int pick[4][2];    // per pass: chosen digit, remaining k
+  int pick[4][3];    // per pass: chosen digit, remaining k, keys in the chosen bin
   int scr[32];       // per-wave key maxima / minima
   int wave_tot[16];
 };
@@ -137,6 +137,7 @@ __device__ __forceinline__ void select_row_topk(const float* src, int n_pages, i
           if (run < k_rem && k_rem <= run + hcnt[j]) {
             sm.pick[pass][0] = 255 - 4 * lane - j;
             sm.pick[pass][1] = k_rem - run;
+            sm.pick[pass][2] = hcnt[j];
           }
           run += hcnt[j];
         }
@@ -147,9 +148,16 @@ __device__ __forceinline__ void select_row_topk(const float* src, int n_pages, i
     prefix_mask |= dmask << shift;
     k_rem = sm.pick[pass][1];
     top = shift;
+    if (k_rem == sm.pick[pass][2] && top > 0 && prefix != 0u) {
+      // every key of the chosen bin is taken: the remaining digits need not be resolved (after
+      // two passes a bin mostly holds one or two keys). Keys >= prefix are the selection.
+      prefix -= 1u;
+      k_rem = 0;
+      break;
+    }
     ++pass;
   }
-  const uint32_t T = prefix;  // k-th largest key; k_rem of the keys equal to T are taken
+  const uint32_t T = prefix;  // keys > T are taken, and k_rem of the keys equal to T
 
   // ---- ordered compaction ------------------------------------------------------------------
   int packed = 0;  // (count of key > T) << 16 | (count of key == T)
