@@ -39,7 +39,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 QUEST_SCORE_TRAFFIC_BYTES_DEFAULT = int((131404.9 * 2.000 + 2048.0 * 1.000) * 1024)
 # The same for select_estimate_prune_kernel (FETCH_SIZE KiB x 2.000 + WRITE_SIZE KiB x 1.000).
 ROW_KERNEL_TRAFFIC_BYTES_RECORDS = int((213640.2 * 2.000 + 596.1 * 1.000) * 1024)  # --no-planes
-ROW_KERNEL_TRAFFIC_BYTES_DEFAULT = int((148074.8 * 2.000 + 596.1 * 1.000) * 1024)  # plane layout
+ROW_KERNEL_TRAFFIC_BYTES_DEFAULT = int((148094.6 * 2.000 + 596.1 * 1.000) * 1024)  # plane layout
 
 
 def _time_calls(fn, iters: int, warmup: int) -> float:
