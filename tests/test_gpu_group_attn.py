@@ -177,3 +177,48 @@ def test_group_attention_rejects_bad_arguments(dev):
     cnt = torch.zeros((1, 4), dtype=torch.int32, device=dev)
     with pytest.raises(RuntimeError):                                    # bitmap limit
         K.group_union_lists(idx, cnt, 2, 1 << 20)
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_group_attention_random_shapes(dev, seed):
+    # random batch, grouping, dtype and request lengths around the chunk and page boundaries,
+    # dense form and list form (random per-group subsets) against the masked reference
+    rng = np.random.default_rng(100 + seed)
+    dt = [torch.float16, torch.bfloat16][seed % 2]
+    G = int(rng.choice([1, 2, 4, 8]))
+    Hkv = int(rng.choice([1, 2, 3, 4, 8]))
+    H = G * Hkv
+    B = int(rng.integers(1, 5))
+    edges = [1, 2, 15, 16, 17, 63, 64, 65, 127, 128, 129, 255, 256, 257, 511, 513, 1000, 2047]
+    lens = [int(rng.choice(edges)) for _ in range(B)]
+    N = max(lens)
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn((B, H, 1, 128), generator=g).to(dt)
+    k = torch.randn((B, Hkv, N, 128), generator=g).to(dt)
+    v = torch.randn((B, Hkv, N, 128), generator=g).to(dt)
+    npg = (N + 15) // 16
+    cache = PagedKVCache.from_dense(k, v, dev, page_perm=torch.randperm(B * npg, generator=g))
+    _ragged(cache, lens)
+    qd = q[:, :, 0].contiguous().to(dev)
+    krep, vrep = k.float().repeat_interleave(G, dim=1), v.float().repeat_interleave(G, dim=1)
+    dense_mask = torch.zeros((B, H, 1, N), dtype=torch.bool)
+    for b, n in enumerate(lens):
+        dense_mask[b, :, :, :n] = True
+    out = K.group_paged_decode_attention(qd, cache.k_cache, cache.v_cache, cache.kv_page_indices,
+                                         cache.kv_page_indptr, cache.kv_last_page_len, max_tokens=N)
+    ref = P.masked_attention(q.float(), krep, vrep, dense_mask)[:, :, 0]
+    assert torch.allclose(out.cpu().float(), ref, rtol=_tol(dt), atol=_tol(dt)), (lens, H, Hkv)
+    # list form: a random subset of each request's tokens per kv head (some empty)
+    gmask = (torch.rand((B, Hkv, 1, N), generator=g) < float(rng.uniform(0.05, 0.9))) & dense_mask[:, ::G]
+    gmask[0, 0] = False
+    gidx, gcount = P.mask_to_lists(gmask)
+    out2 = K.group_paged_decode_attention(
+        qd, cache.k_cache, cache.v_cache, cache.kv_page_indices, cache.kv_page_indptr,
+        group_idx=torch.from_numpy(np.maximum(gidx, 0)).reshape(B, Hkv, N).to(dev),
+        group_count=torch.from_numpy(gcount).reshape(B, Hkv).to(dev))
+    umask = gmask.repeat_interleave(G, dim=1)
+    ref2 = P.masked_attention(q.float(), krep, vrep, umask)[:, :, 0]
+    rows = umask.any(-1)[:, :, 0]
+    got2 = out2.cpu().float()
+    assert torch.all(got2[~rows] == 0)
+    assert torch.allclose(got2[rows], ref2[rows], rtol=_tol(dt), atol=_tol(dt)), (lens, H, Hkv)
