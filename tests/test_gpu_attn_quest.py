@@ -135,3 +135,23 @@ def test_sparse_attention_split_rows_share_a_workspace(dev):
         ref = P.masked_attention(q.float(), k.float(), v.float(), mask, prob_dtype=torch.float16)[:, :, 0]
         assert torch.allclose(out.cpu().float(), ref, rtol=1e-3, atol=1e-3), trial
         assert int(ws[:B * H * 4].view(torch.int32).abs().sum()) == 0
+
+
+def test_attention_folds_positions_outside_the_request(dev):
+    # a list entry beyond the request's pages must not be read past the page table: it is folded
+    # onto the request's last page (the kernel must finish and give finite numbers)
+    g = torch.Generator().manual_seed(21)
+    B, H, N = 1, 2, 100
+    q = torch.randn((B, H, 128), generator=g).half().to(dev)
+    k = torch.randn((B, H, N, 128), generator=g).half()
+    cache = PagedKVCache.from_dense(k, k, dev)
+    idx = torch.tensor([[[0, 5, 1 << 20, -7], [3, 99, 100000, 0]]], dtype=torch.int32, device=dev)
+    cnt = torch.tensor([[4, 3]], dtype=torch.int32, device=dev)
+    out = K.sparse_paged_decode_attention(q, cache.k_cache, cache.v_cache, idx, cnt,
+                                          cache.kv_page_indices, cache.kv_page_indptr)
+    assert torch.isfinite(out).all()
+    gi = torch.tensor([[[0, 1 << 22], [5, -3]]], dtype=torch.int32, device=dev)
+    gc = torch.tensor([[2, 2]], dtype=torch.int32, device=dev)
+    out2 = K.group_paged_decode_attention(q, cache.k_cache, cache.v_cache, cache.kv_page_indices,
+                                          cache.kv_page_indptr, group_idx=gi, group_count=gc)
+    assert torch.isfinite(out2).all()

@@ -98,9 +98,13 @@ __global__ __launch_bounds__(kGrpThreads) void group_attn_partial_kernel(GroupAt
 
     // ---- resolve the chunk's token addresses once --------------------------------------------
     const int pbase = a.kv_page_indptr[b];
+    const int plast = max(a.kv_page_indptr[b + 1] - pbase - 1, 0);
     for (int i = tx; i < cn; i += kGrpThreads) {
-      const int tok = a.idx ? a.idx[((size_t)b * a.num_kv_heads + kvh) * a.idx_stride + j0 + i] : j0 + i;
-      slot_id[i] = a.kv_page_indices[pbase + (tok >> 4)] * TWL_PAGE + (tok & 15);
+      const int tok =
+          a.idx ? a.idx[((size_t)b * a.num_kv_heads + kvh) * a.idx_stride + j0 + i] : j0 + i;
+      // a position outside the request (a corrupt list) is folded onto its last page rather than
+      // read past the page table
+      slot_id[i] = a.kv_page_indices[pbase + min(max(tok >> 4, 0), plast)] * TWL_PAGE + (tok & 15);
     }
     float qf[G][8];
 #pragma unroll

@@ -86,7 +86,11 @@ __device__ __forceinline__ void attn_chunk(const AttnArgs& a, AttnSmem& sm, uint
     int sid = 0;
     if (tx < cn) {
       const int tok = HAVE_TOK ? tok_pre : a.idx[(size_t)row * a.idx_stride + j0 + tx];
-      sid = a.kv_page_indices[a.kv_page_indptr[b] + (tok >> 4)] * TWL_PAGE + (tok & 15);
+      // a position outside the request (a corrupt list) is folded onto its last page rather than
+      // read past the page table
+      const int pg_lo = a.kv_page_indptr[b], pg_hi = a.kv_page_indptr[b + 1];
+      const int pg = min(max(tok >> 4, 0), max(pg_hi - pg_lo - 1, 0));
+      sid = a.kv_page_indices[pg_lo + pg] * TWL_PAGE + (tok & 15);
     }
     slot_id[tx] = sid;
   }
