@@ -14,6 +14,12 @@ the kernel with the largest HBM term (the Quest metadata stream); ``kernels`` li
 the layer with its algorithmic bytes, time and fraction of the 8 TB/s peak, and ``gemv_cfg2`` the
 stand-alone INT4 GEMV at 8 x 32 x 32768 candidates. ``cpu_baseline`` is the CPU oracle (a port of
 the reference's torch path) timed on this host on one of the 8 batch elements and scaled by 8.
+
+Other workloads (``--workload``), each printing one JSON line of its own: ``llama3`` (the same
+layer with 32 q heads on 8 kv heads, bf16, p 0.9, plus dense-decode comparisons), ``topp`` (the
+pruner alone), ``ftka`` (the NHD GEMV call shapes and the Double-Sparse label ops),
+``llama3-model`` (whole-model decode of a random-initialised Llama-3-8B shape, tokens/s, dense
+against the patched model).
 """
 from __future__ import annotations
 
