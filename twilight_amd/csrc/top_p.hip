@@ -157,46 +157,36 @@ __global__ __launch_bounds__(THREADS) void top_p_kernel(TopPArgs a) {
   if (a.idx || a.count) {
     int32_t* dst = a.idx ? a.idx + (size_t)row * a.idx_stride : nullptr;
     const int32_t* pages = a.sel_pages ? a.sel_pages + (size_t)row * a.sel_stride : nullptr;
+    // every chunk's wave totals go to LDS first, so the whole emission needs one barrier
+    __shared__ int chunk_tot[CHUNKS][16];
+    int mine[CHUNKS], excl[CHUNKS];
+    uint32_t keep[CHUNKS];
+#pragma unroll
+    for (int c = 0; c < CHUNKS; ++c) {
+      keep[c] = (x[4 * c + 0] > low ? 1u : 0u) | (x[4 * c + 1] > low ? 2u : 0u) |
+                (x[4 * c + 2] > low ? 4u : 0u) | (x[4 * c + 3] > low ? 8u : 0u);
+      mine[c] = __builtin_popcount(keep[c]);
+      const int scan = wave_inclusive_scan(mine[c]);   // in lane order
+      excl[c] = scan - mine[c];
+      if (lane == kWave - 1) chunk_tot[c][wave] = scan;
+    }
+    if (NWAVES > 1) __syncthreads();
     int base = 0;  // survivors emitted by earlier chunks (uniform)
 #pragma unroll
     for (int c = 0; c < CHUNKS; ++c) {
       const uint32_t e0 = 4u * (uint32_t)(tx + THREADS * c);
-      bool k0 = x[4 * c + 0] > low, k1 = x[4 * c + 1] > low;
-      bool k2 = x[4 * c + 2] > low, k3 = x[4 * c + 3] > low;
-      const int mine = (int)k0 + (int)k1 + (int)k2 + (int)k3;
-      // inclusive scan of `mine` across the wave, in lane order
-      int scan = mine;
-      {
-        int t;
-        t = dpp<0x111>(0, scan); scan += t;                    // row_shr:1
-        t = dpp<0x112>(0, scan); scan += t;                    // row_shr:2
-        t = dpp<0x114>(0, scan); scan += t;                    // row_shr:4
-        t = dpp<0x118>(0, scan); scan += t;                    // row_shr:8
-        t = dpp<kDppBcast15, 0xA>(0, scan); scan += t;         // rows 1,3 += end of rows 0,2
-        t = dpp<kDppBcast31, 0xC>(0, scan); scan += t;         // rows 2,3 += end of row 1
-      }
-      const int wtot = __builtin_amdgcn_readlane(scan, 63);
-      if (NWAVES > 1) {
-        __syncthreads();  // previous chunk's readers are done with wave_tot
-        if (lane == 0) wave_tot[wave] = wtot;
-        __syncthreads();
-      }
-      int before = 0, total = wtot;
-      if (NWAVES > 1) {
-        total = 0;
+      int before = 0, total = 0;
 #pragma unroll
-        for (int w = 0; w < NWAVES; ++w) {
-          const int t = wave_tot[w];
-          before += (w < wave) ? t : 0;
-          total += t;
-        }
+      for (int w = 0; w < NWAVES; ++w) {
+        const int t = chunk_tot[c][w];
+        before += (w < wave) ? t : 0;
+        total += t;
       }
-      if (dst && mine) {
-        int pos = base + before + scan - mine;
-        const bool kk[4] = {k0, k1, k2, k3};
+      if (dst && mine[c]) {
+        int pos = base + before + excl[c];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          if (kk[j]) {
+          if (keep[c] & (1u << j)) {
             const uint32_t e = e0 + j;
             dst[pos++] = pages ? (pages[e >> 4] * TWL_PAGE + (int)(e & 15u)) : (int)e;
           }
