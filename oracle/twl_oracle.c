@@ -11,7 +11,8 @@
  *                          pivots live in the 16-bit type, the partial sums are kept in fp32
  *                          (the reference sums in the 16-bit type, in an order fixed by CUB's
  *                          block reduction, which a sequential restatement cannot reproduce:
- *                          PARITY UNPINNED for the 16-bit entry)
+ *                          PARITY UNPINNED for the 16-bit entry, except on rows whose sums and
+ *                          midpoints are exact in every width, tests/golden "top_p_dyadic")
  *   twl_oracle_nucleus     textbook nucleus set (sort descending, cumulative sum in fp64):
  *                          the mathematical definition the bisection approximates
  *   twl_oracle_int4_quant  twilight/pyimpl/quantize.py:4-13 applied per group, with the fp16

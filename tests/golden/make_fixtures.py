@@ -13,6 +13,8 @@ cross-checked against the literal it is expected to equal:
   exactly 0.9, so p = 0.89 keeps the answer away from the rounding of that sum.
 * ``top_p_trace`` — a three-element row whose bisection (csrc/include/sampling.cuh:156-231, with
   ``high`` = the first element) is followed by hand: 3 iterations, final low 0.25.
+* ``top_p_dyadic`` — rows of powers of two, whose bisection is exact in every arithmetic width: the
+  one vector that pins the 16-bit entry point independently of how its sums are ordered.
 * ``gemv_constant`` — the constant inputs of benchmark/efficiency/bench_gemv.py:390-422: q = 1,
   every nibble 3, scale 1, zero 0, so every raw score is 3 * 128.
 """
@@ -67,6 +69,40 @@ def top_p_trace():
             "mask": [1 if x > low else 0 for x in probs], "low": low, "iterations": iters}
 
 
+def top_p_dyadic():
+    """Rows of powers of two: every sum and every midpoint is exact in fp32, fp16 and bf16 alike
+    (asserted below: at most 8 significant bits), so the bisection's trace does not depend on the
+    width of the arithmetic or on the order of a sum. Token 0 is the row maximum, so both choices
+    of the upper bound agree."""
+    from fractions import Fraction as F
+    rows = [[F(1, 2), F(1, 4), F(1, 8), F(1, 16), F(1, 32), F(1, 32)],
+            [F(1, 2), F(1, 8), F(1, 8), F(1, 8), F(1, 16), F(1, 16)],
+            [F(1, 4), F(1, 4), F(1, 4), F(1, 8), F(1, 16), F(1, 16)]]
+    p = F(7, 8)                     # exact in every width; compared with ">="
+    out = []
+    for probs in rows:
+        assert sum(probs) == 1
+        low, high, iters = F(0), probs[0], 0
+        while True:                  # sampling.cuh:171-217
+            iters += 1
+            mid = (low + high) / 2
+            n = mid.numerator
+            assert n.bit_length() <= 8 and mid.denominator & (mid.denominator - 1) == 0
+            s = sum(x for x in probs if x > mid)
+            a = min([high] + [x for x in probs if x > low])
+            b = max([low] + [x for x in probs if x <= high])
+            if s >= p:
+                low = mid
+            else:
+                high = min(mid, b)
+            if b - a <= F(1, 100000):
+                break
+        out.append({"probs": [float(x) for x in probs], "mask": [1 if x > low else 0 for x in probs],
+                    "low": float(low), "iterations": iters})
+    return {"source": "csrc/include/sampling.cuh:156-231 followed in exact rational arithmetic",
+            "p": float(p), "rows": out}
+
+
 def gemv_constant():
     return {"source": "benchmark/efficiency/bench_gemv.py:390-422", "q": 1.0, "nibble": 3,
             "scale": 1.0, "zero": 0.0, "head_dim": 128, "raw_score": 3 * 128}
@@ -74,7 +110,7 @@ def gemv_constant():
 
 if __name__ == "__main__":
     out = {"int4_quant": int4_quant(), "top_p_figure": top_p_figure(), "top_p_trace": top_p_trace(),
-           "gemv_constant": gemv_constant()}
+           "top_p_dyadic": top_p_dyadic(), "gemv_constant": gemv_constant()}
     path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "known_answers.json")
     with open(path, "w") as f:
         json.dump(out, f, indent=1)

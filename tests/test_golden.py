@@ -23,6 +23,7 @@ def test_fixture_file_is_what_the_generator_writes():
     spec.loader.exec_module(m)
     assert m.int4_quant() == KA["int4_quant"] and m.top_p_figure() == KA["top_p_figure"]
     assert m.top_p_trace() == KA["top_p_trace"] and m.gemv_constant() == KA["gemv_constant"]
+    assert m.top_p_dyadic() == KA["top_p_dyadic"]
 
 
 def test_oracle_quantiser_on_the_reference_vector():
@@ -45,6 +46,23 @@ def test_oracle_top_p_on_the_figure_and_the_hand_trace():
     assert mask[0].tolist() == tr["mask"] and iters[0] == tr["iterations"] and low[0] == np.float32(tr["low"])
 
 
+def test_oracle_top_p_on_the_dyadic_rows_in_every_width():
+    # exact in fp32, fp16 and bf16: the one known answer for the 16-bit restatement
+    dy = KA["top_p_dyadic"]
+    for r in dy["rows"]:
+        pr = np.array([r["probs"]], np.float32)
+        for mode in (native.HIGH_FIRST, native.HIGH_MAX):
+            mask, low, iters = native.top_p_mask_f32(pr, dy["p"], mode)
+            assert mask[0].tolist() == r["mask"] and low[0] == np.float32(r["low"])
+            assert iters[0] == r["iterations"]
+            bits16 = pr.astype(np.float16).view(np.uint16)
+            bitsbf = (pr.view(np.uint32) >> 16).astype(np.uint16)          # exact: dyadic values
+            for bits, code in ((bits16, 0), (bitsbf, 1)):
+                m16, low16, it16 = native.top_p_mask_f16(bits, code, dy["p"], mode)
+                assert m16[0].tolist() == r["mask"] and float(low16[0]) == r["low"]
+                assert it16[0] == r["iterations"]
+
+
 def test_oracle_estimator_on_the_constant_inputs():
     c = KA["gemv_constant"]
     deq = native.int4_dequant(np.full((1, c["head_dim"]), c["nibble"], np.uint8),
@@ -65,6 +83,23 @@ def test_hip_top_p_on_the_figure_and_the_hand_trace(dev):
     tr = KA["top_p_trace"]                                  # token 0 is the maximum: both bounds agree
     pr = torch.tensor(tr["probs"], dtype=torch.float32, device=dev).reshape(1, 1, 1, -1)
     assert K.top_p_fp32_return_mask(pr, tr["p"])[0, 0, 0].int().tolist() == tr["mask"]
+
+
+@pytest.mark.gpu
+def test_hip_top_p_on_the_dyadic_rows_in_every_width(dev):
+    import twilight_amd.kernel as K
+    dy = KA["top_p_dyadic"]
+    pr = torch.tensor([r["probs"] for r in dy["rows"]], dtype=torch.float32, device=dev)
+    pr = pr.reshape(1, len(dy["rows"]), 1, -1)
+    want = torch.tensor([r["mask"] for r in dy["rows"]], dtype=torch.bool)
+    for high in ("first", "max"):
+        assert torch.equal(K.top_p_fp32_return_mask(pr, dy["p"], high=high)[0, :, 0].cpu(), want)
+        idx, count, low, iters = K.top_p_select(pr, dy["p"], high=high, return_stats=True)
+        assert low.flatten().tolist() == [r["low"] for r in dy["rows"]]
+        assert iters.flatten().tolist() == [r["iterations"] for r in dy["rows"]]
+        for dt in (torch.float16, torch.bfloat16):
+            m16 = K.top_p_fp16_return_mask(pr.to(dt), dy["p"], high=high)
+            assert torch.equal(m16[0, :, 0].cpu(), want)
 
 
 @pytest.mark.gpu
