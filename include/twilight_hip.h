@@ -65,7 +65,8 @@ enum twl_status {
   TWL_EDTYPE = -3,   /* unsupported element type code */
   TWL_EALIGN = -4,   /* a pointer or stride breaks the alignment the kernel needs */
   TWL_ELAUNCH = -5,  /* the HIP runtime rejected the launch (hipGetLastError != hipSuccess) */
-  TWL_ENODEVICE = -6 /* no usable HIP device */
+  TWL_ENODEVICE = -6, /* no usable HIP device */
+  TWL_ETOOBIG = -7    /* the problem does not fit a fixed-size buffer of the library */
 };
 
 enum twl_dtype { TWL_F16 = 0, TWL_BF16 = 1, TWL_F32 = 2 };
@@ -79,7 +80,7 @@ enum twl_top_p_high {
 const char* twl_strerror(int status);
 /* ABI version of this header; bumps when a signature changes. twl_abi_version() returns the
  * version the library was built with: a caller compares the two before anything else. */
-#define TWL_ABI_VERSION 7
+#define TWL_ABI_VERSION 8
 int twl_abi_version(void);
 /* Number of HIP devices visible, or a negative twl_status. */
 int twl_device_count(void);
@@ -245,6 +246,24 @@ int twl_sparse_attn(const void* q, void* out, int dtype, const void* k_cache, co
                     const int32_t* kv_page_indices, const int32_t* kv_page_indptr, uint32_t batch,
                     uint32_t num_q_heads, uint32_t num_kv_heads, float sm_scale, float* lse_out,
                     void* workspace, uint64_t workspace_bytes, void* stream);
+/* twl_sparse_attn for callers that cannot allocate (code under HIP graph capture, serving loops
+ * and harnesses that forbid hipMalloc, callers with no workspace to bring). It has no counterpart
+ * in the reference. Same arguments and results as twl_sparse_attn without the workspace: the
+ * split-row partial results and tickets live in an array of TWL_STATIC_SCRATCH_BYTES bytes that is
+ * part of the library's device image (every GPU the library runs on holds it until the process
+ * ends). The call allocates and frees nothing. Returns TWL_ETOOBIG when
+ * twl_sparse_attn_workspace_bytes(batch * num_q_heads, idx_stride) exceeds that size (24 MiB hold
+ * 512 rows of up to 8192 survivors). The first call on a device looks up the array's address
+ * there and should happen outside graph capture. All calls on one GPU share the array: calls that
+ * overlap in time on one GPU (two streams, two threads) race; the ticket words are cleared by a
+ * small kernel on `stream` ahead of the attention kernel. */
+#define TWL_STATIC_SCRATCH_BYTES (24u << 20)
+int twl_sparse_attn_static(const void* q, void* out, int dtype, const void* k_cache,
+                           const void* v_cache, uint64_t page_stride, uint64_t token_stride,
+                           uint64_t head_stride, const int32_t* idx, uint32_t idx_stride,
+                           const int32_t* count, const int32_t* kv_page_indices,
+                           const int32_t* kv_page_indptr, uint32_t batch, uint32_t num_q_heads,
+                           uint32_t num_kv_heads, float sm_scale, float* lse_out, void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Paged decode attention with ONE token list per (request, kv head), shared by the kv head's

@@ -20,7 +20,7 @@ def test_header_symbols_are_exported(hip_lib):
     assert declared == set(_lib.EXPORTS)
     for name in declared:
         assert hasattr(hip_lib, name), name
-    assert hip_lib.twl_abi_version() == int(re.search(r"#define TWL_ABI_VERSION (\d+)", hdr).group(1)) == 7
+    assert hip_lib.twl_abi_version() == int(re.search(r"#define TWL_ABI_VERSION (\d+)", hdr).group(1)) == _lib.ABI_VERSION
 
 
 def test_header_compiles_as_c():
@@ -49,7 +49,7 @@ def test_layer_struct_matches_header(hip_lib):
 
 def test_strerror(hip_lib):
     assert _lib.strerror(0) == "ok"
-    for rc in range(-6, 0):
+    for rc in range(-7, 0):
         assert _lib.strerror(rc) and "unknown" not in _lib.strerror(rc)
     assert "unknown" in _lib.strerror(-99)
 
@@ -85,6 +85,14 @@ def test_c_level_validation_without_gpu(hip_lib):
                              1, 1, 1, 1.0, 0, fake, ws - 1, 0) == -2      # workspace too small
     assert L.twl_sparse_attn(fake, fake, 0, fake, fake, 4096, 256, 128, fake, 8, fake, fake, fake,
                              1, 1, 1, 1.0, 0, 0, ws, 0) == -1             # workspace NULL
+    # the entry without a workspace argument: same checks, and a size limit (24 MiB of partials)
+    assert L.twl_sparse_attn_static(fake, fake, 0, fake, fake, 4096, 256, 128, 0, 8, fake, fake,
+                                    fake, 1, 1, 1, 1.0, 0, 0) == -1
+    assert L.twl_sparse_attn_static(fake, fake, 0, fake, fake, 4096, 256, 130, fake, 8, fake, fake,
+                                    fake, 1, 1, 1, 1.0, 0, 0) == -4
+    assert L.twl_sparse_attn_workspace_bytes(512, 8192) <= _lib.STATIC_SCRATCH_BYTES
+    assert L.twl_sparse_attn_static(fake, fake, 0, fake, fake, 4096, 256, 128, fake, 8192, fake,
+                                    fake, fake, 128, 32, 32, 1.0, 0, 0) == -7   # 4096 rows: too big
     assert L.twl_quest_select(fake, 0, fake, fake, fake, 1, 1, 1, 0, 4, fake, 4, fake, fake, 4, 0) == -2
     assert L.twl_quest_select(fake, 0, fake, fake, fake, 1, 1, 1, 64, 4, fake, 2, fake, fake, 4, 0) == -2
     assert L.twl_quest_select(fake, 0, fake, fake, fake, 1, 1, 1, 64, 4, 0, 4, fake, fake, 4, 0) == -1

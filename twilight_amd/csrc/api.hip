@@ -11,6 +11,7 @@ extern "C" const char* twl_strerror(int status) {
     case TWL_EALIGN: return "pointer or stride alignment not supported";
     case TWL_ELAUNCH: return "HIP kernel launch failed";
     case TWL_ENODEVICE: return "no usable HIP device";
+    case TWL_ETOOBIG: return "the problem does not fit a fixed-size buffer of the library";
     default: return "unknown twl_status";
   }
 }

@@ -17,6 +17,8 @@
 //     that finishes last (ticket counter) merges them FlashDecoding-style. There the weights
 //     stay in fp32 (no intermediate rounding to the q dtype): the difference is below the output
 //     rounding.
+#include <atomic>
+
 #include "twl_common.h"
 
 namespace twl {
@@ -319,29 +321,15 @@ extern "C" uint64_t twl_sparse_attn_workspace_bytes(uint32_t rows, uint32_t idx_
   return tickets + (uint64_t)rows * splits * twl::kAttnPartial * sizeof(float);
 }
 
-extern "C" int twl_sparse_attn(const void* q, void* out, int dtype, const void* k_cache,
-                               const void* v_cache, uint64_t page_stride, uint64_t token_stride,
-                               uint64_t head_stride, const int32_t* idx, uint32_t idx_stride,
-                               const int32_t* count, const int32_t* kv_page_indices,
-                               const int32_t* kv_page_indptr, uint32_t batch,
-                               uint32_t num_q_heads, uint32_t num_kv_heads, float sm_scale,
-                               float* lse_out, void* workspace, uint64_t workspace_bytes,
-                               void* stream) {
-  if (!q || !out || !k_cache || !v_cache || !idx || !count || !kv_page_indices ||
-      !kv_page_indptr || !workspace)
-    return TWL_ENULL;
-  if (dtype != TWL_F16 && dtype != TWL_BF16) return TWL_EDTYPE;
-  if (batch == 0 || num_q_heads == 0 || num_kv_heads == 0 || num_q_heads % num_kv_heads != 0)
-    return TWL_EINVAL;
-  if (idx_stride == 0 || idx_stride > TWL_MAX_CANDIDATES) return TWL_EINVAL;
-  const uint64_t rows64 = (uint64_t)batch * num_q_heads;
-  if (rows64 > 65535u) return TWL_EINVAL;
-  const uint32_t rows = (uint32_t)rows64;
-  if (workspace_bytes < twl_sparse_attn_workspace_bytes(rows, idx_stride)) return TWL_EINVAL;
-  if ((page_stride | token_stride | head_stride) & 7u) return TWL_EALIGN;  // 16-byte loads
-  if ((((uintptr_t)q) & 15u) || (((uintptr_t)k_cache) & 15u) || (((uintptr_t)v_cache) & 15u) ||
-      (((uintptr_t)out) & 1u) || (((uintptr_t)workspace) & 255u))
-    return TWL_EALIGN;
+// Validation and launch shared by the two entry points; `workspace` holds
+// twl_sparse_attn_workspace_bytes(rows, idx_stride) bytes whose ticket words are zero.
+static int launch_sparse_attn(const void* q, void* out, int dtype, const void* k_cache,
+                              const void* v_cache, uint64_t page_stride, uint64_t token_stride,
+                              uint64_t head_stride, const int32_t* idx, uint32_t idx_stride,
+                              const int32_t* count, const int32_t* kv_page_indices,
+                              const int32_t* kv_page_indptr, uint32_t rows, uint32_t num_q_heads,
+                              uint32_t num_kv_heads, float sm_scale, float* lse_out,
+                              void* workspace, hipStream_t stream) {
   twl::AttnArgs a{};
   a.q = q; a.out = out; a.k_cache = k_cache; a.v_cache = v_cache; a.page_stride = page_stride;
   a.token_stride = token_stride; a.head_stride = head_stride; a.idx = idx;
@@ -359,9 +347,110 @@ extern "C" int twl_sparse_attn(const void* q, void* out, int dtype, const void* 
   dim3 grid(rows + a.pool);
   if (dtype == TWL_F16)
     hipLaunchKernelGGL((twl::sparse_attn_kernel<TWL_F16>), grid, dim3(twl::kAttnThreads), 0,
-                       (hipStream_t)stream, a);
+                       stream, a);
   else
     hipLaunchKernelGGL((twl::sparse_attn_kernel<TWL_BF16>), grid, dim3(twl::kAttnThreads), 0,
-                       (hipStream_t)stream, a);
+                       stream, a);
   return hipGetLastError() == hipSuccess ? TWL_OK : TWL_ELAUNCH;
+}
+
+// Everything of the argument check that does not concern the workspace. Sets *rows_out.
+static int check_sparse_attn(const void* q, const void* out, int dtype, const void* k_cache,
+                             const void* v_cache, uint64_t page_stride, uint64_t token_stride,
+                             uint64_t head_stride, const int32_t* idx, uint32_t idx_stride,
+                             const int32_t* count, const int32_t* kv_page_indices,
+                             const int32_t* kv_page_indptr, uint32_t batch, uint32_t num_q_heads,
+                             uint32_t num_kv_heads, uint32_t* rows_out) {
+  if (!q || !out || !k_cache || !v_cache || !idx || !count || !kv_page_indices || !kv_page_indptr)
+    return TWL_ENULL;
+  if (dtype != TWL_F16 && dtype != TWL_BF16) return TWL_EDTYPE;
+  if (batch == 0 || num_q_heads == 0 || num_kv_heads == 0 || num_q_heads % num_kv_heads != 0)
+    return TWL_EINVAL;
+  if (idx_stride == 0 || idx_stride > TWL_MAX_CANDIDATES) return TWL_EINVAL;
+  const uint64_t rows64 = (uint64_t)batch * num_q_heads;
+  if (rows64 > 65535u) return TWL_EINVAL;
+  if ((page_stride | token_stride | head_stride) & 7u) return TWL_EALIGN;  // 16-byte loads
+  if ((((uintptr_t)q) & 15u) || (((uintptr_t)k_cache) & 15u) || (((uintptr_t)v_cache) & 15u) ||
+      (((uintptr_t)out) & 1u))
+    return TWL_EALIGN;
+  *rows_out = (uint32_t)rows64;
+  return TWL_OK;
+}
+
+extern "C" int twl_sparse_attn(const void* q, void* out, int dtype, const void* k_cache,
+                               const void* v_cache, uint64_t page_stride, uint64_t token_stride,
+                               uint64_t head_stride, const int32_t* idx, uint32_t idx_stride,
+                               const int32_t* count, const int32_t* kv_page_indices,
+                               const int32_t* kv_page_indptr, uint32_t batch,
+                               uint32_t num_q_heads, uint32_t num_kv_heads, float sm_scale,
+                               float* lse_out, void* workspace, uint64_t workspace_bytes,
+                               void* stream) {
+  if (!workspace) return TWL_ENULL;
+  uint32_t rows = 0;
+  const int rc = check_sparse_attn(q, out, dtype, k_cache, v_cache, page_stride, token_stride,
+                                   head_stride, idx, idx_stride, count, kv_page_indices,
+                                   kv_page_indptr, batch, num_q_heads, num_kv_heads, &rows);
+  if (rc != TWL_OK) return rc;
+  if (workspace_bytes < twl_sparse_attn_workspace_bytes(rows, idx_stride)) return TWL_EINVAL;
+  if (((uintptr_t)workspace) & 255u) return TWL_EALIGN;
+  return launch_sparse_attn(q, out, dtype, k_cache, v_cache, page_stride, token_stride,
+                            head_stride, idx, idx_stride, count, kv_page_indices, kv_page_indptr,
+                            rows, num_q_heads, num_kv_heads, sm_scale, lse_out, workspace,
+                            (hipStream_t)stream);
+}
+
+// ---- the same call without a workspace argument -------------------------------------------------
+// The split-row partials and tickets live in an array that is part of the library's device image,
+// so the call allocates nothing. Every GPU holds its own copy of the array at its own address;
+// host code may not use the array's name as an address (it is a host-side stand-in), so the device
+// address is looked up once per device and kept.
+static __device__ __align__(256) unsigned char scratch[TWL_STATIC_SCRATCH_BYTES];
+
+namespace twl {
+constexpr int kMaxDevices = 64;
+static std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+__global__ void zero_words_kernel(int32_t* p, uint32_t n) {
+  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0;
+}
+}  // namespace twl
+
+extern "C" int twl_sparse_attn_static(const void* q, void* out, int dtype, const void* k_cache,
+                                      const void* v_cache, uint64_t page_stride,
+                                      uint64_t token_stride, uint64_t head_stride,
+                                      const int32_t* idx, uint32_t idx_stride,
+                                      const int32_t* count, const int32_t* kv_page_indices,
+                                      const int32_t* kv_page_indptr, uint32_t batch,
+                                      uint32_t num_q_heads, uint32_t num_kv_heads, float sm_scale,
+                                      float* lse_out, void* stream) {
+  uint32_t rows = 0;
+  const int rc = check_sparse_attn(q, out, dtype, k_cache, v_cache, page_stride, token_stride,
+                                   head_stride, idx, idx_stride, count, kv_page_indices,
+                                   kv_page_indptr, batch, num_q_heads, num_kv_heads, &rows);
+  if (rc != TWL_OK) return rc;
+  // rows * ceil(idx_stride / 128) partial results of 520 bytes must fit the array
+  if (twl_sparse_attn_workspace_bytes(rows, idx_stride) > (uint64_t)TWL_STATIC_SCRATCH_BYTES)
+    return TWL_ETOOBIG;
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess) return TWL_ENODEVICE;
+  if (dev < 0 || dev >= twl::kMaxDevices) return TWL_EINVAL;
+  void* ws = twl::g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!ws) {
+    // first call on this device (it is the current one): the array's address on THIS GPU
+    void* p = nullptr;
+    if (hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch)) != hipSuccess || !p)
+      return TWL_ELAUNCH;
+    twl::g_scratch_ptr[dev].store(p, std::memory_order_release);
+    ws = p;
+  }
+  // The array keeps what the last call left. The ticket words must start at zero: a fill kernel,
+  // not a memset node, so that the call can be recorded into a graph.
+  hipLaunchKernelGGL(twl::zero_words_kernel, dim3((rows + 255) / 256), dim3(256), 0,
+                     (hipStream_t)stream, (int32_t*)ws, rows);
+  if (hipGetLastError() != hipSuccess) return TWL_ELAUNCH;
+  return launch_sparse_attn(q, out, dtype, k_cache, v_cache, page_stride, token_stride,
+                            head_stride, idx, idx_stride, count, kv_page_indices, kv_page_indptr,
+                            rows, num_q_heads, num_kv_heads, sm_scale, lse_out, ws,
+                            (hipStream_t)stream);
 }

@@ -34,7 +34,8 @@ def sparse_paged_decode_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cach
                                   kv_page_indices: torch.Tensor, kv_page_indptr: torch.Tensor,
                                   sm_scale: Optional[float] = None, return_lse: bool = False,
                                   out: Optional[torch.Tensor] = None,
-                                  workspace: Optional[torch.Tensor] = None):
+                                  workspace: Optional[torch.Tensor] = None,
+                                  static_scratch: bool = False):
     """Exact softmax attention of one decode token restricted to per-row survivor lists.
 
     ``q`` [B,H,128] fp16/bf16; ``k_cache`` / ``v_cache`` [pages,16,Hkv,128] of the same dtype;
@@ -43,7 +44,10 @@ def sparse_paged_decode_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cach
     to q's dtype before the V product as at attention.py:302-304 (rows of more than 128 survivors
     are split over workgroups and merged in fp32 instead). ``workspace`` is a zero-initialised
     uint8 tensor of :func:`attention_workspace_bytes` bytes that calls on one stream may share;
-    by default a fresh one is allocated.
+    by default a fresh one is allocated. With ``static_scratch`` (and ``out`` given, ``return_lse``
+    off) the call allocates nothing: the split rows meet in a buffer inside the library
+    (``twl_sparse_attn_static``), shared by every such call on the GPU, so those calls must not
+    overlap in time; shapes beyond its 24 MiB raise.
     """
     check_input(q, "q")
     check_dim(3, q, "q")
@@ -80,6 +84,15 @@ def sparse_paged_decode_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cach
                 raise RuntimeError("out must match q")
         lse = torch.empty((B, H), dtype=torch.float32, device=dev) if return_lse else None
         scale = 1.0 / math.sqrt(D) if sm_scale is None else float(sm_scale)
+        if static_scratch:
+            if workspace is not None:
+                raise RuntimeError("static_scratch and workspace exclude each other")
+            rc = _lib.lib().twl_sparse_attn_static(
+                ptr(q), ptr(out), dtype_code(q.dtype, "q"), ptr(k_cache), ptr(v_cache), ks[0],
+                ks[1], ks[2], ptr(idx), idx.size(2), ptr(count), ptr(kv_page_indices),
+                ptr(kv_page_indptr), B, H, Hkv, scale, ptr(lse), stream_of(q))
+            _lib.check(rc, "SparsePagedDecodeAttention")
+            return (out, lse) if return_lse else out
         need = attention_workspace_bytes(B * H, idx.size(2))
         if workspace is None:
             workspace = torch.zeros(need, dtype=torch.uint8, device=dev)
