@@ -101,9 +101,15 @@ int twl_device_count(void);
 int twl_top_p_f32(const float* probs, uint8_t* mask, int32_t* idx, int32_t* count,
                   const float* p_arr, float p, uint32_t rows, uint32_t d, uint32_t idx_stride,
                   int high_mode, float* low_out, int32_t* iters_out, void* stream);
-/* Same for fp16 (dtype = TWL_F16) or bf16 (TWL_BF16) probabilities; the bisection runs in that
- * type's value set (pivots are rounded to it each iteration) like the reference's DType template
- * (sampling.cuh:156-217 with DType = half / nv_bfloat16). */
+/* Same for fp16 (dtype = TWL_F16) or bf16 (TWL_BF16) probabilities, with the arithmetic of the
+ * reference's DType = half / nv_bfloat16 instantiation (csrc/src/sampling.cu:22-43): p, low, high,
+ * mid, the tolerance 1e-5, the bracket width and every partial sum are values of the 16-bit type
+ * (each operation rounds to nearest even), and the additions run in the order of
+ * cub::BlockReduce<DType, 1024, BLOCK_REDUCE_WARP_REDUCTIONS> (sampling.cuh:54,171-217: a thread
+ * folds its VEC = gcd(8, d) items left to right, warps of 32 add pairwise, the 32 warp results
+ * are added in warp order, chunks of 1024 * VEC elements in chunk order; CUB 1.x - 2.4). Masks,
+ * low_out and iters_out therefore equal the reference kernel's bit for bit. TWL_HIGH_MAX is this
+ * library's variant of the upper bound; everything else is unchanged by it. */
 int twl_top_p_f16(const void* probs, int dtype, uint8_t* mask, int32_t* idx, int32_t* count,
                   const float* p_arr, float p, uint32_t rows, uint32_t d, uint32_t idx_stride,
                   int high_mode, float* low_out, int32_t* iters_out, void* stream);
@@ -180,6 +186,10 @@ int twl_select_estimate_prune(const void* q, int dtype, const void* meta, const 
  * ftka.cuda_ops.gemv.batched_sparse_gemv_int4_k whose call site is
  * benchmark/efficiency/bench_gemv.py:445-454.
  * q [batch, num_q_heads, 128] in q_dtype (TWL_F16 or TWL_BF16); k_int4 = the INT4 shadow records.
+ * The dot products run on fp16 pairs with fp32 accumulation, so a bf16 q is converted to fp16
+ * first (here, in twl_gemv_top_p, twl_select_estimate_prune and twl_decode_layer's estimator):
+ * exact for 2^-17 <= |q| <= 65504, rounded to a multiple of 2^-24 below, saturated to +-65504
+ * above. Accepted range of q for results within the 1e-3 score tolerance: |q| <= 65504.
  * out fp32 [rows, out_stride]; candidates past the request's length get -inf. sel_count (nullable
  * with sel_pages) gives pages per row; out_count (nullable) int32 [rows] receives the number of
  * candidate slots written (pages * 16).

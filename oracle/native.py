@@ -40,9 +40,13 @@ def lib() -> ctypes.CDLL:
         L.twl_oracle_top_p_f32.argtypes = [f32p, u8p, f32p, ctypes.c_float, ctypes.c_uint32,
                                            ctypes.c_uint32, ctypes.c_int, f32p, i32p, f32p]
         L.twl_oracle_top_p_f32.restype = None
-        L.twl_oracle_top_p_f16.argtypes = [u16p, ctypes.c_int, u8p, f32p, ctypes.c_float,
-                                           ctypes.c_uint32, ctypes.c_uint32, ctypes.c_int, f32p, i32p, f32p]
-        L.twl_oracle_top_p_f16.restype = None
+        L.twl_oracle_top_p_cub.argtypes = [ctypes.c_void_p, ctypes.c_int, u8p, f32p, ctypes.c_float,
+                                           ctypes.c_uint32, ctypes.c_uint32, ctypes.c_int, f32p, i32p]
+        L.twl_oracle_top_p_cub.restype = None
+        L.twl_oracle_dt_add.argtypes = [ctypes.c_double, ctypes.c_double, ctypes.c_int]
+        L.twl_oracle_dt_add.restype = ctypes.c_double
+        L.twl_oracle_dt_round.argtypes = [ctypes.c_double, ctypes.c_int]
+        L.twl_oracle_dt_round.restype = ctypes.c_double
         L.twl_oracle_nucleus.argtypes = [f32p, ctypes.c_uint32, ctypes.c_double, u8p, f32p,
                                          ctypes.POINTER(ctypes.c_double)]
         L.twl_oracle_nucleus.restype = ctypes.c_uint32
@@ -97,10 +101,19 @@ def top_p_mask_f32(probs: np.ndarray, p, high_mode: int = HIGH_FIRST, return_mar
     return mask, low, iters
 
 
-def top_p_mask_f16(bits: np.ndarray, dtype: int, p, high_mode: int = HIGH_FIRST):
-    """Same bisection with 16-bit pivots; ``bits`` is the uint16 view of fp16 (dtype 0) or bf16 (1)."""
-    bits = np.ascontiguousarray(bits, dtype=np.uint16)
-    rows, d = bits.shape
+DT_F16, DT_BF16, DT_F32 = 0, 1, 2
+
+
+def top_p_mask_cub(values: np.ndarray, dtype: int, p, high_mode: int = HIGH_FIRST):
+    """``TopPReturnMaskKernel`` with every operation in its element type and the additions in the
+    order of ``cub::BlockReduce`` (csrc/include/sampling.cuh:54,119-231; csrc/src/sampling.cu:22-63).
+
+    ``values`` [rows, d]: the uint16 view of fp16 (``dtype`` 0) or bf16 (1) probabilities, or
+    float32 (2). Returns ``(mask uint8 [rows,d], low float32 [rows], iters int32 [rows])``; for
+    this function the result is exact, there is no margin.
+    """
+    values = np.ascontiguousarray(values, dtype=np.float32 if dtype == DT_F32 else np.uint16)
+    rows, d = values.shape
     mask = np.zeros((rows, d), dtype=np.uint8)
     low = np.zeros(rows, dtype=np.float32)
     iters = np.zeros(rows, dtype=np.int32)
@@ -109,10 +122,19 @@ def top_p_mask_f16(bits: np.ndarray, dtype: int, p, high_mode: int = HIGH_FIRST)
         pp, pv = _ptr(p_arr, ctypes.c_float), 0.0
     else:
         pp, pv = None, float(p)
-    lib().twl_oracle_top_p_f16(_ptr(bits, ctypes.c_uint16), int(dtype), _ptr(mask, ctypes.c_uint8),
-                               pp, pv, rows, d, int(high_mode), _ptr(low, ctypes.c_float),
-                               _ptr(iters, ctypes.c_int32), None)
+    lib().twl_oracle_top_p_cub(values.ctypes.data_as(ctypes.c_void_p), int(dtype),
+                               _ptr(mask, ctypes.c_uint8), pp, pv, rows, d, int(high_mode),
+                               _ptr(low, ctypes.c_float), _ptr(iters, ctypes.c_int32))
     return mask, low, iters
+
+
+def dt_add(a: float, b: float, dtype: int) -> float:
+    """One addition in the element type (round to nearest even), as the oracle performs it."""
+    return float(lib().twl_oracle_dt_add(float(a), float(b), int(dtype)))
+
+
+def dt_round(x: float, dtype: int) -> float:
+    return float(lib().twl_oracle_dt_round(float(x), int(dtype)))
 
 
 def nucleus(probs_row: np.ndarray, p: float):

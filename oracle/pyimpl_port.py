@@ -228,18 +228,23 @@ def masked_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: to
 def decode_layer_dense(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, top_p: float,
                        token_budget: Optional[int] = None, chunk_size: int = PAGE,
                        high_mode: int = native.HIGH_MAX, quant: str = "storage",
-                       prob_dtype: torch.dtype = torch.float32, k_deq: Optional[torch.Tensor] = None):
+                       prob_dtype: torch.dtype = torch.float32, k_deq: Optional[torch.Tensor] = None,
+                       mask0: Optional[torch.Tensor] = None):
     """twilight/pyimpl/attention.py:188-306 for one decode step.
 
     q [B,H,1,D], k/v [B,H,N,D] (K already repeated per q head, attention.py:124-126).
     ``quant``: "storage" = group 32 + fp16 scale/zero (this build's estimator), "ref128" = the
     reference's whole-head_dim group in fp32 (quantize.py:4-13 as called at attention.py:247-251).
     ``k_deq`` may carry a pre-dequantised K (variant B of the CPU baseline: quantise on append).
+    ``mask0`` bool [B,H,1,N] replaces the selector's result (tests use it to follow the later
+    stages on a selection that differs from the oracle's only by pages tied at the k-th score).
     Returns dict(scores, mask0, probs, pruned, mask, out, low, iters).
     """
     B, H, _, D = q.shape
     N = k.shape[-2]
-    if token_budget is None:
+    if mask0 is not None:
+        assert mask0.shape == (B, H, 1, N) and mask0.dtype == torch.bool
+    elif token_budget is None:
         mask0 = torch.ones((B, H, 1, N), dtype=torch.bool)                    # attention.py:198-199
     else:
         mask0, _ = quest_selector_dense(q.float(), k.float(), chunk_size, token_budget)

@@ -7,12 +7,10 @@
  * What is restated, and from where:
  *   twl_oracle_top_p_f32   csrc/include/sampling.cuh:156-231 (TopPReturnMaskKernel after its dead
  *                          max pass :135-155), rows/cols as csrc/src/sampling.cu:51-60
- *   twl_oracle_top_p_f16   the same kernel instantiated with a 16-bit DType (sampling.cu:22-43);
- *                          pivots live in the 16-bit type, the partial sums are kept in fp32
- *                          (the reference sums in the 16-bit type, in an order fixed by CUB's
- *                          block reduction, which a sequential restatement cannot reproduce:
- *                          PARITY UNPINNED for the 16-bit entry, except on rows whose sums and
- *                          midpoints are exact in every width, tests/golden "top_p_dyadic")
+ *   twl_oracle_top_p_cub   the same kernel with every operation in its element type (half,
+ *                          nv_bfloat16 or float: sampling.cu:22-63) and the additions in the
+ *                          order of cub::BlockReduce<.., BLOCK_REDUCE_WARP_REDUCTIONS>
+ *                          (sampling.cuh:54); see the comment above the function
  *   twl_oracle_nucleus     textbook nucleus set (sort descending, cumulative sum in fp64):
  *                          the mathematical definition the bisection approximates
  *   twl_oracle_int4_quant  twilight/pyimpl/quantize.py:4-13 applied per group, with the fp16
@@ -20,12 +18,17 @@
  *   twl_oracle_int4_dequant  nibble * scale + zero, one fp32 rounding
  *
  * Pinning (see tests/test_oracle_*.py): top-p against twl_oracle_nucleus + brute force over all
- * subsets for d <= 12 + degenerate rows; quant against the known-answer vector of
+ * subsets for d <= 12 + degenerate rows; twl_oracle_top_p_cub against rows followed in exact
+ * rational arithmetic with explicit round-to-nearest-even (tests/golden "top_p_cub_order": sums
+ * whose order decides, midpoints and widths that are not representable, a subnormal halving;
+ * each row is checked to come out differently under fp32 sums, a left-to-right sum and an
+ * unrounded midpoint), and its fp32 form against twl_oracle_top_p_f32 wherever the margin allows; quant against the known-answer vector of
  * twilight/pyimpl/quantize.py:30-48 evaluated by hand, min/max reproduction and |err| <= scale/2.
  *
- * Block sums: the reference adds fp32 values in a tree order chosen by cub::BlockReduce. Any
- * order is a valid fp32 evaluation of the same sum; this file accumulates in fp64 and rounds once,
- * which is within an ulp or two of every such order.
+ * Block sums of twl_oracle_top_p_f32: the reference adds fp32 values in the order of
+ * cub::BlockReduce; this function accumulates in fp64 and rounds once, which is within an ulp or
+ * two of every order, and reports how close each decision came (margin). twl_oracle_top_p_cub
+ * follows CUB's order itself.
  */
 #include <math.h>
 #include <stdint.h>
@@ -110,19 +113,11 @@ uint16_t twl_oracle_f32_to_f16(float f) { return f32_to_f16_bits(f); }
 float twl_oracle_f16_to_f32(uint16_t h) { return f16_bits_to_f32(h); }
 uint16_t twl_oracle_f32_to_bf16(float f) { return f32_to_bf16_bits(f); }
 
-/* round a float to the value set of the 16-bit type: 0 = fp16, 1 = bf16, 2 = none (fp32) */
-static float round_to(float v, int dtype) {
-  if (dtype == 0) return f16_bits_to_f32(f32_to_f16_bits(v));
-  if (dtype == 1) return bf16_bits_to_f32(f32_to_bf16_bits(v));
-  return v;
-}
-
 /* ---- top-p bisection ------------------------------------------------------------------------- */
-/* One row of csrc/include/sampling.cuh:156-231. x[] already holds the row as floats (for 16-bit
- * inputs: the exact values of the 16-bit numbers). dtype selects the arithmetic of the pivots. */
-static void top_p_row(const float* x, uint32_t d, float p_in, int high_mode, int dtype,
+/* One fp32 row of csrc/include/sampling.cuh:156-231. */
+static void top_p_row(const float* x, uint32_t d, float p_in, int high_mode,
                       uint8_t* mask, float* low_out, int32_t* iters_out, float* margin_out) {
-  float p = round_to(p_in, dtype); /* DType p = DType(top_p...)            sampling.cuh:125 */
+  float p = p_in;                  /* DType p = DType(top_p...)            sampling.cuh:125 */
   float low = 0.0f;                /*                                       sampling.cuh:159 */
   float high;
   if (high_mode == 0) {
@@ -131,12 +126,12 @@ static void top_p_row(const float* x, uint32_t d, float p_in, int high_mode, int
     high = 0.0f;                   /* paper Algorithm 1: r = max(W) */
     for (uint32_t j = 0; j < d; ++j) high = x[j] > high ? x[j] : high;
   }
-  const float eps = round_to(1e-5f, dtype); /*                              sampling.cuh:162 */
+  const float eps = 1e-5f;                  /*                              sampling.cuh:162 */
   float min_gt_low, max_le_high;
   int32_t iters = 0;
   double margin = 1e30; /* smallest |S - p| met: how close a decision came to a rounding flip */
   do {                                       /*                             sampling.cuh:171 */
-    float mid = round_to((low + high) / 2.0f, dtype); /*                    sampling.cuh:173 */
+    float mid = (low + high) / 2.0f;                  /*                    sampling.cuh:173 */
     min_gt_low = high;                       /*                             sampling.cuh:174 */
     max_le_high = low;                       /*                             sampling.cuh:175 */
     double sum = 0.0;
@@ -146,7 +141,7 @@ static void top_p_row(const float* x, uint32_t d, float p_in, int high_mode, int
       if (v > low && v < min_gt_low) min_gt_low = v;          /* :184-186 */
       if (v <= high && v > max_le_high) max_le_high = v;      /* :187-189 */
     }
-    float s = (float)sum; /* fp32 partial sums for every dtype */
+    float s = (float)sum;
     if (fabs(sum - (double)p) < margin) margin = fabs(sum - (double)p);
     if (s >= p) {                            /*                             sampling.cuh:211-213 */
       low = mid;
@@ -155,7 +150,7 @@ static void top_p_row(const float* x, uint32_t d, float p_in, int high_mode, int
     }
     ++iters;
     if (iters > 4096) break; /* cannot happen for finite input; guards a NaN row */
-  } while (round_to(max_le_high - min_gt_low, dtype) > eps); /*             sampling.cuh:217 */
+  } while (max_le_high - min_gt_low > eps);                 /*             sampling.cuh:217 */
   if (mask) {
     for (uint32_t j = 0; j < d; ++j) mask[j] = x[j] > low ? 1 : 0; /*       sampling.cuh:219-230 */
   }
@@ -168,27 +163,154 @@ void twl_oracle_top_p_f32(const float* probs, uint8_t* mask, const float* p_arr,
                           uint32_t rows, uint32_t d, int high_mode, float* low_out,
                           int32_t* iters_out, float* margin_out) {
   for (uint32_t r = 0; r < rows; ++r) {
-    top_p_row(probs + (size_t)r * d, d, p_arr ? p_arr[r] : p, high_mode, 2,
+    top_p_row(probs + (size_t)r * d, d, p_arr ? p_arr[r] : p, high_mode,
               mask ? mask + (size_t)r * d : NULL, low_out ? low_out + r : NULL,
               iters_out ? iters_out + r : NULL, margin_out ? margin_out + r : NULL);
   }
 }
 
-/* probs: 16-bit patterns, dtype 0 = fp16, 1 = bf16 */
-void twl_oracle_top_p_f16(const uint16_t* probs, int dtype, uint8_t* mask, const float* p_arr,
-                          float p, uint32_t rows, uint32_t d, int high_mode, float* low_out,
-                          int32_t* iters_out, float* margin_out) {
-  float* x = (float*)malloc(sizeof(float) * (size_t)d);
+/* ---- the same kernel with every operation in its element type and CUB's summation order ------
+ *
+ * TopPReturnMaskKernel<1024, BLOCK_REDUCE_WARP_REDUCTIONS, VEC, DType> (csrc/include/sampling.cuh:
+ * 119-231, instantiated for half / nv_bfloat16 at csrc/src/sampling.cu:22-43 and for float at
+ * :45-63) keeps p, low, high, mid, eps, the running sum and every partial sum in DType. With a
+ * 16-bit DType the order of the additions decides the result, so it is restated here as CUB
+ * publishes it (cub/block/specializations/block_reduce_warp_reductions.cuh,
+ * cub/warp/specializations/warp_reduce_shfl.cuh, cub/thread/thread_reduce.cuh; the form of CUB
+ * 1.x .. 2.4, which covers the CUDA 11.8 - 12.4 toolkits that torch 2.5.0, requirements.txt:1, is
+ * built for; CUB is a dependency of the reference that is absent from its tree):
+ *   - thread t of 1024 owns, in chunk i, the VEC = gcd(16 / sizeof(DType), d) elements starting at
+ *     (i * 1024 + t) * VEC (sampling.cuh:176-181,239-243), zero-filled past d;
+ *   - BlockReduce::Sum<VEC>(items): ThreadReduce folds a thread's items left to right starting
+ *     from item 0; each warp of 32 then runs five shuffle-down steps with offsets 1, 2, 4, 8, 16,
+ *     lane l adding lane l + offset's value when l + offset <= 31; lane 0 of every warp stores
+ *     its aggregate and thread 0 adds the aggregates of warps 1 .. 31 to its own, in that order;
+ *   - the kernel adds each chunk's block sum to threadlocal_sum (sampling.cuh:191-193).
+ * Every addition rounds to nearest even in DType (__hadd for half and nv_bfloat16, one rounding).
+ * mid = (low + high) / DType(2): the sum rounds, then the halving rounds (it only can for a
+ * subnormal half). max_le_high - min_gt_low rounds too; minima, maxima and comparisons are exact.
+ * high_mode 1 (the row maximum) is this build's variant of :156-159; everything else is the same.
+ *
+ * A DType value is carried as a double (every fp16 / bf16 / fp32 value is one exactly). a + b of
+ * two such values is computed in double and rounded to DType: exact-then-round for fp16, and for
+ * bf16 / fp32 a double rounding that cannot change the result (53 >= 2 * 24 + 2 bits).
+ */
+typedef struct { int mant; int emin; double maxv; } fmt_t; /* significand bits incl. the hidden one */
+static const fmt_t kFmt[3] = {
+  {11, -14, 65504.0},                          /* IEEE binary16 */
+  {8, -126, 3.3895313892515355e38},            /* bfloat16 */
+  {24, -126, 3.4028234663852886e38},           /* IEEE binary32 */
+};
+
+static double dt_round(double x, int dtype) {
+  if (x == 0.0 || isnan(x) || isinf(x)) return x;
+  const fmt_t* f = &kFmt[dtype];
+  int e;
+  (void)frexp(fabs(x), &e);      /* |x| in [2^(e-1), 2^e) */
+  int ex = e - 1;
+  if (ex < f->emin) ex = f->emin; /* subnormal: the spacing stops shrinking */
+  const double quantum = ldexp(1.0, ex - (f->mant - 1));
+  const double y = nearbyint(x / quantum) * quantum; /* the division is an exact scaling; RNE */
+  if (fabs(y) > f->maxv) return x > 0 ? INFINITY : -INFINITY;
+  return y;
+}
+static double dt_add(double a, double b, int dtype) {
+  if (b == 0.0) return a; /* exact, and by far the commonest case in a masked sum */
+  if (a == 0.0) return b;
+  return dt_round(a + b, dtype);
+}
+
+#define CUB_BLOCK 1024u
+#define CUB_WARP 32u
+
+static uint32_t gcd_u32(uint32_t a, uint32_t b) { while (b) { uint32_t t = a % b; a = b; b = t; } return a; }
+
+/* cub::BlockReduce<DType, 1024, BLOCK_REDUCE_WARP_REDUCTIONS>::Sum of one value per thread */
+static double cub_block_sum(double* v /* [1024], destroyed */, int dtype) {
+  for (uint32_t off = 1; off < CUB_WARP; off <<= 1)          /* WarpReduceShfl::ReduceStep */
+    for (uint32_t w = 0; w < CUB_BLOCK; w += CUB_WARP)
+      for (uint32_t l = 0; l + off < CUB_WARP; ++l)           /* l + off <= last_lane */
+        v[w + l] = dt_add(v[w + l], v[w + l + off], dtype);   /* lane l + off is still this step's input */
+  double agg = v[0];                                          /* ApplyWarpAggregates, thread 0 */
+  for (uint32_t w = 1; w < CUB_BLOCK / CUB_WARP; ++w) agg = dt_add(agg, v[w * CUB_WARP], dtype);
+  return agg;
+}
+
+static void top_p_row_cub(const double* x, uint32_t d, float p_in, int high_mode, int dtype,
+                          uint8_t* mask, float* low_out, int32_t* iters_out) {
+  const uint32_t vec = gcd_u32(dtype == 2 ? 4u : 8u, d);                 /* sampling.cuh:239 */
+  const uint32_t chunks = (d + CUB_BLOCK * vec - 1) / (CUB_BLOCK * vec); /* sampling.cuh:176 */
+  const double p = dt_round((double)p_in, dtype);                        /* sampling.cuh:125 */
+  double low = 0.0, high;                                                /* sampling.cuh:159 */
+  if (high_mode == 0) {
+    high = x[0];                                                         /* sampling.cuh:156-159 */
+  } else {
+    high = 0.0;
+    for (uint32_t j = 0; j < d; ++j) high = x[j] > high ? x[j] : high;
+  }
+  const double eps = dt_round(1e-5, dtype);                              /* sampling.cuh:162 */
+  double min_gt_low, max_le_high;
+  double part[CUB_BLOCK];
+  int32_t iters = 0;
+  do {                                                                   /* sampling.cuh:171 */
+    double threadlocal_sum = 0.0;                                        /* :172 */
+    const double mid = dt_round(dt_round(low + high, dtype) / 2.0, dtype); /* :173 */
+    min_gt_low = high;                                                   /* :174 */
+    max_le_high = low;                                                   /* :175 */
+    for (uint32_t i = 0; i < chunks; ++i) {                              /* :176 */
+      for (uint32_t t = 0; t < CUB_BLOCK; ++t) {
+        const uint64_t e0 = ((uint64_t)i * CUB_BLOCK + t) * vec;
+        double acc = 0.0;
+        for (uint32_t j = 0; j < vec; ++j) {
+          const double v = (e0 + j < d) ? x[e0 + j] : 0.0;               /* fill(0), :177-180 */
+          const double g = (v > mid) ? v : 0.0;                          /* :183 */
+          acc = (j == 0) ? g : dt_add(acc, g, dtype);                    /* ThreadReduce */
+          if (e0 + j < d) {
+            if (v > low && v < min_gt_low) min_gt_low = v;               /* :184-186 */
+            if (v <= high && v > max_le_high) max_le_high = v;           /* :187-189 */
+          }
+        }
+        part[t] = acc;
+      }
+      threadlocal_sum = dt_add(threadlocal_sum, cub_block_sum(part, dtype), dtype); /* :191-193 */
+    }
+    if (threadlocal_sum >= p) {                                          /* :211-213 */
+      low = mid;
+    } else {                                                             /* :214-216 */
+      high = mid < max_le_high ? mid : max_le_high;
+    }
+    ++iters;
+    if (iters > 4096) break; /* cannot happen for finite input; guards a NaN row */
+  } while (dt_round(max_le_high - min_gt_low, dtype) > eps);             /* :217 */
+  if (mask)
+    for (uint32_t j = 0; j < d; ++j) mask[j] = x[j] > low ? 1 : 0;       /* :219-230 */
+  if (low_out) *low_out = (float)low;
+  if (iters_out) *iters_out = iters;
+}
+
+/* probs: 16-bit patterns (dtype 0 = fp16, 1 = bf16) or floats (dtype 2), [rows, d] */
+void twl_oracle_top_p_cub(const void* probs, int dtype, uint8_t* mask, const float* p_arr, float p,
+                          uint32_t rows, uint32_t d, int high_mode, float* low_out,
+                          int32_t* iters_out) {
+  double* x = (double*)malloc(sizeof(double) * (size_t)d);
   for (uint32_t r = 0; r < rows; ++r) {
-    const uint16_t* src = probs + (size_t)r * d;
-    for (uint32_t j = 0; j < d; ++j)
-      x[j] = dtype == 0 ? f16_bits_to_f32(src[j]) : bf16_bits_to_f32(src[j]);
-    top_p_row(x, d, p_arr ? p_arr[r] : p, high_mode, dtype, mask ? mask + (size_t)r * d : NULL,
-              low_out ? low_out + r : NULL, iters_out ? iters_out + r : NULL,
-              margin_out ? margin_out + r : NULL);
+    for (uint32_t j = 0; j < d; ++j) {
+      if (dtype == 2) {
+        x[j] = (double)((const float*)probs)[(size_t)r * d + j];
+      } else {
+        const uint16_t b = ((const uint16_t*)probs)[(size_t)r * d + j];
+        x[j] = (double)(dtype == 0 ? f16_bits_to_f32(b) : bf16_bits_to_f32(b));
+      }
+    }
+    top_p_row_cub(x, d, p_arr ? p_arr[r] : p, high_mode, dtype, mask ? mask + (size_t)r * d : NULL,
+                  low_out ? low_out + r : NULL, iters_out ? iters_out + r : NULL);
   }
   free(x);
 }
+
+/* one addition / one rounding in the element type, exported so that tests can pin them */
+double twl_oracle_dt_add(double a, double b, int dtype) { return dt_add(a, b, dtype); }
+double twl_oracle_dt_round(double x, int dtype) { return dt_round(x, dtype); }
 
 /* ---- textbook nucleus set -------------------------------------------------------------------- */
 typedef struct { float v; uint32_t i; } vi_t;

@@ -24,6 +24,7 @@ def test_fixture_file_is_what_the_generator_writes():
     assert m.int4_quant() == KA["int4_quant"] and m.top_p_figure() == KA["top_p_figure"]
     assert m.top_p_trace() == KA["top_p_trace"] and m.gemv_constant() == KA["gemv_constant"]
     assert m.top_p_dyadic() == KA["top_p_dyadic"]
+    assert m.top_p_cub_order() == KA["top_p_cub_order"]
 
 
 def test_oracle_quantiser_on_the_reference_vector():
@@ -58,9 +59,41 @@ def test_oracle_top_p_on_the_dyadic_rows_in_every_width():
             bits16 = pr.astype(np.float16).view(np.uint16)
             bitsbf = (pr.view(np.uint32) >> 16).astype(np.uint16)          # exact: dyadic values
             for bits, code in ((bits16, 0), (bitsbf, 1)):
-                m16, low16, it16 = native.top_p_mask_f16(bits, code, dy["p"], mode)
+                m16, low16, it16 = native.top_p_mask_cub(bits, code, dy["p"], mode)
                 assert m16[0].tolist() == r["mask"] and float(low16[0]) == r["low"]
                 assert it16[0] == r["iterations"]
+
+
+def _cub_row(r):
+    """(bits uint16 [1, d], dtype code, high mode) of one ``top_p_cub_order`` fixture row."""
+    bits = np.zeros((1, r["d"]), np.uint16)
+    for i, b in r["nonzero"]:
+        bits[0, i] = b
+    return bits, (0 if r["dtype"] == "f16" else 1), \
+        (native.HIGH_FIRST if r["high"] == "first" else native.HIGH_MAX)
+
+
+def _low_bits(low: float, code: int) -> int:
+    if code == 0:
+        return int(np.float32(low).astype(np.float16).view(np.uint16))
+    return int(np.float32(low).view(np.uint32) >> 16)
+
+
+def test_oracle_top_p_in_16_bit_arithmetic_and_cub_order():
+    # rows followed in exact rational arithmetic with explicit rounding; each one comes out
+    # differently under at least one plausible mistake (see make_fixtures.top_p_cub_order)
+    rows = KA["top_p_cub_order"]["rows"]
+    seen = set()
+    for r in rows:
+        bits, code, mode = _cub_row(r)
+        mask, low, iters = native.top_p_mask_cub(bits, code, r["p"], mode)
+        assert np.nonzero(mask[0])[0].tolist() == r["kept"], (r["dtype"], r["d"])
+        assert _low_bits(low[0], code) == r["low_bits"] and iters[0] == r["iterations"]
+        seen |= {(r["dtype"], a) for a in r["differs_under"]}
+    for fmt in ("f16", "bf16"):
+        for alt in ("exact_sums", "flat_sum", "thread_tree", "warp_tree", "chunks_merged",
+                    "exact_mid", "exact_eps"):
+            assert (fmt, alt) in seen
 
 
 def test_oracle_estimator_on_the_constant_inputs():
@@ -100,6 +133,22 @@ def test_hip_top_p_on_the_dyadic_rows_in_every_width(dev):
         for dt in (torch.float16, torch.bfloat16):
             m16 = K.top_p_fp16_return_mask(pr.to(dt), dy["p"], high=high)
             assert torch.equal(m16[0, :, 0].cpu(), want)
+
+
+@pytest.mark.gpu
+def test_hip_top_p_in_16_bit_arithmetic_and_cub_order(dev):
+    import twilight_amd.kernel as K
+    for r in KA["top_p_cub_order"]["rows"]:
+        bits, code, _ = _cub_row(r)
+        t = torch.from_numpy(bits.view(np.int16)).view(torch.float16 if code == 0 else torch.bfloat16)
+        t = t.reshape(1, 1, 1, -1).to(dev)
+        idx, count, mask, low, iters = K.top_p_select(t, r["p"], high=r["high"], return_mask=True,
+                                                      return_stats=True)
+        kept = torch.nonzero(mask[0, 0, 0]).flatten().tolist()
+        assert kept == r["kept"], (r["dtype"], r["d"], r["differs_under"])
+        assert idx[0, 0, :int(count[0, 0])].tolist() == r["kept"]
+        assert _low_bits(float(low[0]), code) == r["low_bits"] and int(iters[0]) == r["iterations"]
+        assert torch.equal(K.top_p_fp16_return_mask(t, r["p"], high=r["high"]), mask)
 
 
 @pytest.mark.gpu

@@ -90,13 +90,37 @@ def test_gemv_full_context_shuffled_pages(dev, qdt):
     codes, scale, zero = P.unpack_int4_records(rec.numpy())
     deq = native.int4_dequant(codes, scale, zero)            # [P,Hkv,16,128]
     got = out.cpu().numpy()
-    qh = q.to(torch.float16).float() if qdt == torch.bfloat16 else q.float()
+    qh = q.float()                                            # the true q, bf16 included
     for b in range(B):
         phys = ids[indptr[b]:indptr[b + 1]].long().numpy()
         for h in range(H):
             want = _gemv_oracle(qh[b, h], deq[phys, h // 2].reshape(-1, 128), 1 / math.sqrt(128))
             want[(npg - 1) * 16 + 9:] = -np.inf
             assert_scores_close(got[b, h], want)
+
+
+def test_gemv_bf16_query_range(dev):
+    # a bf16 query is converted to fp16 for the dot products: exact from 2^-17 to 65504, tiny
+    # values rounded to multiples of 2^-24, larger ones saturated (finite scores, never NaN)
+    npg = 5
+    rec = synth.int4_records_random(npg, 1, seed=31)
+    ids, indptr, last = synth.identity_page_table(1, npg, last_len=16)
+    codes, scale, zero = P.unpack_int4_records(rec.numpy())
+    deq = native.int4_dequant(codes, scale, zero)[:, 0].reshape(-1, 128)
+    g = torch.Generator().manual_seed(32)
+    base = torch.randn((1, 1, 128), generator=g)
+    for mag, exact in ((1.0, True), (300.0, True), (2.0 ** -15, True), (2.0 ** -21, False), (3e5, False)):
+        q = (base * mag).to(torch.bfloat16)
+        out, _ = K.sparse_gemv_int4(q.to(dev), rec.to(dev), ids.to(dev), indptr.to(dev), last.to(dev),
+                                    max_pages=npg)
+        got = out.cpu().numpy()[0, 0]
+        assert np.isfinite(got).all(), mag
+        # what the kernel is documented to compute: q rounded to fp16 with saturation
+        qk = q.float().clamp(-65504.0, 65504.0).to(torch.float16).float()[0, 0]
+        assert_scores_close(got, _gemv_oracle(qk, deq, 1 / math.sqrt(128)))
+        if exact and mag >= 1.0:   # inside the exact range the true bf16 q gives the same scores
+            assert torch.equal(qk, q.float()[0, 0])
+            assert_scores_close(got, _gemv_oracle(q.float()[0, 0], deq, 1 / math.sqrt(128)))
 
 
 def test_gemv_selected_pages_and_ragged_counts(dev):

@@ -24,6 +24,28 @@ def _lists_to_mask(idx, count, N):
     return m
 
 
+def _pages_to_mask(sel, selc, npg):
+    """Page lists [rows, k] with counts -> bool token mask [rows, npg * 16]."""
+    m = np.zeros((sel.shape[0], npg * 16), dtype=bool)
+    for r in range(sel.shape[0]):
+        for pg in sel[r, :selc[r]]:
+            m[r, pg * 16:(pg + 1) * 16] = True
+    return m
+
+
+def _assert_selection_ties(page_scores, gpu_pages, ora_mask0, npg):
+    """A page on one side of the selection only must score within 1e-3 * max(1, |k-th|) of the
+    oracle's k-th page score (the two top-k sets differ by ties at the boundary only)."""
+    padded = np.zeros(npg * 16, dtype=bool)
+    padded[:ora_mask0.size] = ora_mask0.reshape(-1)
+    ora_pages = set(np.nonzero(padded.reshape(npg, 16).any(-1))[0].tolist())
+    mine = set(int(x) for x in gpu_pages)
+    assert len(mine) == len(ora_pages)
+    kth = float(torch.sort(page_scores, descending=True).values[len(ora_pages) - 1])
+    for pg in ora_pages.symmetric_difference(mine):
+        assert abs(float(page_scores[pg]) - kth) <= 1e-3 * max(1.0, abs(kth)), (pg, float(page_scores[pg]), kth)
+
+
 def _run_case(dev, B, H, Hkv, N, budget, p, dt, seed, shuffle=True, n_heavy=16, fused=True,
               planes=False):
     q, k, v = synth.heavy_hitter_qkv(B, H, N, n_heavy=n_heavy, mass=0.6, seed=seed, dtype=dt)
@@ -41,22 +63,26 @@ def _run_case(dev, B, H, Hkv, N, budget, p, dt, seed, shuffle=True, n_heavy=16, 
     ref = P.decode_layer_dense(q, krep, vrep, top_p=p, token_budget=budget if budget < N else None,
                                high_mode=native.HIGH_MAX, quant="storage", prob_dtype=dt)
     rows = B * H
-    # 1. selector: same pages (a page whose score ties the k-th within rounding may differ)
+    # 1. selector: the oracle's pages, except pages whose score ties the k-th within rounding
+    #    (checked on the oracle's own page scores); the later stages are then followed on the
+    #    GPU's own selection, for every row
     sel = layer.sel_pages.cpu().numpy().reshape(rows, -1)
     selc = layer.sel_count.cpu().numpy().reshape(rows)
     mask0 = ref["mask0"].reshape(rows, N).numpy()
-    same_sel = np.zeros(rows, dtype=bool)
-    for r in range(rows):
-        m = np.zeros(npg * 16, dtype=bool)
-        for pg in sel[r, :selc[r]]:
-            m[pg * 16:(pg + 1) * 16] = True
-        same_sel[r] = np.array_equal(m[:N], mask0[r])
-    assert same_sel.mean() >= 0.9, same_sel.mean()
+    gmask0 = _pages_to_mask(sel, selc, npg)[:, :N]
+    differ = np.nonzero((gmask0 != mask0).any(-1))[0]
+    if differ.size:
+        est_pg = P.quest_chunk_scores_dense(q.float(), krep.float(), 16)[:, :, 0].reshape(rows, -1)
+        for r in differ:
+            _assert_selection_ties(est_pg[r], sel[r, :selc[r]], mask0[r], npg)
+        ref = P.decode_layer_dense(q, krep, vrep, top_p=p, token_budget=budget, high_mode=native.HIGH_MAX,
+                                   quant="storage", prob_dtype=dt,
+                                   mask0=torch.from_numpy(gmask0).reshape(B, H, 1, N))
     # 2. estimator scores on the selected candidates (1e-3 relative)
     scores = layer.scores.cpu().numpy().reshape(rows, -1)
     est = ref["scores"].reshape(rows, N).double().numpy()
     cand_tok = (sel[:, :, None] * 16 + np.arange(16)[None, None, :]).reshape(rows, -1)
-    for r in np.nonzero(same_sel)[0]:
+    for r in range(rows):
         n = selc[r] * 16
         tok = cand_tok[r, :n]
         inside = tok < N
@@ -68,15 +94,13 @@ def _run_case(dev, B, H, Hkv, N, budget, p, dt, seed, shuffle=True, n_heavy=16, 
     gm = _lists_to_mask(idx, cnt, N)
     probs = ref["probs"].reshape(rows, N).numpy()
     _, _, _, margin = native.top_p_mask_f32(probs, p, native.HIGH_MAX, return_margin=True)
-    ok = np.nonzero(same_sel)[0]
-    n_exact = assert_top_p_parity(probs[ok], p, gm[ok], ref["mask"].reshape(rows, N).numpy()[ok],
-                                  ref["low"][ok], margin[ok], margin_tol=5e-6)
-    assert n_exact >= 0.9 * len(ok)
+    assert_top_p_parity(probs, p, gm, ref["mask"].reshape(rows, N).numpy(), ref["low"], margin,
+                        margin_tol=5e-6)
     # 4. attention: exact over the GPU's own survivors, and end to end against the oracle
     tol = 1e-3 if dt == torch.float16 else 8e-3
     own = P.masked_attention(q, krep, vrep, torch.from_numpy(gm).reshape(B, H, 1, N), prob_dtype=dt)
     assert torch.allclose(out, own[:, :, 0], rtol=tol, atol=tol)
-    e2e = (out.reshape(rows, 128)[ok] - ref["out"].reshape(rows, 128)[ok]).abs().max().item()
+    e2e = (out.reshape(rows, 128) - ref["out"].reshape(rows, 128)).abs().max().item()
     assert e2e < 5 * tol, e2e
     return layer, ref
 
@@ -258,7 +282,6 @@ def test_full_size_layer_sampled_rows_and_properties(dev, B, H, Hkv, dt, p, plan
     long_row = int(np.argmax(cnt))
     picks = sorted(set([long_row] + [int(r) for r in rng.integers(0, rows, 5)]))
     tol = 1e-3 if dt == torch.float16 else 8e-3
-    compared = 0
     for r in picks:
         b, h = divmod(r, H)
         kvh = h // (H // Hkv)
@@ -273,7 +296,14 @@ def test_full_size_layer_sampled_rows_and_properties(dev, B, H, Hkv, dt, p, plan
         for pg in sel[r, :selc[r]].cpu().numpy():
             m0[pg * 16:(pg + 1) * 16] = True
         if not np.array_equal(m0, ref["mask0"].reshape(N).numpy()):
-            continue  # a page tied with the 512th score within rounding: rows are incomparable
+            # pages tied with the 512th score within rounding: checked as ties, then the later
+            # stages are followed on the GPU's own selection
+            est_pg = P.quest_chunk_scores_dense(qd, kd, 16)[0, 0, 0]
+            _assert_selection_ties(est_pg, sel[r, :selc[r]].cpu().numpy(),
+                                   ref["mask0"].reshape(N).numpy(), npg)
+            ref = P.decode_layer_dense(qd, kd, vd, top_p=p, token_budget=budget,
+                                       high_mode=native.HIGH_MAX, quant="storage", prob_dtype=dt,
+                                       mask0=torch.from_numpy(m0).reshape(1, 1, 1, N))
         gm = np.zeros((1, N), dtype=bool)
         gm[0, idx[r, :cnt[r]].cpu().numpy()] = True
         pr = ref["probs"].reshape(1, N).numpy()
@@ -283,8 +313,8 @@ def test_full_size_layer_sampled_rows_and_properties(dev, B, H, Hkv, dt, p, plan
         own = P.masked_attention(qd, kd, vd, torch.from_numpy(gm).reshape(1, 1, 1, N),
                                  prob_dtype=dt if cnt[r] <= 128 else torch.float32)
         assert torch.allclose(out[b, h].float().cpu(), own[0, 0, 0], rtol=tol, atol=tol), r
-        compared += 1
-    assert compared >= len(picks) - 1, (compared, len(picks))
+        e2e = (out[b, h].float().cpu() - ref["out"][0, 0, 0]).abs().max().item()
+        assert e2e < 5 * tol, (r, e2e)
 
 
 @pytest.mark.parametrize("H,Hkv", [(8, 8), (8, 2)])

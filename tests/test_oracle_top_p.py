@@ -134,10 +134,48 @@ def test_top_p_unnormalized_wrapper_shapes_and_mask_of_masked_entries():
     assert torch.all((probs * mask).sum(-1) >= 0.9 - 1e-6)
 
 
-def test_f16_variant_runs_in_half_value_set():
+def test_16_bit_addition_against_numpy_and_bf16_by_bit_trick():
+    # one addition of the element type, the building block of the CUB-order restatement: fp16
+    # against numpy's float16 arithmetic, bf16 against fp32 addition + round-to-nearest-even of
+    # the upper half (24 >= 2 * 8 + 2 bits: the double rounding is innocuous)
+    rng = np.random.default_rng(5)
+    a = (rng.random(3000) * 2.0 ** rng.integers(-26, 1, 3000)).astype(np.float16)
+    b = (rng.random(3000) * 2.0 ** rng.integers(-26, 1, 3000)).astype(np.float16)
+    for x, y in zip(a, b):
+        assert native.dt_add(float(x), float(y), native.DT_F16) == float(np.float16(x + y))
+    def bf(v):
+        u = np.float32(v).view(np.uint32)
+        return float(np.uint32(((int(u) + 0x7FFF + ((int(u) >> 16) & 1)) >> 16) << 16).view(np.float32))
+    for x, y in zip(a[:1500], b[:1500]):
+        xb, yb = bf(float(x)), bf(float(y))
+        assert native.dt_add(xb, yb, native.DT_BF16) == bf(np.float32(xb) + np.float32(yb))
+    # fp16 specials: the tolerance, a subnormal tie, overflow
+    assert native.dt_round(1e-5, native.DT_F16) == 168 * 2.0 ** -24
+    assert native.dt_round(1e-5, native.DT_BF16) == 168 * 2.0 ** -24
+    assert native.dt_round(1.5 * 2.0 ** -24, native.DT_F16) == 2.0 ** -23
+    assert native.dt_round(2.5 * 2.0 ** -24, native.DT_F16) == 2.0 ** -23
+    assert native.dt_round(65520.0, native.DT_F16) == float("inf")
+
+
+def test_cub_order_in_fp32_agrees_with_the_fp64_sum_form_where_the_margin_allows():
+    # the float instantiation (csrc/src/sampling.cu:45-63) in CUB's order against the same
+    # bisection with sums accumulated in fp64: wherever no decision came close to a rounding flip
+    # both must give the same mask, pivot and iteration count
+    rng = np.random.default_rng(9)
+    pr = softmax_rows(rng.standard_normal((24, 5000)).astype(np.float32) * 4)
+    for mode in (native.HIGH_FIRST, native.HIGH_MAX):
+        m0, low0, it0, margin = native.top_p_mask_f32(pr, 0.9, mode, return_margin=True)
+        m1, low1, it1 = native.top_p_mask_cub(pr, native.DT_F32, 0.9, mode)
+        clear = margin > 2e-6
+        assert clear.sum() >= 20
+        assert np.array_equal(m0[clear], m1[clear]) and np.array_equal(low0[clear], low1[clear])
+        assert np.array_equal(it0[clear], it1[clear])
+
+
+def test_16_bit_rows_stay_in_the_value_set():
     rng = np.random.default_rng(6)
     pr = softmax_rows(rng.standard_normal((8, 400)).astype(np.float32) * 3).astype(np.float16)
-    m, low, _ = native.top_p_mask_f16(pr.view(np.uint16), 0, 0.9, native.HIGH_MAX)
+    m, low, _ = native.top_p_mask_cub(pr.view(np.uint16), native.DT_F16, 0.9, native.HIGH_MAX)
     assert np.all(low.astype(np.float16).astype(np.float32) == low)   # pivots are fp16 values
     assert np.array_equal(m, (pr.astype(np.float32) > low[:, None]).astype(np.uint8))
     assert np.all((pr.astype(np.float64) * m).sum(-1) >= 0.9 - 5e-3)

@@ -9,7 +9,7 @@ from concurrent.futures import ThreadPoolExecutor
 _PKG = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(_PKG, "csrc")
 LIB_PATH = os.path.join(_PKG, "libtwilight_hip.so")
-SOURCES = ["api.hip", "top_p.hip", "gemv_int4.hip", "fused_row.hip", "layer_row.hip", "gemv_nhd.hip", "sparse_attn.hip", "group_attn.hip", "rope.hip", "quest.hip", "kv_shadow.hip", "meta_planes.hip", "label_ops.hip", "qk_int8.hip"]
+SOURCES = ["api.hip", "top_p.hip", "top_p_dtype.hip", "gemv_int4.hip", "fused_row.hip", "layer_row.hip", "gemv_nhd.hip", "sparse_attn.hip", "group_attn.hip", "rope.hip", "quest.hip", "kv_shadow.hip", "meta_planes.hip", "label_ops.hip", "qk_int8.hip"]
 
 # Packed-fp32 VALU forms are disabled for every kernel of this library.
 HIPCC_FLAGS = [

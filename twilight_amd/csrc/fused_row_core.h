@@ -119,11 +119,11 @@ __device__ __forceinline__ void estimate_prune_row(const FusedArgs& a, FusedSmem
     for (int w = 0; w < 4; ++w)
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
-        half2_t pr = {(_Float16)qf[8 * w + s], (_Float16)qf[8 * w + s + 4]};
+        half2_t pr = {q_to_half(qf[8 * w + s]), q_to_half(qf[8 * w + s + 4])};
         qp[4 * w + s] = pr;
       }
 #pragma unroll
-    for (int i = 0; i < 32; ++i) qsum += (float)(_Float16)qf[i];
+    for (int i = 0; i < 32; ++i) qsum += (float)q_to_half(qf[i]);
   }
 
   // ---- stream the run: scores into x[] --------------------------------------------------------

@@ -142,11 +142,11 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_int4_kernel(GemvArgs a) {
     for (int w = 0; w < 4; ++w)
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
-        half2_t pr = {(_Float16)qf[8 * w + s], (_Float16)qf[8 * w + s + 4]};
+        half2_t pr = {q_to_half(qf[8 * w + s]), q_to_half(qf[8 * w + s + 4])};
         qp[4 * w + s] = pr;
       }
 #pragma unroll
-    for (int i = 0; i < 32; ++i) qsum += (float)(_Float16)qf[i];
+    for (int i = 0; i < 32; ++i) qsum += (float)q_to_half(qf[i]);
   }
 
   const size_t rec_stride = (size_t)a.num_kv_heads * TWL_INT4_RECORD_BYTES;
@@ -253,11 +253,11 @@ __global__ __launch_bounds__(kGemvRowThreads) void gemv_int4_rows_kernel(GemvArg
     for (int w = 0; w < 4; ++w)
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
-        half2_t pr = {(_Float16)qf[8 * w + s], (_Float16)qf[8 * w + s + 4]};
+        half2_t pr = {q_to_half(qf[8 * w + s]), q_to_half(qf[8 * w + s + 4])};
         qp[4 * w + s] = pr;
       }
 #pragma unroll
-    for (int i = 0; i < 32; ++i) qsum += (float)(_Float16)qf[i];
+    for (int i = 0; i < 32; ++i) qsum += (float)q_to_half(qf[i]);
   }
   const size_t rec_stride = (size_t)a.num_kv_heads * TWL_INT4_RECORD_BYTES;
   const uint8_t* base = a.k_int4 + (size_t)kvh * TWL_INT4_RECORD_BYTES + 16 * lane;
@@ -357,7 +357,6 @@ extern "C" int twl_gemv_int4(const void* q, int q_dtype, float* out, uint32_t ou
   (void)twl::device_cu_count(&cus);
   const uint64_t want_waves = 8ull * (uint64_t)cus;
   // about one row per compute unit and a row of scores that fits LDS: a workgroup per row
-#ifndef TWL_GEMV_NO_ROWS
   // (measured at 256 rows: 2048 pages per row 122.7 -> 114.2 us, 512 pages per row no change)
   if (max_pages_per_row > 512u && max_pages_per_row <= 2048u && 2u * rows >= (uint32_t)cus &&
       rows <= 2u * (uint32_t)cus) {
@@ -381,12 +380,7 @@ extern "C" int twl_gemv_int4(const void* q, int q_dtype, float* out, uint32_t ou
 #undef TWL_GEMV_ROWS
     return hipGetLastError() == hipSuccess ? TWL_OK : TWL_ELAUNCH;
   }
-#endif
-#ifdef TWL_GEMV_PW
-  const int pw = TWL_GEMV_PW;
-#else
   const int pw = row_pages / 64 >= want_waves ? 64 : (row_pages / 16 >= want_waves ? 16 : 8);
-#endif
   if (q_dtype == TWL_F16) {
     if (sel_pages) twl::launch_gemv<TWL_F16, true>(a, rows, pw, st);
     else twl::launch_gemv<TWL_F16, false>(a, rows, pw, st);

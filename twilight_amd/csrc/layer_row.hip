@@ -37,10 +37,7 @@ struct RowArgs {
 
 constexpr int kRowThreads = 1024;
 constexpr int kRowWaves = kRowThreads / kWave;
-#ifndef TWL_ROW_UNROLL
-#define TWL_ROW_UNROLL 4
-#endif
-constexpr int kRowUnroll = TWL_ROW_UNROLL;  // 16-byte loads in flight per lane (2 pages each)
+constexpr int kRowUnroll = 4;  // 16-byte loads in flight per lane (2 pages each)
 
 // PLANES: page scores from the plane layout (half the metadata bytes: only the run the sign of
 // q_d selects is read, 2 pages per lane, channels in ascending order), else from the 512-byte

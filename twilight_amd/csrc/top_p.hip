@@ -22,7 +22,7 @@
 namespace twl {
 
 struct TopPArgs {
-  const void* in;        // probs (any dtype) or raw fp32 scores
+  const void* in;        // fp32 probabilities or raw fp32 scores
   uint32_t in_stride;    // elements between rows
   const int32_t* lens;   // nullable: per-row length (<= d)
   uint32_t d;
@@ -58,7 +58,8 @@ __global__ __launch_bounds__(THREADS) void top_p_kernel(TopPArgs a) {
   // ---- load the row once ----------------------------------------------------------------
   float x[VPT];
   const float fill = FUSED_SOFTMAX ? -__builtin_inff() : 0.0f;
-  if (DT == TWL_F32) {
+  {
+    static_assert(DT == TWL_F32, "16-bit probabilities have a kernel of their own (top_p_dtype.hip)");
     const float* src = (const float*)a.in + (size_t)row * a.in_stride;
     const bool vec_ok = ((((uintptr_t)src) & 15u) == 0);
 #pragma unroll
@@ -70,26 +71,6 @@ __global__ __launch_bounds__(THREADS) void top_p_kernel(TopPArgs a) {
       } else {
 #pragma unroll
         for (int j = 0; j < 4; ++j) x[4 * c + j] = (e0 + j < len) ? src[e0 + j] : fill;
-      }
-    }
-  } else {
-    const uint16_t* src = (const uint16_t*)a.in + (size_t)row * a.in_stride;
-    const bool vec_ok = ((((uintptr_t)src) & 7u) == 0);
-#pragma unroll
-    for (int c = 0; c < CHUNKS; ++c) {
-      const uint32_t e0 = 4u * (uint32_t)(tx + THREADS * c);
-      if (vec_ok && e0 + 4 <= len) {
-        u32x2 v = *(const u32x2*)(src + e0);
-        x[4 * c + 0] = bits16_to_f32<DT == TWL_F32 ? TWL_F16 : DT>(v.x & 0xFFFFu);
-        x[4 * c + 1] = bits16_to_f32<DT == TWL_F32 ? TWL_F16 : DT>(v.x >> 16);
-        x[4 * c + 2] = bits16_to_f32<DT == TWL_F32 ? TWL_F16 : DT>(v.y & 0xFFFFu);
-        x[4 * c + 3] = bits16_to_f32<DT == TWL_F32 ? TWL_F16 : DT>(v.y >> 16);
-      } else {
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-          x[4 * c + j] = (e0 + j < len)
-                             ? bits16_to_f32<DT == TWL_F32 ? TWL_F16 : DT>(src[e0 + j])
-                             : fill;
       }
     }
   }
@@ -246,22 +227,6 @@ extern "C" int twl_top_p_f32(const float* probs, uint8_t* mask, int32_t* idx, in
   a.high_mode = high_mode; a.mask = mask; a.idx = idx; a.idx_stride = idx_stride; a.count = count;
   a.low_out = low_out; a.iters_out = iters_out;
   return twl::launch_top_p<TWL_F32, false>(a, rows, (hipStream_t)stream);
-}
-
-extern "C" int twl_top_p_f16(const void* probs, int dtype, uint8_t* mask, int32_t* idx,
-                             int32_t* count, const float* p_arr, float p, uint32_t rows,
-                             uint32_t d, uint32_t idx_stride, int high_mode, float* low_out,
-                             int32_t* iters_out, void* stream) {
-  int rc = check_top_p_common(probs, mask, idx, count, p, p_arr, rows, d, idx_stride, high_mode);
-  if (rc != TWL_OK) return rc;
-  if (dtype != TWL_F16 && dtype != TWL_BF16) return TWL_EDTYPE;
-  if (((uintptr_t)probs) & 1u) return TWL_EALIGN;
-  TopPArgs a{};
-  a.in = probs; a.in_stride = d; a.lens = nullptr; a.d = d; a.p_arr = p_arr; a.p = p;
-  a.high_mode = high_mode; a.mask = mask; a.idx = idx; a.idx_stride = idx_stride; a.count = count;
-  a.low_out = low_out; a.iters_out = iters_out;
-  if (dtype == TWL_F16) return twl::launch_top_p<TWL_F16, false>(a, rows, (hipStream_t)stream);
-  return twl::launch_top_p<TWL_BF16, false>(a, rows, (hipStream_t)stream);
 }
 
 extern "C" int twl_softmax_top_p_f32(const float* scores, uint32_t score_stride,

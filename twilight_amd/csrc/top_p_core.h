@@ -64,23 +64,14 @@ __device__ __forceinline__ float row_max_regs(const float (&x)[VPT], float (*red
 }
 
 // LDS of the bisection's single-wavefront phase (see bisect_regs)
-#ifndef TWL_HEAVY_PER_LANE
-#define TWL_HEAVY_PER_LANE 4
-#endif
-#ifndef TWL_HEAVY_J
-#define TWL_HEAVY_J 8
-#endif
-constexpr int kHeavyPerLane = TWL_HEAVY_PER_LANE;
+constexpr int kHeavyPerLane = 4;   // list slots per lane of the single-wavefront phase
+constexpr int kHeavyShift = 8;     // tau = high / 2^kHeavyShift
 constexpr int kHeavyCap = kWave * kHeavyPerLane;
 struct BisectSmem {
   float hlist[kHeavyCap];
   uint32_t wcnt[16], wmax[16], wmin[16];
   uint32_t state[8];
 };
-
-#ifndef TWL_BISECT_HEAVY
-#define TWL_BISECT_HEAVY 1
-#endif
 
 // The bisection of csrc/include/sampling.cuh:156-217 on probabilities held in registers, starting
 // from the bracket (0, high]. Returns the final `low` (keep x > low); x is clamped to >= 0.
@@ -100,7 +91,7 @@ __device__ __forceinline__ float bisect_regs(float (&x)[VPT], float p, float hig
                                              float (*red)[2][16], int& buf, int& iters,
                                              BisectSmem& bs, bool high_is_row_max) {
   constexpr int NWAVES = THREADS / kWave;
-  constexpr bool HEAVY = TWL_BISECT_HEAVY && NWAVES > 1 && THREADS * VPT >= 2048;
+  constexpr bool HEAVY = NWAVES > 1 && THREADS * VPT >= 2048;
   const int lane = lane_id();
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   float low = 0.0f;
@@ -213,7 +204,7 @@ __device__ __forceinline__ float bisect_regs(float (&x)[VPT], float p, float hig
   };
 
   if constexpr (HEAVY) {
-    const float tau = high * (1.0f / (float)(1 << TWL_HEAVY_J));
+    const float tau = high * (1.0f / (float)(1 << kHeavyShift));
     const uint32_t tau_b = as_u32(tau);
     // ---- census: elements above tau per wavefront, largest element <= tau, smallest positive
     uint32_t cnt = 0, mx = 0u, mn1 = 0xFFFFFFFFu;

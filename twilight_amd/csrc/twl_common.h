@@ -54,6 +54,14 @@ __device__ __forceinline__ float round_to(float f) {
   return f;
 }
 
+// A query value as the INT4 estimator's fp16 dot products take it. fp16 queries pass unchanged.
+// A bf16 query is converted to fp16: exact for 2^-17 <= |q| <= 65504 (8 significand bits fit 11),
+// rounded to a multiple of 2^-24 below that, and SATURATED to +-65504 above (so that a score can
+// never become inf - inf = NaN; attention queries are nowhere near that magnitude).
+__device__ __forceinline__ _Float16 q_to_half(float v) {
+  return (_Float16)__builtin_fminf(__builtin_fmaxf(v, -65504.0f), 65504.0f);
+}
+
 // eight 16-bit values of a 16-byte load, widened to fp32 (element order = memory order)
 template <int DT>
 __device__ __forceinline__ void unpack8(const u32x4& v, float* f) {

@@ -102,7 +102,12 @@ def top_p_fp32_return_mask(probs: torch.Tensor, top_p: Union[torch.Tensor, float
 def top_p_fp16_return_mask(probs: torch.Tensor, top_p: Union[torch.Tensor, float],
                            high: str = "first") -> torch.Tensor:
     """Drop-in for twilight/kernel/cuda/sampling.py:118-124 (fp16 or bf16 probabilities,
-    csrc/src/sampling.cu:22-43). Pivots are kept in the 16-bit type; partial sums in fp32."""
+    csrc/src/sampling.cu:22-43). Like that instantiation of the kernel, p, the pivots, the
+    tolerance and every partial sum are values of the 16-bit type, and the additions run in the
+    order of the reference's cub::BlockReduce (csrc/include/sampling.cuh:54), so the mask is the
+    one the reference's arithmetic gives, bit for bit. Note what that arithmetic does: a sum of
+    many small probabilities stalls in 16 bits, so the kept mass can differ visibly from the fp32
+    entry's on the same row."""
     check_input(probs, "probs")
     if probs.dtype not in (torch.float16, torch.bfloat16):
         raise RuntimeError(f"probs must be float16 or bfloat16, got {probs.dtype}")
