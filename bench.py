@@ -12,8 +12,12 @@ context 32768, Quest budget 8192, top-p 0.95.
 Prints ONE JSON line. ``value`` is microseconds per layer (lower is better). ``roofline`` is for
 the kernel with the largest HBM term (the Quest metadata stream); ``kernels`` lists every kernel of
 the layer with its algorithmic bytes, time and fraction of the 8 TB/s peak, and ``gemv_cfg2`` the
-stand-alone INT4 GEMV at 8 x 32 x 32768 candidates. ``cpu_baseline`` is the CPU oracle (a port of
-the reference's torch path) timed on this host on one of the 8 batch elements and scaled by 8.
+stand-alone INT4 GEMV at 8 x 32 x 32768 candidates. ``cfg4_b16`` (the same layer at batch 16) and
+``cfg5_layer`` (32 q heads on 8 kv heads, bf16, p 0.9, with the dense paged decode beside it) are
+the other two layer shapes of the headline figure, measured the same way with fewer steps.
+``cpu_baseline`` is the CPU oracle (a port of the reference's torch path) timed on this host on
+one of the 8 batch elements and scaled by 8, plus the reference's own CPU case (B=1, context 4096)
+with warm-ups, repeats, median and per-stage times.
 
 Other workloads (``--workload``), each printing one JSON line of its own: ``llama3`` (the same
 layer with 32 q heads on 8 kv heads, bf16, p 0.9, plus dense-decode comparisons), ``topp`` (the
@@ -63,11 +67,59 @@ def _time_calls(fn, iters: int, warmup: int) -> float:
     return e0.elapsed_time(e1) * 1000.0 / iters
 
 
-def cpu_baseline(N: int, H: int, budget: int, top_p: float, batch_scale: int, dev, seed: int = 0):
-    """Times the CPU oracle (torch fp32 + the C top-p restatement) on one batch element drawn by
-    the generator the GPU workload uses (same planted heavy hitters), un-paged to dense K / V."""
+def _median_time(fn, warmups: int, repeats: int):
+    """(median seconds, last result) of ``fn`` after ``warmups`` untimed calls."""
+    for _ in range(warmups):
+        out = fn()
+    ts = []
+    for _ in range(repeats):
+        t0 = time.perf_counter()
+        out = fn()
+        ts.append(time.perf_counter() - t0)
+    ts.sort()
+    return ts[len(ts) // 2], out
+
+
+def cpu_baseline_cfg1(warmups: int = 3, repeats: int = 20):
+    """The CPU restatement of the reference's decode math on its own CPU-runnable case: B=1, 32 MHA
+    heads, head_dim 128, context 4096, fp32, 16 heavy hitters per head with ~60 % of the softmax
+    mass, every token a candidate, p = 0.95. time.perf_counter, warm-ups, repeats, median; stages
+    timed one by one and two totals: (A) K re-quantised inside the step as
+    twilight/pyimpl/attention.py:247-251 does, (B) K quantised beforehand."""
     from oracle import native, pyimpl_port as P
     from twilight_amd import synth
+    q, k, v = synth.heavy_hitter_qkv(1, 32, 4096, n_heavy=16, mass=0.6, seed=0)
+    mask0 = torch.ones((1, 32, 1, 4096), dtype=torch.bool)
+    t_quant, quant = _median_time(lambda: torch.from_numpy(P.int4_quant_storage(k)[3]), warmups, repeats)
+    t_gemv, est = _median_time(lambda: P.estimator_scores(q, quant), warmups, repeats)
+    t_topp, pruned = _median_time(lambda: P.top_p_unnormalized(est, 0.95, native.HIGH_MAX), warmups, repeats)
+    mask = mask0 & pruned[0]
+    t_attn, _ = _median_time(lambda: P.masked_attention(q, k, v, mask, torch.float32), warmups, repeats)
+    t_a, ra = _median_time(lambda: P.decode_layer_dense(q, k, v, top_p=0.95, token_budget=None,
+                                                       high_mode=native.HIGH_MAX, quant="storage"),
+                           warmups, repeats)
+    t_b, _ = _median_time(lambda: P.decode_layer_dense(q, k, v, top_p=0.95, token_budget=None,
+                                                      high_mode=native.HIGH_MAX, k_deq=quant),
+                          warmups, repeats)
+    us = lambda t: round(t * 1e6, 1)
+    return {"workload": "B=1, 32 MHA heads, head_dim 128, context 4096, fp32, 16 heavy hitters per "
+                        "head (~60 % of the mass), all tokens candidates, p 0.95, INT4 group 32",
+            "warmups": warmups, "repeats": repeats, "statistic": "median",
+            "us_A_requantise_every_step": us(t_a), "us_B_k_prequantised": us(t_b),
+            "stages_us": {"quantise": us(t_quant), "gemv": us(t_gemv), "softmax_top_p": us(t_topp),
+                          "attention": us(t_attn)},
+            "survivors_mean": float(ra["mask"].sum(-1).float().mean())}
+
+
+def cpu_baseline(N: int, H: int, budget: int, top_p: float, batch_scale: int, dev, seed: int = 0,
+                 warmups: int = 1, repeats: int = 3):
+    """Times the CPU oracle (torch fp32 + the C quantiser and top-p restatement) on one batch
+    element drawn by the generator the GPU workload uses (same planted heavy hitters), un-paged to
+    dense K / V: one warm-up, the median of three runs, scaled by the batch size. The reference's
+    own CPU case (B=1, context 4096) is timed as well, with its per-stage split."""
+    from oracle import native, pyimpl_port as P
+    from twilight_amd import synth
+    torch.set_num_threads(os.cpu_count() or 1)
     threads = torch.get_num_threads()
     qd, kd, vd, (ids, _, _) = synth.layer_inputs_device(1, H, H, N, torch.float16, dev, seed=seed)
     order = ids.long()
@@ -76,25 +128,27 @@ def cpu_baseline(N: int, H: int, budget: int, top_p: float, batch_scale: int, de
     v = vd[order].reshape(N, H, 128).permute(1, 0, 2).float().cpu().reshape(1, H, N, 128).contiguous()
     del qd, kd, vd
     # (A) as the reference does it: K is re-quantised inside every decode step
-    t0 = time.perf_counter()
-    ra = P.decode_layer_dense(q, k, v, top_p=top_p, token_budget=budget, high_mode=native.HIGH_MAX,
-                              quant="storage", prob_dtype=torch.float16)
-    ta = time.perf_counter() - t0
+    ta, ra = _median_time(lambda: P.decode_layer_dense(
+        q, k, v, top_p=top_p, token_budget=budget, high_mode=native.HIGH_MAX, quant="storage",
+        prob_dtype=torch.float16), warmups, repeats)
     # (B) K quantised once on append, as the GPU path does
     k_deq = torch.from_numpy(P.int4_quant_storage(k)[3])
-    t0 = time.perf_counter()
-    P.decode_layer_dense(q, k, v, top_p=top_p, token_budget=budget, high_mode=native.HIGH_MAX,
-                         k_deq=k_deq, prob_dtype=torch.float16)
-    tb = time.perf_counter() - t0
+    tb, _ = _median_time(lambda: P.decode_layer_dense(
+        q, k, v, top_p=top_p, token_budget=budget, high_mode=native.HIGH_MAX, k_deq=k_deq,
+        prob_dtype=torch.float16), warmups, repeats)
+    del k, v, k_deq
     return {
         "value": ta * 1e6 * batch_scale, "unit": "us/layer", "cores": threads, "kind": "port",
         "value_k_prequantised": tb * 1e6 * batch_scale,
         "sample": (f"1 of {batch_scale} batch elements (32 heads x {N} tokens, budget {budget}, "
-                   f"p {top_p}; same generator as the GPU workload) through oracle.pyimpl_port.decode_layer_dense, one run each, "
-                   f"time x {batch_scale}; `value` re-quantises K every step like "
-                   "twilight/pyimpl/attention.py:247-251, `value_k_prequantised` does not; torch "
-                   f"uses {threads} threads, the C quantiser / top-p one"),
+                   f"p {top_p}; same generator as the GPU workload) through "
+                   f"oracle.pyimpl_port.decode_layer_dense, {warmups} warm-up, median of {repeats} "
+                   f"runs, time x {batch_scale}; `value` re-quantises K every step like "
+                   "twilight/pyimpl/attention.py:247-251 (variant A), `value_k_prequantised` does "
+                   f"not (variant B); torch uses {threads} threads "
+                   f"(os.cpu_count() = {os.cpu_count()}), the C quantiser / top-p one"),
         "survivors_mean": float(ra["mask"].sum(-1).float().mean()),
+        "cfg1": cpu_baseline_cfg1(),
     }
 
 
@@ -415,6 +469,100 @@ class _Timed:
         return getattr(self._layer, name)
 
 
+def measure_shape(L, dev, B, H, Hkv, N, dt, budget, top_p, n_layers, steps, warmup,
+                  dense: bool = False):
+    """One more shape of the same layer, measured the way the headline figure is: ``n_layers``
+    independent caches visited round-robin, wall time per ``twl_decode_layer`` step, and the two
+    kernels of the step timed alone with events. Returns a dict for the JSON line."""
+    from twilight_amd import synth
+    from twilight_amd.cache import PagedKVCache
+    from twilight_amd.layer import TwilightDecodeLayer
+    D, npg = 128, N // 16
+    qcode = 1 if dt == torch.bfloat16 else 0
+    layers, qs = [], []
+    for li in range(n_layers):
+        q, k, v, (ids, indptr, last) = synth.layer_inputs_device(B, H, Hkv, N, dt, dev, seed=500 + 10 * li)
+        cache = PagedKVCache(B * npg, Hkv, dt, dev)
+        cache.k_cache, cache.v_cache = k, v
+        cache.set_page_table(ids, indptr, last)
+        cache.rebuild_shadow()
+        cache.enable_planes()
+        layers.append(TwilightDecodeLayer(cache, H, token_budget=budget, top_p=top_p, high="max"))
+        qs.append(q)
+    torch.cuda.synchronize()
+    for i in range(warmup):
+        layers[i % n_layers].forward(qs[i % n_layers])
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        layers[i % n_layers].forward(qs[i % n_layers])
+    torch.cuda.synchronize()
+    wall_us = (time.perf_counter() - t0) * 1e6 / steps
+    for i in range(n_layers):
+        layers[i].forward(qs[i])
+    torch.cuda.synchronize()
+    n_bar = float(torch.stack([l.count for l in layers]).float().mean())
+    rows, kp = B * H, layers[0].k_pages
+    M = kp * 16
+    stream = torch.cuda.current_stream().cuda_stream
+    p = lambda t: 0 if t is None else t.data_ptr()
+    sm = 1.0 / math.sqrt(D)
+    state = {"i": 0}
+
+    def rot(make):
+        fns = [make(layers[i], layers[i].cache, qs[i]) for i in range(n_layers)]
+
+        def call():
+            fns[state["i"] % n_layers]()
+            state["i"] += 1
+        return call
+    row_us = _time_calls(rot(lambda l, c, q: lambda: L.twl_select_estimate_prune(
+        p(q), qcode, p(c.meta), p(c.k_int4), p(c.kv_page_indices), p(c.kv_page_indptr),
+        p(c.kv_last_page_len), B, H, Hkv, budget, npg, sm, 0, top_p, 1, p(l.sel_pages), kp,
+        p(l.sel_count), p(l.idx), M, p(l.count), 0, 0, 0, M, p(l.cand_count), p(c.meta_planes),
+        c.meta_planes.size(4), 0, 0, stream)), max(steps, 40), 2 * n_layers)
+    attn_us = _time_calls(rot(lambda l, c, q: lambda: L.twl_sparse_attn(
+        p(q), p(l.out), qcode, p(c.k_cache), p(c.v_cache), *c.k_cache.stride()[:3], p(l.idx), M,
+        p(l.count), p(c.kv_page_indices), p(c.kv_page_indptr), B, H, Hkv, sm, 0,
+        p(l.attn_workspace), l.attn_workspace.numel(), stream)), max(steps, 40), 2 * n_layers)
+    attn_bytes = int(rows * n_bar) * (2 * D * 2 + 4) + rows * D * 4
+    lists = rows * npg * 4 + rows * kp * 8 + int(rows * n_bar) * 4 + rows * 12 + rows * D * 2
+    # per q head, as the reference's code selects and prunes (attention.py:124-126): metadata once
+    # per kv head (the record is shared by the group), INT4 records once per q-head row
+    per_head = B * Hkv * npg * 512 + rows * M * 80 + lists + attn_bytes
+    # one candidate list per kv head (INT4 records read once for the group's q heads, fp32
+    # scores per q head): the lower count for GQA; equal to the above without GQA
+    shared = B * Hkv * npg * 512 + B * Hkv * M * 80 + rows * M * 4 * (1 if H != Hkv else 0) \
+        + lists + attn_bytes
+    by_design = per_head - (B * Hkv * npg * 512 >> (H // Hkv))
+    gb = lambda n: round(n / wall_us / 1e3 / HBM_PEAK_GBS, 4)
+    out = {"workload": f"B={B}, {H} q / {Hkv} kv heads, {'bf16' if qcode else 'fp16'}, context {N}, "
+                       f"budget {budget}, p {top_p}, {n_layers} caches rotated",
+           "us_per_layer": round(wall_us, 2), "steps": steps,
+           "select_estimate_prune_us": round(row_us, 2), "sparse_attn_us": round(attn_us, 2),
+           "survivors_mean": round(n_bar, 1),
+           "layer_bytes_per_q_head_lists": per_head, "frac_of_hbm_peak_per_q_head_lists": gb(per_head),
+           "layer_bytes_read_by_design": by_design, "frac_of_hbm_peak_read_by_design": gb(by_design)}
+    if H != Hkv:
+        out["layer_bytes_shared_candidate_lists"] = shared
+        out["frac_of_hbm_peak_shared_candidate_lists"] = gb(shared)
+    if dense:
+        gws = torch.empty(int(L.twl_group_attn_workspace_bytes(B, H, Hkv, N, 0)), dtype=torch.uint8,
+                          device=dev)
+        outd = torch.empty_like(qs[0])
+        us = _time_calls(rot(lambda l, c, q: lambda: L.twl_group_attn(
+            p(q), p(outd), qcode, p(c.k_cache), p(c.v_cache), *c.k_cache.stride()[:3], 0, 0, 0, N,
+            p(c.kv_page_indices), p(c.kv_page_indptr), p(c.kv_last_page_len), B, H, Hkv, sm, 0,
+            p(gws), gws.numel(), stream)), 40, n_layers)
+        nbytes = B * Hkv * N * 2 * D * 2
+        out["dense_group_attn_us"] = round(us, 2)
+        out["dense_group_attn_frac_of_hbm_peak"] = round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)
+        out["speedup_vs_dense_decode"] = round(us / wall_us, 2)
+    del layers, qs
+    torch.cuda.empty_cache()
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -451,6 +599,8 @@ def main() -> int:
     ap.add_argument("--group-union", action="store_true",
                     help="attention over the union of each kv head's survivor lists (GQA)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extra-shapes", action="store_true",
+                    help="default workload: skip the B=16 and the Llama-3-shape sections")
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel breakdown")
     args = ap.parse_args()
     if args.top_p is None:
@@ -669,7 +819,13 @@ def main() -> int:
                                else dom_name + "_kernel"),
                     "achieved": dom["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                     "frac": dom["frac_of_hbm_peak"], "bytes_per_launch": dom["bytes"],
-                    "us_per_launch": dom["us"], "traffic": traffic}
+                    "us_per_launch": dom["us"], "traffic": traffic,
+                    "frac_traffic": (None if traffic is None else
+                                     round(traffic / dom["us"] / 1e3 / HBM_PEAK_GBS, 4)),
+                    "traffic_source": (None if traffic is None else
+                                       "HBM counters of an earlier rocprofv3 --pmc run of this "
+                                       "command (FETCH_SIZE, WRITE_SIZE scaled by a 1 GiB copy; "
+                                       "summary under profiles/), not read in this run")}
         if "bytes_read_by_design" in dom:
             roofline["note"] = ("achieved = algorithmic bytes / time; the kernel reads only the "
                                 "min or max runs that the signs of its queries select (plane "
@@ -745,6 +901,16 @@ def main() -> int:
             dense["torch_sdpa_us"] = None
             dense["torch_sdpa_what"] = f"not available: {type(e).__name__}: {e}"
 
+    # ---- the two other layer shapes of the headline figure, in the same line ------------------
+    extra = {}
+    if (not llama and not args.no_extra_shapes and not args.split_estimator and not args.no_planes
+            and (B, N, args.budget) == (8, 32768, 8192)):
+        es, ew = max(20, min(args.steps, 60)), max(4, min(args.warmup, 10))
+        extra["cfg4_b16"] = measure_shape(L, dev, 16, 32, 32, N, torch.float16, args.budget,
+                                          args.top_p, 2, es, ew)
+        extra["cfg5_layer"] = measure_shape(L, dev, 8, 32, 8, N, torch.bfloat16, args.budget, 0.9,
+                                            4, es, ew, dense=True)
+
     cpu = None
     if not args.no_cpu_baseline and not llama:
         cpu = cpu_baseline(N, H, args.budget, args.top_p, B, dev)
@@ -771,6 +937,7 @@ def main() -> int:
     }
     if dense:
         line["dense_decode_baseline"] = dense
+    line.update(extra)
     print(json.dumps(line))
     return 0
 
