@@ -49,10 +49,10 @@ struct FusedArgs {
 // a nibble at mantissa bits 4..7 of an fp16 with exponent 0 is exactly 1 + n/64 (see gemv_int4.hip)
 __device__ __forceinline__ float fused_dot8(uint32_t w, const half2_t* qp, float acc) {
   const uint32_t m = 0x00F000F0u, one = 0x3C003C00u;
-  acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, ((w << 4) & m) | one), qp[0], acc, false);
-  acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, (w & m) | one), qp[1], acc, false);
-  acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, ((w >> 4) & m) | one), qp[2], acc, false);
-  acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, ((w >> 8) & m) | one), qp[3], acc, false);
+  acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, and_or(w << 4, m, one)), qp[0], acc, false);
+  acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, and_or(w, m, one)), qp[1], acc, false);
+  acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, and_or(w >> 4, m, one)), qp[2], acc, false);
+  acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(half2_t, and_or(w >> 8, m, one)), qp[3], acc, false);
   return acc;
 }
 

@@ -51,10 +51,10 @@ constexpr int kGemvUnroll = 4;          // pages in flight per wavefront
 // the cancellation costs about one fp32 ulp of sum q).
 __device__ __forceinline__ float dot8_nibbles(uint32_t w, const half2_t* qp, float acc) {
   const uint32_t m = 0x00F000F0u, one = 0x3C003C00u;
-  half2_t a0 = __builtin_bit_cast(half2_t, ((w << 4) & m) | one);
-  half2_t a1 = __builtin_bit_cast(half2_t, (w & m) | one);
-  half2_t a2 = __builtin_bit_cast(half2_t, ((w >> 4) & m) | one);
-  half2_t a3 = __builtin_bit_cast(half2_t, ((w >> 8) & m) | one);
+  half2_t a0 = __builtin_bit_cast(half2_t, and_or(w << 4, m, one));
+  half2_t a1 = __builtin_bit_cast(half2_t, and_or(w, m, one));
+  half2_t a2 = __builtin_bit_cast(half2_t, and_or(w >> 4, m, one));
+  half2_t a3 = __builtin_bit_cast(half2_t, and_or(w >> 8, m, one));
   acc = __builtin_amdgcn_fdot2(a0, qp[0], acc, false);
   acc = __builtin_amdgcn_fdot2(a1, qp[1], acc, false);
   acc = __builtin_amdgcn_fdot2(a2, qp[2], acc, false);

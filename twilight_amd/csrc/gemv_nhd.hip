@@ -44,14 +44,6 @@ constexpr int kNhdTilePad = 8;  // halves between the rows of the output tile
 // up to 16 different heads at once, and rows a multiple of 256 bytes apart share their banks
 constexpr int kNhdQRow = TWL_HEAD_DIM + 8;
 
-// (x & m) | o in one instruction (the compiler emits the two-instruction form here; one of the
-// two constants has to sit in a vector register: an instruction reads one scalar operand)
-__device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t m, uint32_t o) {
-  uint32_t r;
-  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "s"(m), "v"(o));
-  return r;
-}
-
 template <int KIND>
 __global__ __launch_bounds__(kNhdThreads) void gemv_nhd_kernel(GemvNhdArgs a) {
   constexpr int LPT = KIND == kNhdF16 ? 16 : (KIND == kNhdInt8 ? 8 : 4);  // lanes per token-head

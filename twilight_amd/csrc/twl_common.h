@@ -54,6 +54,15 @@ __device__ __forceinline__ float round_to(float f) {
   return f;
 }
 
+// (x & m) | o in one VALU operation. The compiler splits the expression into v_and + v_or when
+// both constants are literals (a three-operand instruction cannot carry a literal on this
+// target), so the mask travels in a scalar register and `o` in a vector register.
+__device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t m, uint32_t o) {
+  uint32_t r;
+  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "s"(m), "v"(o));
+  return r;
+}
+
 // A query value as the INT4 estimator's fp16 dot products take it. fp16 queries pass unchanged.
 // A bf16 query is converted to fp16: exact for 2^-17 <= |q| <= 65504 (8 significand bits fit 11),
 // rounded to a multiple of 2^-24 below that, and SATURATED to +-65504 above (so that a score can
