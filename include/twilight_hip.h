@@ -243,9 +243,10 @@ int twl_gemv_f16_single(const void* q, void* o, const void* k, uint32_t num_head
  * k_cache / v_cache: element type kv_dtype (TWL_F16 / TWL_BF16, must equal q's type); element
  * (page, token, kv_head, d) lives at page*page_stride + token*token_stride + kv_head*head_stride + d.
  * Rows longer than 128 survivors are split over several workgroups that meet in `workspace`
- * (256-byte aligned, at least twl_sparse_attn_workspace_bytes(rows, idx_stride) bytes). Its first
- * rows*4 bytes are ticket counters that must be zero before the first call; every call leaves
- * them zero again. Two calls that share a workspace must not overlap in time. In a split row the
+ * (256-byte aligned, at least twl_sparse_attn_workspace_bytes(rows, idx_stride) bytes, no initial
+ * contents required: its first rows*4 bytes are ticket words tagged with a per-call number, so a
+ * word left by a call that never finished counts as zero; a finished call leaves them zero).
+ * Two calls that share a workspace must not overlap in time. In a split row the
  * softmax weights are not rounded to the q dtype before the V product (the partial sums are
  * merged in fp32); a row of at most 128 survivors follows the reference rounding exactly.
  * ------------------------------------------------------------------------------------------- */
@@ -265,8 +266,8 @@ int twl_sparse_attn(const void* q, void* out, int dtype, const void* k_cache, co
  * twl_sparse_attn_workspace_bytes(batch * num_q_heads, idx_stride) exceeds that size (24 MiB hold
  * 512 rows of up to 8192 survivors). The first call on a device looks up the array's address
  * there and should happen outside graph capture. All calls on one GPU share the array: calls that
- * overlap in time on one GPU (two streams, two threads) race; the ticket words are cleared by a
- * small kernel on `stream` ahead of the attention kernel. */
+ * overlap in time on one GPU (two streams, two threads) race. Nothing in the array has to be
+ * cleared between calls (the ticket words are tagged per call), so the call is one launch. */
 #define TWL_STATIC_SCRATCH_BYTES (24u << 20)
 int twl_sparse_attn_static(const void* q, void* out, int dtype, const void* k_cache,
                            const void* v_cache, uint64_t page_stride, uint64_t token_stride,

@@ -42,7 +42,7 @@ def sparse_paged_decode_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cach
     ``idx`` int32 [B,H,S] ascending logical token positions, ``count`` int32 [B,H]. Returns
     ``out`` [B,H,128] in q's dtype (and ``lse`` fp32 [B,H] when asked). Probabilities are rounded
     to q's dtype before the V product as at attention.py:302-304 (rows of more than 128 survivors
-    are split over workgroups and merged in fp32 instead). ``workspace`` is a zero-initialised
+    are split over workgroups and merged in fp32 instead). ``workspace`` is a
     uint8 tensor of :func:`attention_workspace_bytes` bytes that calls on one stream may share;
     by default a fresh one is allocated. With ``static_scratch`` (and ``out`` given, ``return_lse``
     off) the call allocates nothing: the split rows meet in a buffer inside the library
@@ -95,7 +95,7 @@ def sparse_paged_decode_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cach
             return (out, lse) if return_lse else out
         need = attention_workspace_bytes(B * H, idx.size(2))
         if workspace is None:
-            workspace = torch.zeros(need, dtype=torch.uint8, device=dev)
+            workspace = torch.empty(need, dtype=torch.uint8, device=dev)
         else:
             check_input(workspace, "workspace"); check_dtype(workspace, torch.uint8, "workspace")
             if workspace.numel() < need or workspace.device != dev:
