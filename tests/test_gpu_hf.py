@@ -266,3 +266,35 @@ def test_fused_rotary_embedding_equals_the_tensor_form(dev, dt):
     assert torch.equal(q3, want_q[:, :, 0]) and torch.equal(k3, want_k[:, :, 0])
     with pytest.raises(RuntimeError):
         K.rope_qk_(q3, k3, cos.float(), sin.float())
+
+
+def test_decode_refuses_a_mask_that_hides_positions_and_takes_a_single_first_token(dev):
+    # the reference asserts the decode-step mask away (twilight/pyimpl/attention.py:186); here a
+    # mask that hides nothing passes, one that hides a position (a left-padded batch) raises, and
+    # a single token with nothing cached is a one-token prefill through the model's own forward
+    model = _tiny_llama(layers=3, heads=4, kv_heads=2, dtype=torch.float16).to(dev)
+    hf.enable_sparse_attention(model, json.loads(json.dumps(CFG)), reserve_tokens=32)
+    ids = torch.randint(0, 97, (2, 40), generator=torch.Generator().manual_seed(5)).to(dev)
+    with torch.no_grad():
+        out = model(ids, use_cache=True)
+        past = out.past_key_values
+        nxt = out.logits[:, -1].argmax(-1, keepdim=True)
+        full = torch.ones((2, 41), dtype=torch.long, device=dev)
+        ok = model(nxt, past_key_values=past, use_cache=True, attention_mask=full)
+        assert torch.isfinite(ok.logits).all()
+        padded = full.clone()
+        padded = torch.cat([padded, torch.ones((2, 1), dtype=torch.long, device=dev)], dim=1)
+        padded[1, :3] = 0
+        with pytest.raises(RuntimeError, match="attention_mask"):
+            model(nxt, past_key_values=ok.past_key_values, use_cache=True, attention_mask=padded)
+    hf.disable_sparse_attention(model)
+    # one token, empty cache: prefill path, then ordinary decode steps
+    model2 = _tiny_llama(layers=3, heads=4, kv_heads=2, dtype=torch.float16).to(dev)
+    from transformers import DynamicCache
+    with torch.no_grad():
+        ref = model2(ids[:, :1], past_key_values=DynamicCache(config=model2.config), use_cache=True)
+        hf.enable_sparse_attention(model2, json.loads(json.dumps(CFG)), reserve_tokens=32)
+        got = model2(ids[:, :1], past_key_values=DynamicCache(config=model2.config), use_cache=True)
+        assert torch.allclose(got.logits.float(), ref.logits.float(), rtol=1e-3, atol=1e-3)
+        step = model2(ids[:, 1:2], past_key_values=got.past_key_values, use_cache=True)
+        assert torch.isfinite(step.logits).all()

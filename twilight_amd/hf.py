@@ -201,13 +201,33 @@ def fill_from_prefill(st: _LayerState, k: torch.Tensor, v: torch.Tensor, num_q_h
     st.layer = TwilightDecodeLayer(st.cache, num_q_heads, reserve_pages=npg + spare_per_req, **st.cfg)
 
 
+_mask_checked = None   # weak reference to the mask the last check passed (one check per step)
+
+
+def _check_mask_hides_nothing(mask) -> None:
+    """Raise for a decode-step attention mask that hides a position. Every layer of a step gets
+    the same tensor, so the (synchronising) look at its values happens once per step."""
+    global _mask_checked
+    if _mask_checked is not None and _mask_checked() is mask:
+        return
+    hides = (~mask).any() if mask.dtype == torch.bool else (mask < 0).any()
+    if bool(hides):
+        raise RuntimeError("the Select-then-Prune decode step cannot honour an attention_mask "
+                           "that hides positions (padded batches are not supported)")
+    import weakref
+    _mask_checked = weakref.ref(mask)
+
+
 def _twilight_attention_forward(self, hidden_states, position_embeddings=None, attention_mask=None,
                                 past_key_values=None, **kwargs):
     """Replacement of ``LlamaAttention.forward``: the module's own forward for prefill, the
     Select-then-Prune layer for decode (twilight/pyimpl/attention.py:59-306 split the same way)."""
     st: _LayerState = self._twilight_state
     q_len = hidden_states.shape[1]
-    if q_len > 1 or past_key_values is None:
+    # a single token with nothing cached yet is a (one-token) prefill, not a decode step
+    first_token = (past_key_values is not None and st.cache is None and st.seq_len == 0
+                   and past_key_values.get_seq_length(self.layer_idx) == 0)
+    if q_len > 1 or past_key_values is None or first_token:
         if past_key_values is None or past_key_values.get_seq_length(self.layer_idx) == 0:
             st.reset()                                    # a new sequence starts
         out = self._twilight_orig_forward(hidden_states, position_embeddings=position_embeddings,
@@ -216,6 +236,12 @@ def _twilight_attention_forward(self, hidden_states, position_embeddings=None, a
         st.seq_len += q_len
         st.cache = st.layer = None                        # paged lazily at the next decode step
         return out
+    if attention_mask is not None and not st.recorded:
+        # The paged path attends to every cached position of every request, as the reference's
+        # decode branch does (it asserts the mask away, twilight/pyimpl/attention.py:186): a mask
+        # that hides positions (a left-padded batch) cannot be honoured, so it is refused rather
+        # than ignored. Masks that hide nothing pass.
+        _check_mask_hides_nothing(attention_mask)
     if st.cache is None:
         # first decode step after a prefill (possibly a prefill that ran before patching): page
         # the K / V the model's own cache holds for this layer
