@@ -128,7 +128,12 @@ __device__ __forceinline__ void estimate_prune_row(const FusedArgs& a, FusedSmem
 
   // ---- stream the run: scores into x[] --------------------------------------------------------
   const size_t rec_stride = (size_t)a.num_kv_heads * TWL_INT4_RECORD_BYTES;
-  const uint8_t* base = a.k_int4 + (size_t)kvh * TWL_INT4_RECORD_BYTES + 16 * lane;
+  // record address = (wave-uniform pointer) + (lane offset): the uniform half is computed on the
+  // scalar unit and a load needs one 32-bit vector register for its address instead of two per
+  // page in flight
+  const uint8_t* sbase = a.k_int4 + (size_t)kvh * TWL_INT4_RECORD_BYTES;
+  const uint32_t nib_off = 16u * (uint32_t)lane;
+  const uint32_t sz_off = 1024u + 4u * (uint32_t)lane;
   const float ninf = -__builtin_inff();
   float x[VPT];
 #pragma unroll
@@ -141,15 +146,19 @@ __device__ __forceinline__ void estimate_prune_row(const FusedArgs& a, FusedSmem
       u32x4 nib[4];
       uint32_t sz[4];
       int logical[4];
+      // (the empty asm keeps the widening of the lane offsets inside this block, next to the
+      // loads, which is what lets them take the scalar base + 32-bit vector offset form)
+      uint32_t o16 = nib_off, o4 = sz_off;
+      asm volatile("" : "+v"(o16), "+v"(o4));
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
         // entries past the list reuse the group's first entry: a valid address, result discarded
         const int src = (i0 + u < n_pages) ? (4 * (g % 16) + u) : (4 * (g % 16));
         const int phys = __builtin_amdgcn_readlane(my_phys[r], src);
         logical[u] = __builtin_amdgcn_readlane(my_logical[r], src);
-        const uint8_t* rec = base + (size_t)phys * rec_stride;
-        nib[u] = __builtin_nontemporal_load((const u32x4*)rec);
-        sz[u] = __builtin_nontemporal_load((const uint32_t*)(rec + 1024 - 12 * lane));
+        const uint8_t* rec = sbase + (size_t)(uint32_t)phys * rec_stride;   // wave-uniform
+        nib[u] = __builtin_nontemporal_load((const u32x4*)(rec + o16));
+        sz[u] = __builtin_nontemporal_load((const uint32_t*)(rec + o4));
       }
       float mine = ninf;
 #pragma unroll
