@@ -14,7 +14,9 @@ the kernel with the largest HBM term (the Quest metadata stream); ``kernels`` li
 the layer with its algorithmic bytes, time and fraction of the 8 TB/s peak, and ``gemv_cfg2`` the
 stand-alone INT4 GEMV at 8 x 32 x 32768 candidates. ``cfg4_b16`` (the same layer at batch 16) and
 ``cfg5_layer`` (32 q heads on 8 kv heads, bf16, p 0.9, with the dense paged decode beside it) are
-the other two layer shapes of the headline figure, measured the same way with fewer steps.
+the other two layer shapes of the headline figure, measured the same way with fewer steps, and
+``cfg5_model`` is the whole 32-layer model at that shape (random weights, tokens/s, 8 decode steps
+replayed from one HIP graph, against the model's own dense decode).
 ``cpu_baseline`` is the CPU oracle (a port of the reference's torch path) timed on this host on
 one of the 8 batch elements and scaled by 8, plus the reference's own CPU case (B=1, context 4096)
 with warm-ups, repeats, median and per-stage times.
@@ -292,7 +294,7 @@ def bench_ftka(args, dev) -> int:
     return 0
 
 
-def bench_llama3_model(args, dev) -> int:
+def bench_llama3_model(args, dev, emit: bool = True):
     """Whole-model decode at the Llama-3-8B shape: every layer of a random-initialised model
     (GQA 32 / 8 heads, bf16), B requests with a synthetic context of N tokens already in the
     caches, decode steps timed end to end — once dense (torch SDPA over a static KV cache) and once
@@ -429,7 +431,8 @@ def bench_llama3_model(args, dev) -> int:
               position_ids=torch.full((B, 1), N + steps + warmup, device=dev))
     torch.cuda.synchronize()
     layer_us = sum(a.elapsed_time(b) for a, b in ev) * 1e3 / max(len(ev), 1)
-    print(json.dumps({
+    hf.disable_sparse_attention(model)
+    line = {
         "metric": "tokens/s, whole-model decode with Twilight applied", "value": round(B / twi_ms * 1e3, 1),
         "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": round(twi_ms, 3), "higher_is_better": True, "scaling": "weak",
@@ -452,8 +455,13 @@ def bench_llama3_model(args, dev) -> int:
         "kept_tokens_per_head_mean": round(kept, 1),
         "twilight_layer_us": round(layer_us, 1),
         "finite_logits": bool(torch.isfinite(logits).all()),
-    }))
-    return 0
+    }
+    del model, cache, states
+    torch.cuda.empty_cache()
+    if emit:
+        print(json.dumps(line))
+        return 0
+    return line
 
 
 class _Timed:
@@ -910,6 +918,15 @@ def main() -> int:
                                           args.top_p, 2, es, ew)
         extra["cfg5_layer"] = measure_shape(L, dev, 8, 32, 8, N, torch.bfloat16, args.budget, 0.9,
                                             4, es, ew, dense=True)
+        # the whole model at that shape (32 layers, random weights), a few decode steps: tokens/s
+        # of the patched model replayed from one HIP graph against the model's own dense decode
+        margs = argparse.Namespace(**vars(args))
+        margs.steps, margs.warmup, margs.top_p, margs.model_mode, margs.no_dense = 8, 2, 0.9, "paged+graph", False
+        m = bench_llama3_model(margs, dev, emit=False)
+        extra["cfg5_model"] = {k: m[k] for k in ("config", "value", "unit", "ms_per_step", "steps",
+                                                 "dense", "speedup_vs_dense",
+                                                 "kept_tokens_per_head_mean", "twilight_layer_us",
+                                                 "finite_logits")}
 
     cpu = None
     if not args.no_cpu_baseline and not llama:

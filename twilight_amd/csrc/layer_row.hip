@@ -118,19 +118,13 @@ __global__ __launch_bounds__(kRowThreads) void select_estimate_prune_kernel(RowA
         const int pg0 = w0 + 2 * lane;                 // this lane's two pages
         const int pgc = min(pg0, (int)a.plane_cap - 2);  // loads stay inside the run
         float s0 = 0.0f, s1 = 0.0f;
-        // run address = wave-uniform pointer + this lane's byte offset (kept in one 32-bit
-        // register; the empty asm keeps its widening inside this block, next to the loads)
-        uint32_t lane_off = 2u * (uint32_t)pgc;
-        asm volatile("" : "+v"(lane_off));
 #pragma unroll 16
         for (int d = 0; d < TWL_HEAD_DIM; ++d) {
-          const int qbits = __builtin_amdgcn_readlane(as_i32(d < 64 ? q_lo : q_hi), d & 63);
-          const float qd = as_f32(qbits);
-          // max run for q_d > 0, else min run; a float is > 0 exactly when its bit pattern is a
-          // positive integer, and that comparison runs on the scalar unit
-          const int plane = qbits > 0 ? 1 : 0;
-          const uint8_t* run = (const uint8_t*)(pl + (size_t)(2 * d + plane) * a.plane_cap);
-          const uint32_t w = __builtin_nontemporal_load((const uint32_t*)(run + lane_off));
+          const float qd =
+              as_f32(__builtin_amdgcn_readlane(as_i32(d < 64 ? q_lo : q_hi), d & 63));
+          const int plane = qd > 0.0f ? 1 : 0;         // max run for q_d > 0, else min run
+          const uint32_t w = __builtin_nontemporal_load(
+              (const uint32_t*)(pl + (size_t)(2 * d + plane) * a.plane_cap + pgc));
           s0 = fmaf(qd, bits16_to_f32<QDT>(w & 0xFFFFu), s0);
           s1 = fmaf(qd, bits16_to_f32<QDT>(w >> 16), s1);
         }
