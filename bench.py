@@ -186,13 +186,36 @@ def bench_topp(args, L, dev) -> int:
         res[str(p)] = {"us": round(us, 2), "survivors_median": float(sv.median()),
                        "survivors_mean": round(float(sv.mean()), 1), "survivors_max": int(sv.max()),
                        "bytes": nbytes, "GBps": round(nbytes / us / 1e3, 1)}
+    # the drop-in mask ops on normalised probabilities (top_p_fp32_return_mask /
+    # top_p_fp16_return_mask, high = probs[..., 0] as the reference has it, token 0 the maximum)
+    xs1 = [synth.topp_scores(B, H, M, seed=100 * i + 7, max_spikes=512, first_is_max=True).to(dev)
+           for i in range(4)]
+    masks = {}
+    mask = torch.empty((rows, M), dtype=torch.uint8, device=dev)
+    for name, dt in (("fp32", torch.float32), ("fp16", torch.float16), ("bf16", torch.bfloat16)):
+        ps = [torch.softmax(x, -1).to(dt).contiguous() for x in xs1]
+        state = {"i": 0}
+
+        def call_mask():
+            pr = ps[state["i"] % 4]
+            state["i"] += 1
+            if dt == torch.float32:
+                L.twl_top_p_f32(pr.data_ptr(), mask.data_ptr(), 0, 0, 0, 0.95, rows, M, M, 0, 0, 0, stream)
+            else:
+                L.twl_top_p_f16(pr.data_ptr(), 0 if dt == torch.float16 else 1, mask.data_ptr(), 0, 0, 0,
+                                0.95, rows, M, M, 0, 0, 0, stream)
+        masks[name] = round(_time_calls(call_mask, args.steps, args.warmup), 2)
     line = {"metric": "us/top-p call (softmax + top-p + compaction)", "value": res["0.95"]["us"],
             "unit": "us", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
             "ms_per_step": round(res["0.95"]["us"] / 1e3, 5), "higher_is_better": False,
             "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
             "config": {"workload": "top-p pruner alone, fp32 scores [8, 32, 8192], Zipf(1.2) spike "
                                    "sets of 1-512 tokens per row, high = row max"},
-            "per_p": res}
+            "per_p": res,
+            "mask_ops_us_p095": masks,
+            "mask_ops_what": "twl_top_p_f32 / twl_top_p_f16 on [8, 32, 8192] probabilities writing "
+                             "the byte mask; the 16-bit forms run the reference's 16-bit arithmetic "
+                             "in cub::BlockReduce's order (1024 threads per row)"}
     print(json.dumps(line))
     return 0
 
