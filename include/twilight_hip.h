@@ -80,7 +80,7 @@ enum twl_top_p_high {
 const char* twl_strerror(int status);
 /* ABI version of this header; bumps when a signature changes. twl_abi_version() returns the
  * version the library was built with: a caller compares the two before anything else. */
-#define TWL_ABI_VERSION 8
+#define TWL_ABI_VERSION 9
 int twl_abi_version(void);
 /* Number of HIP devices visible, or a negative twl_status. */
 int twl_device_count(void);
@@ -275,6 +275,25 @@ int twl_sparse_attn_static(const void* q, void* out, int dtype, const void* k_ca
                            const int32_t* count, const int32_t* kv_page_indices,
                            const int32_t* kv_page_indptr, uint32_t batch, uint32_t num_q_heads,
                            uint32_t num_kv_heads, float sm_scale, float* lse_out, void* stream);
+
+/* Attention over the survivor lists with GIVEN weights in place of the q.K logits.
+ * Replaces: twilight/pyimpl/attention.py:295-296 (use_estimated_weights_in_attn: the estimator's
+ * logits stand in for the exact ones) followed by the masked softmax.V of :299-306. The softmax
+ * over the survivors of the estimator's logits equals the estimator's candidate probabilities
+ * renormalised over the survivors, so the weights are those probabilities:
+ *   out[row] = sum_j w[row, j] * V[idx[row, j]] / sum_j w[row, j],   j < count[row]
+ * weights: float [batch * num_q_heads, idx_stride], entry j beside idx[row, j]; negative values
+ * count as zero; a row whose weights sum to zero gives NaN, as a softmax over nothing does.
+ * Neither q nor K is read. Rounding as in twl_sparse_attn: in a row of at most 128 survivors the
+ * normalised weights are rounded to `dtype` before the V product (attention.py:302-304), longer
+ * rows keep fp32. lse_out (nullable) receives log(sum_j w[row, j]). Workspace as twl_sparse_attn. */
+int twl_sparse_attn_weighted(void* out, int dtype, const void* v_cache, uint64_t page_stride,
+                             uint64_t token_stride, uint64_t head_stride, const int32_t* idx,
+                             uint32_t idx_stride, const int32_t* count, const float* weights,
+                             const int32_t* kv_page_indices, const int32_t* kv_page_indptr,
+                             uint32_t batch, uint32_t num_q_heads, uint32_t num_kv_heads,
+                             float* lse_out, void* workspace, uint64_t workspace_bytes,
+                             void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Paged decode attention with ONE token list per (request, kv head), shared by the kv head's
@@ -515,6 +534,13 @@ typedef struct twl_layer_args {
   int32_t* group_idx; uint32_t group_idx_stride;
   int32_t* group_count;
   void* group_workspace; uint64_t group_workspace_bytes;
+  /* use_estimated_weights != 0: the attention takes the estimator's weights instead of exact q.K
+   * logits (use_estimated_weights_in_attn, attention.py:295-296; see twl_sparse_attn_weighted).
+   * surv_probs: float [rows, idx_stride], required then; it receives the estimator's probability
+   * of every survivor beside idx. Whenever surv_probs is given it is filled, whatever the flag.
+   * Not available together with group_idx. */
+  float* surv_probs;
+  int use_estimated_weights;
 } twl_layer_args;
 
 int twl_decode_layer(const twl_layer_args* args, void* stream);

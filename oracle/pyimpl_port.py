@@ -13,7 +13,10 @@ How each function is pinned (tests/test_oracle_*.py):
   estimator_scores       reduces to a float64 matmul (library routine)
   top_p_unnormalized     softmax is torch's; the bisection is oracle.native.top_p_mask_f32
                          (pinned against the textbook nucleus set and brute force)
-  masked_attention       reduces to softmax + matmul over gathered survivors (checked both ways)
+  masked_attention       reduces to softmax + matmul over gathered survivors (checked both ways),
+                         also with given logits (use_estimated_weights_in_attn); a K the 4-bit
+                         grid holds exactly makes both attention modes of decode_layer_dense meet
+  sparsity_rate          closed forms of the budget rule: rate 1 keeps all, rate 0 one chunk
   get_label_tensor_ref, bgemv_int8_ref
                          the reference's own torch checks (channel.py:82-110, bgemv_int8.py:78-93),
                          i.e. a gather and a matmul
@@ -208,14 +211,19 @@ def top_p_unnormalized(weights: torch.Tensor, threshold, high_mode: int = native
 # a-7  attention over the surviving tokens, dense-masked form
 # --------------------------------------------------------------------------------------------
 def masked_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: torch.Tensor,
-                     prob_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+                     prob_dtype: torch.dtype = torch.float32,
+                     logits: Optional[torch.Tensor] = None) -> torch.Tensor:
     """twilight/pyimpl/attention.py:188-190,299-306 with every tensor held in fp32 on the CPU.
 
     ``prob_dtype`` is the reference's ``query_states.dtype`` to which the probabilities are cast
-    (attention.py:302-304) before the V product. Returns fp32 [B,H,1,D].
+    (attention.py:302-304) before the V product. ``logits`` [B,H,1,N], when given, take the place
+    of q.K/sqrt(D) (attention.py:295-296, use_estimated_weights_in_attn). Returns fp32 [B,H,1,D].
     """
     D = q.shape[-1]
-    w = torch.matmul(q.float(), k.float().transpose(2, 3)) / math.sqrt(D)     # attention.py:188-190
+    if logits is not None:
+        w = logits.float().clone()                                            # attention.py:295-296
+    else:
+        w = torch.matmul(q.float(), k.float().transpose(2, 3)) / math.sqrt(D)  # attention.py:188-190
     w = w.masked_fill(~mask, torch.finfo(torch.float32).min)                  # attention.py:299
     pr = torch.nn.functional.softmax(w, dim=-1, dtype=torch.float32)          # attention.py:302
     pr = pr.to(prob_dtype).float()                                            # attention.py:302-304
@@ -229,7 +237,8 @@ def decode_layer_dense(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, top
                        token_budget: Optional[int] = None, chunk_size: int = PAGE,
                        high_mode: int = native.HIGH_MAX, quant: str = "storage",
                        prob_dtype: torch.dtype = torch.float32, k_deq: Optional[torch.Tensor] = None,
-                       mask0: Optional[torch.Tensor] = None):
+                       mask0: Optional[torch.Tensor] = None, sparsity_rate: float = -1,
+                       use_estimated_weights: bool = False):
     """twilight/pyimpl/attention.py:188-306 for one decode step.
 
     q [B,H,1,D], k/v [B,H,N,D] (K already repeated per q head, attention.py:124-126).
@@ -238,10 +247,14 @@ def decode_layer_dense(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, top
     ``k_deq`` may carry a pre-dequantised K (variant B of the CPU baseline: quantise on append).
     ``mask0`` bool [B,H,1,N] replaces the selector's result (tests use it to follow the later
     stages on a selection that differs from the oracle's only by pages tied at the k-th score).
+    ``sparsity_rate`` != -1 replaces the budget by int(N * rate) (quest.py:45-46);
+    ``use_estimated_weights`` makes the attention use the estimator's logits (attention.py:295-296).
     Returns dict(scores, mask0, probs, pruned, mask, out, low, iters).
     """
     B, H, _, D = q.shape
     N = k.shape[-2]
+    if sparsity_rate != -1:
+        token_budget = int(N * sparsity_rate)                                 # quest.py:45-46
     if mask0 is not None:
         assert mask0.shape == (B, H, 1, N) and mask0.dtype == torch.bool
     elif token_budget is None:
@@ -257,7 +270,8 @@ def decode_layer_dense(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, top
     est = est.masked_fill(~mask0, torch.finfo(torch.float32).min)             # attention.py:255
     pruned, probs, low, iters = top_p_unnormalized(est, top_p, high_mode)     # attention.py:274-278
     mask = mask0 & pruned                                                     # attention.py:280-281
-    out = masked_attention(q, k, v, mask, prob_dtype)                         # attention.py:295-306
+    out = masked_attention(q, k, v, mask, prob_dtype,                         # attention.py:295-306
+                           logits=est if use_estimated_weights else None)
     return dict(scores=est, mask0=mask0, probs=probs, pruned=pruned, mask=mask, out=out,
                 low=low, iters=iters)
 

@@ -93,6 +93,13 @@ def test_c_level_validation_without_gpu(hip_lib):
     assert L.twl_sparse_attn_workspace_bytes(512, 8192) <= _lib.STATIC_SCRATCH_BYTES
     assert L.twl_sparse_attn_static(fake, fake, 0, fake, fake, 4096, 256, 128, fake, 8192, fake,
                                     fake, fake, 128, 32, 32, 1.0, 0, 0) == -7   # 4096 rows: too big
+    # attention on given weights: weights and workspace required, V strides and sizes as above
+    wat = lambda **kw: L.twl_sparse_attn_weighted(
+        kw.get("out", fake), 0, fake, 4096, 256, kw.get("hs", 128), fake, kw.get("stride", 8), fake,
+        kw.get("w", fake), fake, fake, 1, 1, 1, 0, kw.get("ws", fake), kw.get("wsb", ws), 0)
+    assert wat(w=0) == -1 and wat(ws=0) == -1 and wat(out=0) == -1
+    assert wat(hs=130) == -4 and wat(w=fake + 2) == -4
+    assert wat(stride=0) == -2 and wat(wsb=ws - 1) == -2
     assert L.twl_quest_select(fake, 0, fake, fake, fake, 1, 1, 1, 0, 4, fake, 4, fake, fake, 4, 0) == -2
     assert L.twl_quest_select(fake, 0, fake, fake, fake, 1, 1, 1, 64, 4, fake, 2, fake, fake, 4, 0) == -2
     assert L.twl_quest_select(fake, 0, fake, fake, fake, 1, 1, 1, 64, 4, 0, 4, fake, fake, 4, 0) == -1
@@ -183,7 +190,14 @@ def test_sparse_config_parsing():
            "weight_estimator": {"type": "min_max_quant", "quant_bit": 4},
            "weight_pruner": {"type": "top_p", "threshold": 0.85},
            "skip_first_two_layers": True, "use_estimated_weights_in_attn": False}
-    assert parse_sparse_config(cfg) == {"token_budget": 8192, "top_p": 0.85}
+    assert parse_sparse_config(cfg) == {"token_budget": 8192, "top_p": 0.85, "sparsity_rate": -1,
+                                        "use_estimated_weights": False}
+    knobs = dict(cfg, use_estimated_weights_in_attn=True,
+                 selector={"type": "quest", "sparsity_rate": 0.25, "chunk_size": 16})
+    assert parse_sparse_config(knobs)["sparsity_rate"] == 0.25
+    assert parse_sparse_config(knobs)["use_estimated_weights"] is True
+    with pytest.raises(RuntimeError, match="sparsity_rate"):
+        parse_sparse_config(dict(cfg, selector={"type": "quest", "sparsity_rate": 1.5}))
     bad = dict(cfg, selector={"type": "ds"})
     with pytest.raises(RuntimeError):
         parse_sparse_config(bad)

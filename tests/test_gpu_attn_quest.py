@@ -93,6 +93,46 @@ def test_sparse_attention_vs_masked_reference(dev, dt):
     assert torch.allclose(lse.cpu()[rows], ref_lse[rows], rtol=1e-5, atol=1e-5)
 
 
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16])
+def test_weighted_attention_vs_closed_form(dev, dt):
+    """Given weights in place of q.K logits (attention.py:295-296): out = sum w V / sum w over
+    the listed tokens, for rows of one survivor, a few, exactly 128, and thousands (split rows)."""
+    B, H, Hkv, N = 2, 8, 2, 3000
+    g = torch.Generator().manual_seed(14)
+    k = torch.randn((B, Hkv, N, 128), generator=g).to(dt)
+    v = torch.randn((B, Hkv, N, 128), generator=g).to(dt)
+    npg = (N + 15) // 16
+    cache = PagedKVCache.from_dense(k, v, dev, page_perm=torch.randperm(B * npg, generator=g))
+    counts = [1, 0, 7, 128, 129, 1000, N, 300, 64, 2, 2999, 257, 5, 90, 511, 12]
+    idx = torch.zeros((B, H, N), dtype=torch.int32)
+    w = torch.rand((B, H, N), generator=g) ** 4 + 1e-6
+    for r, n in enumerate(counts):
+        idx[r // H, r % H, :n] = torch.sort(torch.randperm(N, generator=g)[:n]).values.int()
+    cnt = torch.tensor(counts, dtype=torch.int32).reshape(B, H)
+    out, lse = K.weighted_paged_decode_attention(w.to(dev), cache.v_cache, idx.to(dev), cnt.to(dev),
+                                                 cache.kv_page_indices, cache.kv_page_indptr,
+                                                 return_lse=True)
+    got = out.cpu().double()
+    vrep = v.double().repeat_interleave(H // Hkv, dim=1)
+    tol = 1e-3 if dt == torch.float16 else 8e-3
+    for r, n in enumerate(counts):
+        b, h = r // H, r % H
+        if n == 0:
+            assert torch.all(got[b, h] == 0)
+            continue
+        ww = w[b, h, :n].double()
+        pr = ww / ww.sum()
+        if n <= 128:
+            pr = pr.float().to(dt).double()                                # attention.py:302-304
+        ref = pr @ vrep[b, h, idx[b, h, :n].long()]
+        assert torch.allclose(got[b, h], ref, rtol=tol, atol=tol), (r, n)
+        assert abs(float(lse[b, h]) - math.log(float(ww.sum()))) < 1e-4
+    # the same lists a second time on the same workspace words
+    out2 = K.weighted_paged_decode_attention(w.to(dev), cache.v_cache, idx.to(dev), cnt.to(dev),
+                                             cache.kv_page_indices, cache.kv_page_indptr)
+    assert torch.allclose(out2.float(), out.float(), rtol=tol, atol=tol)
+
+
 def test_sparse_attention_hnd_layout_view(dev):
     # the same kernel over an HND-stored cache ([pages, Hkv, 16, 128] viewed as [pages,16,Hkv,128])
     g = torch.Generator().manual_seed(6)

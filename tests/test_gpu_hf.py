@@ -63,6 +63,31 @@ def test_decode_with_p_one_equals_dense_decode(dev, kv_heads):
     assert torch.allclose(again, ref_logits, rtol=1e-3, atol=1e-3)
 
 
+def test_decode_with_estimated_weights_and_sparsity_rate(dev):
+    """use_estimated_weights_in_attn and selector.sparsity_rate through the model patch: with
+    everything kept the estimator's weights move the logits only by the 4-bit error, and the
+    reported selector budget follows the context length."""
+    model = _tiny_llama(layers=4, heads=4, kv_heads=2, dtype=torch.float16).to(dev)
+    ids = torch.randint(0, 97, (2, 200), generator=torch.Generator().manual_seed(5)).to(dev)
+    ref_logits, toks = _decode(model, ids, 4)
+    cfg = json.loads(json.dumps(CFG))
+    cfg["selector"] = {"type": "quest", "sparsity_rate": 0.5, "chunk_size": 16}
+    cfg["weight_pruner"]["threshold"] = 1.0
+    cfg["use_estimated_weights_in_attn"] = True
+    info, _ = hf.enable_sparse_attention(model, cfg, enable_budget_info=True, reserve_tokens=32)
+    got = _forced_decode(model, ids, toks)
+    assert torch.isfinite(got).all()
+    cos = torch.nn.functional.cosine_similarity(got.flatten(1), ref_logits.flatten(1), dim=1)
+    assert float(cos.min()) > 0.8
+    assert info.get_avg_budget_per_query_B0() == [float(int((201 + s) * 0.5)) for s in range(4)]
+    hf.disable_sparse_attention(model)
+    # a recorded step would freeze the first budget: refused
+    hf.enable_sparse_attention(model, cfg, reserve_tokens=32, dense_layers="paged", keep_hf_cache=False)
+    with pytest.raises(RuntimeError, match="sparsity_rate"):
+        hf.GraphedDecodeStep(model)
+    hf.disable_sparse_attention(model)
+
+
 def test_decode_prunes_and_reports_budgets(dev):
     model = _tiny_llama(layers=4, heads=4, kv_heads=2, dtype=torch.float16).to(dev)
     ids = torch.randint(0, 97, (3, 333), generator=torch.Generator().manual_seed(3)).to(dev)

@@ -47,7 +47,7 @@ def _assert_selection_ties(page_scores, gpu_pages, ora_mask0, npg):
 
 
 def _run_case(dev, B, H, Hkv, N, budget, p, dt, seed, shuffle=True, n_heavy=16, fused=True,
-              planes=False):
+              planes=False, rate=-1, use_est=False):
     q, k, v = synth.heavy_hitter_qkv(B, H, N, n_heavy=n_heavy, mass=0.6, seed=seed, dtype=dt)
     group = H // Hkv
     kk, vv = k[:, ::group].contiguous(), v[:, ::group].contiguous()        # one K/V per kv head
@@ -56,12 +56,16 @@ def _run_case(dev, B, H, Hkv, N, budget, p, dt, seed, shuffle=True, n_heavy=16, 
     cache = PagedKVCache.from_dense(kk.to(dt), vv.to(dt), dev, page_perm=perm,
                                     plane_pages=npg if planes else None)
     layer = TwilightDecodeLayer(cache, H, token_budget=budget, top_p=p, high="max",
-                                fused_estimator=fused, keep_scores=True)
+                                fused_estimator=fused, keep_scores=True, sparsity_rate=rate,
+                                use_estimated_weights=use_est)
+    if rate != -1:
+        budget = int(N * rate)                                              # quest.py:45-46
     out = layer(q[:, :, 0].to(dt).to(dev)).cpu().float()
     krep = kk.repeat_interleave(group, dim=1)                               # attention.py:124-126
     vrep = vv.repeat_interleave(group, dim=1)
     ref = P.decode_layer_dense(q, krep, vrep, top_p=p, token_budget=budget if budget < N else None,
-                               high_mode=native.HIGH_MAX, quant="storage", prob_dtype=dt)
+                               high_mode=native.HIGH_MAX, quant="storage", prob_dtype=dt,
+                               sparsity_rate=rate, use_estimated_weights=use_est)
     rows = B * H
     # 1. selector: the oracle's pages, except pages whose score ties the k-th within rounding
     #    (checked on the oracle's own page scores); the later stages are then followed on the
@@ -76,7 +80,7 @@ def _run_case(dev, B, H, Hkv, N, budget, p, dt, seed, shuffle=True, n_heavy=16, 
         for r in differ:
             _assert_selection_ties(est_pg[r], sel[r, :selc[r]], mask0[r], npg)
         ref = P.decode_layer_dense(q, krep, vrep, top_p=p, token_budget=budget, high_mode=native.HIGH_MAX,
-                                   quant="storage", prob_dtype=dt,
+                                   quant="storage", prob_dtype=dt, use_estimated_weights=use_est,
                                    mask0=torch.from_numpy(gmask0).reshape(B, H, 1, N))
     # 2. estimator scores on the selected candidates (1e-3 relative)
     scores = layer.scores.cpu().numpy().reshape(rows, -1)
@@ -98,7 +102,13 @@ def _run_case(dev, B, H, Hkv, N, budget, p, dt, seed, shuffle=True, n_heavy=16, 
                         margin_tol=5e-6)
     # 4. attention: exact over the GPU's own survivors, and end to end against the oracle
     tol = 1e-3 if dt == torch.float16 else 8e-3
-    own = P.masked_attention(q, krep, vrep, torch.from_numpy(gm).reshape(B, H, 1, N), prob_dtype=dt)
+    if use_est:
+        # the estimator's probability of every survivor, in list order beside idx
+        sp = layer.surv_probs.cpu().numpy().reshape(rows, -1)
+        for r in range(rows):
+            np.testing.assert_allclose(sp[r, :cnt[r]], probs[r, idx[r, :cnt[r]]], rtol=1e-4, atol=1e-9)
+    own = P.masked_attention(q, krep, vrep, torch.from_numpy(gm).reshape(B, H, 1, N), prob_dtype=dt,
+                             logits=ref["scores"] if use_est else None)
     assert torch.allclose(out, own[:, :, 0], rtol=tol, atol=tol)
     e2e = (out.reshape(rows, 128) - ref["out"].reshape(rows, 128)).abs().max().item()
     assert e2e < 5 * tol, e2e
@@ -148,6 +158,55 @@ def test_layer_dispatch_regimes(dev, B, H, Hkv, planes):
     metadata layout): every branch gives the oracle's result."""
     _run_case(dev, B, H, Hkv, 512, 128, 0.9, torch.float16, seed=B * H + Hkv, n_heavy=4,
               planes=planes)
+
+
+@pytest.mark.parametrize("B,H,Hkv,N,budget,dt,fused,planes", [
+    (1, 32, 32, 4096, 4096, torch.float16, True, False),   # every token a candidate, few rows
+    (8, 32, 32, 1024, 256, torch.float16, True, True),     # the one-launch row kernel
+    (20, 32, 32, 512, 128, torch.bfloat16, True, False),   # estimator + pruner in one launch
+    (2, 8, 2, 2048, 512, torch.bfloat16, False, False),    # every stage its own launch, GQA
+    (3, 4, 4, 1000, 250, torch.float16, True, False),      # ragged, budget not a page multiple
+])
+def test_layer_attention_on_estimated_weights(dev, B, H, Hkv, N, budget, dt, fused, planes):
+    """use_estimated_weights_in_attn (attention.py:295-296): the survivors' estimator
+    probabilities are emitted beside the index lists and weigh V; K is not read again."""
+    _run_case(dev, B, H, Hkv, N, budget, 0.95, dt, seed=7 * B + H, n_heavy=8, fused=fused,
+              planes=planes, use_est=True)
+
+
+def test_layer_estimated_weights_long_rows(dev):
+    """Rows of more than 128 survivors (flat attention: no heavy tokens, p close to 1) take the
+    split path of the weighted attention and its merge."""
+    layer, _ = _run_case(dev, 2, 8, 8, 4096, 2048, 0.99, torch.float16, seed=5, n_heavy=0,
+                         use_est=True)
+    assert int(layer.count.max()) > 256
+
+
+@pytest.mark.parametrize("N,rate,planes", [(2048, 0.25, False), (1000, 0.13, True), (300, 0.0, False),
+                                           (777, 1.0, False)])
+def test_layer_sparsity_rate(dev, N, rate, planes):
+    """selector.sparsity_rate (quest.py:45-46): the budget follows the context length."""
+    layer, ref = _run_case(dev, 2, 8, 8, N, 99999, 0.9, torch.float16, seed=N, n_heavy=4, planes=planes,
+                           rate=rate)
+    kc = P.quest_chunk_budget(int(N * rate), 16, (N + 15) // 16)
+    assert (layer.sel_count.cpu().numpy() == kc).all()
+
+
+def test_sparsity_rate_follows_appends(dev):
+    """The budget is recomputed from the host-side length every step."""
+    B, H, N = 2, 4, 160
+    q, k, v = synth.heavy_hitter_qkv(B, H, N, n_heavy=2, mass=0.5, seed=3, dtype=torch.float16)
+    k, v = k.half(), v.half()
+    cache = PagedKVCache.from_dense(k, v, dev, spare_pages=8)
+    layer = TwilightDecodeLayer(cache, H, top_p=0.9, sparsity_rate=0.5, reserve_pages=20)
+    qd = q[:, :, 0].half().to(dev)
+    layer(qd)
+    assert (layer.sel_count.cpu().numpy() == 5).all()                 # int(160 * 0.5) = 80 tokens
+    free = list(range(cache.num_pages - 8, cache.num_pages))
+    for _ in range(33):                                               # 193 tokens: budget 96
+        cache.append(k[:, :, 0].to(dev), v[:, :, 0].to(dev), free)
+    layer(qd)
+    assert (layer.sel_count.cpu().numpy() == P.quest_chunk_budget(96, 16, 13)).all()
 
 
 @pytest.mark.parametrize("seed", range(int(os.environ.get("TWL_RANDOM_SHAPES", "12"))))

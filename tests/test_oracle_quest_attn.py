@@ -107,6 +107,52 @@ def test_masked_attention_equals_gathered_softmax():
     assert count.sum() == int(mask.sum()) and idx[0, 0] == 0
 
 
+def test_masked_attention_on_given_logits():
+    """attention.py:295-296: given logits replace q.K. Pinned by the gathered closed form with
+    logits unrelated to q.K, and by logits equal to q.K reproducing the default path."""
+    g = torch.Generator().manual_seed(5)
+    B, H, N, D = 1, 2, 96, 128
+    q = torch.randn((B, H, 1, D), generator=g)
+    k = torch.randn((B, H, N, D), generator=g)
+    v = torch.randn((B, H, N, D), generator=g)
+    logits = torch.randn((B, H, 1, N), generator=g) * 3
+    mask = torch.rand((B, H, 1, N), generator=g) < 0.3
+    mask[..., 5] = True
+    out = P.masked_attention(q, k, v, mask, logits=logits)
+    for h in range(H):
+        sel = mask[0, h, 0].nonzero().squeeze(-1)
+        pr = torch.softmax(logits[0, h, 0, sel].double(), -1)
+        assert torch.allclose(out[0, h, 0].double(), pr @ v[0, h, sel].double(), rtol=1e-5, atol=1e-6)
+    same = P.masked_attention(q, k, v, mask, logits=torch.matmul(q, k.transpose(2, 3)) / math.sqrt(D))
+    assert torch.allclose(same, P.masked_attention(q, k, v, mask), rtol=1e-5, atol=1e-6)
+    assert not torch.allclose(out, same, atol=1e-2)      # the given logits are really used
+
+
+def test_decode_layer_dense_knobs():
+    """sparsity_rate (quest.py:45-46) and use_estimated_weights_in_attn (attention.py:295-296)."""
+    from twilight_amd import synth
+    q, k, v = synth.heavy_hitter_qkv(1, 2, 512, n_heavy=8, mass=0.6, seed=1)
+    # rate 1 keeps everything, rate 0 keeps the one chunk the budget rule never goes below
+    assert P.decode_layer_dense(q, k, v, top_p=0.9, sparsity_rate=1.0)["mask0"].all()
+    assert P.decode_layer_dense(q, k, v, top_p=0.9, sparsity_rate=0.0)["mask0"].sum(-1).unique().tolist() == [16]
+    assert P.decode_layer_dense(q, k, v, top_p=0.9, sparsity_rate=0.26)["mask0"].sum(-1).unique().tolist() == [144]
+    # a K that the 4-bit grid holds exactly: the estimator's logits are the exact ones and the two
+    # attention modes meet
+    g = torch.Generator().manual_seed(2)
+    codes = torch.randint(0, 16, (1, 2, 512, 128), generator=g).float()
+    codes[..., 0::32] = 0
+    codes[..., 1::32] = 15                     # every group of 32 spans the full range
+    kq = codes * 0.125 - 1.0                   # scale 1/8, zero -1: fp16-exact
+    a = P.decode_layer_dense(q, kq, v, top_p=0.9, token_budget=256)
+    b = P.decode_layer_dense(q, kq, v, top_p=0.9, token_budget=256, use_estimated_weights=True)
+    assert torch.equal(a["mask"], b["mask"])
+    assert torch.allclose(a["out"], b["out"], rtol=1e-4, atol=1e-5)
+    # with an inexact K the estimated weights change the result
+    c = P.decode_layer_dense(q, k, v, top_p=0.9, token_budget=256, use_estimated_weights=True)
+    d = P.decode_layer_dense(q, k, v, top_p=0.9, token_budget=256)
+    assert not torch.allclose(c["out"], d["out"], atol=1e-4)
+
+
 def test_decode_layer_dense_consistency():
     from twilight_amd import synth
     q, k, v = synth.heavy_hitter_qkv(1, 2, 512, n_heavy=8, mass=0.6, seed=0)

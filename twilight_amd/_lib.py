@@ -14,7 +14,7 @@ from .build import LIB_PATH
 
 TWL_OK = 0
 TWL_F16, TWL_BF16, TWL_F32 = 0, 1, 2
-ABI_VERSION = 8  # TWL_ABI_VERSION of include/twilight_hip.h, checked when the library is loaded
+ABI_VERSION = 9  # TWL_ABI_VERSION of include/twilight_hip.h, checked when the library is loaded
 TWL_HIGH_FIRST, TWL_HIGH_MAX = 0, 1
 PAGE = 16
 HEAD_DIM = 128
@@ -28,7 +28,8 @@ EXPORTS = (
     "twl_strerror", "twl_abi_version", "twl_device_count", "twl_top_p_f32", "twl_top_p_f16",
     "twl_softmax_top_p_f32", "twl_gemv_top_p", "twl_select_estimate_prune", "twl_gemv_int4", "twl_gemv_int4_nhd",
     "twl_gemv_int8_nhd", "twl_gemv_f16_nhd", "twl_gemv_f16_single", "twl_sparse_attn",
-    "twl_sparse_attn_workspace_bytes", "twl_sparse_attn_static", "twl_group_attn",
+    "twl_sparse_attn_workspace_bytes", "twl_sparse_attn_static", "twl_sparse_attn_weighted",
+    "twl_group_attn",
     "twl_group_attn_workspace_bytes",
     "twl_group_union", "twl_rope_qk", "twl_quest_select",
     "twl_quest_page_scores", "twl_quest_topk_pages", "twl_kv_shadow_build", "twl_kv_append", "twl_meta_planes_build", "twl_quest_page_scores_planes", "twl_dequant_int4",
@@ -61,6 +62,7 @@ class LayerArgs(ctypes.Structure):
         ("group_idx", c_void_p), ("group_idx_stride", c_uint32),
         ("group_count", c_void_p),
         ("group_workspace", c_void_p), ("group_workspace_bytes", c_uint64),
+        ("surv_probs", c_void_p), ("use_estimated_weights", c_int),
     ]
 
 
@@ -107,6 +109,8 @@ def lib() -> ctypes.CDLL:
     L.twl_sparse_attn_workspace_bytes.argtypes = [u32, u32]
     L.twl_sparse_attn_static.argtypes = [vp, vp, i32, vp, vp, u64, u64, u64, vp, u32, vp, vp, vp, u32,
                                          u32, u32, f32, vp, vp]
+    L.twl_sparse_attn_weighted.argtypes = [vp, i32, vp, u64, u64, u64, vp, u32, vp, vp, vp, vp, u32,
+                                           u32, u32, vp, vp, u64, vp]
     L.twl_group_attn_workspace_bytes.argtypes = [u32, u32, u32, u32, i32]
     L.twl_group_attn.argtypes = [vp, vp, i32, vp, vp, u64, u64, u64, vp, u32, vp, u32, vp, vp, vp,
                                  u32, u32, u32, f32, vp, vp, u64, vp]

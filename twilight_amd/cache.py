@@ -87,6 +87,11 @@ class PagedKVCache:
         return self.kv_page_indptr.numel() - 1
 
     # ---- filling ------------------------------------------------------------------------------
+    @property
+    def max_seq_len(self) -> int:
+        """Longest request of the batch in tokens (host-side count, no device read)."""
+        return max(self._seq_lens) if self._seq_lens else 0
+
     def rebuild_shadow(self, page_ids: Optional[torch.Tensor] = None,
                        valid_len: Optional[torch.Tensor] = None) -> None:
         """(Re)build INT4 records and Quest metadata of ``page_ids`` (default: every page, all 16

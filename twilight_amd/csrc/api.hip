@@ -34,6 +34,8 @@ extern "C" int twl_decode_layer(const twl_layer_args* a, void* stream) {
       !a->out)
     return TWL_ENULL;
   if (a->group_idx && (!a->group_count || !a->group_workspace)) return TWL_ENULL;
+  if (a->use_estimated_weights && !a->surv_probs) return TWL_ENULL;
+  if (a->use_estimated_weights && a->group_idx) return TWL_EINVAL;
   if (a->batch == 0 || a->num_q_heads == 0) return TWL_EINVAL;
   const uint32_t rows = a->batch * a->num_q_heads;
   uint32_t k = (a->token_budget / TWL_PAGE ? a->token_budget / TWL_PAGE : 1) +
@@ -69,14 +71,14 @@ extern "C" int twl_decode_layer(const twl_layer_args* a, void* stream) {
                           2u * rows >= (uint32_t)cus && (planes_fit || rows <= 2u * (uint32_t)cus);
   if (row_kernel) {
     // 1+2+3. page scores, top-k pages, INT4 estimate, softmax, top-p, compaction: one launch
-    rc = twl_select_estimate_prune(
+    rc = twl::select_estimate_prune_ex(
         a->q, a->dtype, a->meta, a->k_int4, a->kv_page_indices, a->kv_page_indptr,
         a->kv_last_page_len, a->batch, a->num_q_heads, a->num_kv_heads, a->token_budget,
         a->max_pages_per_req, a->sm_scale, nullptr, a->top_p, a->high_mode, a->sel_pages,
         a->sel_stride, a->sel_count, a->idx, a->idx_stride, a->count,
         a->keep_scores ? a->page_scores : nullptr, a->page_score_stride,
         a->keep_scores ? a->scores : nullptr, a->score_stride, a->cand_count, a->meta_planes,
-        a->plane_cap_pages, a->plane_slots, a->plane_num_slots, stream);
+        a->plane_cap_pages, a->plane_slots, a->plane_num_slots, a->surv_probs, stream);
     if (rc != TWL_OK) return rc;
   } else {
     // 1. Quest page scores + top-k pages; without GQA sharing the plane layout halves the read
@@ -106,12 +108,12 @@ extern "C" int twl_decode_layer(const twl_layer_args* a, void* stream) {
     if (rc != TWL_OK) return rc;
     if (!split) {
       // 2+3. INT4 estimate, softmax, top-p and compaction in one launch
-      rc = twl_gemv_top_p(a->q, a->dtype, a->k_int4, a->sel_pages, a->sel_count, a->sel_stride,
+      rc = twl::gemv_top_p_ex(a->q, a->dtype, a->k_int4, a->sel_pages, a->sel_count, a->sel_stride,
                           a->kv_page_indices, a->kv_page_indptr, a->kv_last_page_len, a->batch,
                           a->num_q_heads, a->num_kv_heads, k, a->sm_scale, nullptr, a->top_p,
                           a->high_mode, a->idx, a->idx_stride, a->count,
                           a->keep_scores ? a->scores : nullptr, a->score_stride, a->cand_count,
-                          nullptr, stream);
+                          nullptr, a->surv_probs, stream);
       if (rc != TWL_OK) return rc;
     } else {
       // 2. INT4 estimate over the selected pages
@@ -121,9 +123,10 @@ extern "C" int twl_decode_layer(const twl_layer_args* a, void* stream) {
                          a->num_kv_heads, k, a->sm_scale, stream);
       if (rc != TWL_OK) return rc;
       // 3. softmax + top-p + compaction to token positions
-      rc = twl_softmax_top_p_f32(a->scores, a->score_stride, a->cand_count, rows, k * TWL_PAGE,
+      rc = twl::softmax_top_p_ex(a->scores, a->score_stride, a->cand_count, rows, k * TWL_PAGE,
                                  nullptr, a->top_p, a->high_mode, a->sel_pages, a->sel_stride,
-                                 a->idx, a->idx_stride, a->count, nullptr, nullptr, stream);
+                                 a->idx, a->idx_stride, a->count, nullptr, nullptr,
+                                 a->surv_probs, stream);
       if (rc != TWL_OK) return rc;
     }
   }
@@ -141,6 +144,12 @@ extern "C" int twl_decode_layer(const twl_layer_args* a, void* stream) {
                           a->sm_scale, nullptr, a->group_workspace, a->group_workspace_bytes,
                           stream);
   }
+  if (a->use_estimated_weights)
+    return twl_sparse_attn_weighted(a->out, a->dtype, a->v_cache, a->page_stride, a->token_stride,
+                                    a->head_stride, a->idx, a->idx_stride, a->count, a->surv_probs,
+                                    a->kv_page_indices, a->kv_page_indptr, a->batch,
+                                    a->num_q_heads, a->num_kv_heads, nullptr, a->attn_workspace,
+                                    a->attn_workspace_bytes, stream);
   return twl_sparse_attn(a->q, a->out, a->dtype, a->k_cache, a->v_cache, a->page_stride,
                          a->token_stride, a->head_stride, a->idx, a->idx_stride, a->count,
                          a->kv_page_indices, a->kv_page_indptr, a->batch, a->num_q_heads,

@@ -54,7 +54,7 @@ static void launch_fused(const FusedArgs& a, uint32_t rows, hipStream_t s) {
 
 }  // namespace twl
 
-extern "C" int twl_gemv_top_p(const void* q, int q_dtype, const void* k_int4,
+int twl::gemv_top_p_ex(const void* q, int q_dtype, const void* k_int4,
                               const int32_t* sel_pages, const int32_t* sel_count,
                               uint32_t sel_stride, const int32_t* kv_page_indices,
                               const int32_t* kv_page_indptr, const int32_t* kv_last_page_len,
@@ -62,7 +62,8 @@ extern "C" int twl_gemv_top_p(const void* q, int q_dtype, const void* k_int4,
                               uint32_t max_pages_per_row, float sm_scale, const float* p_arr,
                               float p, int high_mode, int32_t* idx, uint32_t idx_stride,
                               int32_t* count, float* scores_out, uint32_t score_stride,
-                              int32_t* cand_count, float* low_out, void* stream) {
+                              int32_t* cand_count, float* low_out, float* surv_probs,
+                              void* stream) {
   if (!q || !k_int4 || !sel_pages || !kv_page_indices || !kv_page_indptr || !kv_last_page_len ||
       !idx || !count)
     return TWL_ENULL;
@@ -85,9 +86,24 @@ extern "C" int twl_gemv_top_p(const void* q, int q_dtype, const void* k_int4,
   a.num_kv_heads = num_kv_heads; a.max_pages = max_pages_per_row; a.sm_scale = sm_scale;
   a.p_arr = p_arr; a.p = p; a.high_mode = high_mode; a.idx = idx; a.idx_stride = idx_stride;
   a.count = count; a.scores_out = scores_out; a.score_stride = score_stride;
-  a.cand_count = cand_count; a.low_out = low_out;
+  a.cand_count = cand_count; a.low_out = low_out; a.surv_probs = surv_probs;
   const uint32_t rows = batch * num_q_heads;
   if (q_dtype == TWL_F16) twl::launch_fused<TWL_F16>(a, rows, (hipStream_t)stream);
   else twl::launch_fused<TWL_BF16>(a, rows, (hipStream_t)stream);
   return hipGetLastError() == hipSuccess ? TWL_OK : TWL_ELAUNCH;
+}
+
+extern "C" int twl_gemv_top_p(const void* q, int q_dtype, const void* k_int4,
+                              const int32_t* sel_pages, const int32_t* sel_count,
+                              uint32_t sel_stride, const int32_t* kv_page_indices,
+                              const int32_t* kv_page_indptr, const int32_t* kv_last_page_len,
+                              uint32_t batch, uint32_t num_q_heads, uint32_t num_kv_heads,
+                              uint32_t max_pages_per_row, float sm_scale, const float* p_arr,
+                              float p, int high_mode, int32_t* idx, uint32_t idx_stride,
+                              int32_t* count, float* scores_out, uint32_t score_stride,
+                              int32_t* cand_count, float* low_out, void* stream) {
+  return twl::gemv_top_p_ex(q, q_dtype, k_int4, sel_pages, sel_count, sel_stride, kv_page_indices,
+                            kv_page_indptr, kv_last_page_len, batch, num_q_heads, num_kv_heads,
+                            max_pages_per_row, sm_scale, p_arr, p, high_mode, idx, idx_stride,
+                            count, scores_out, score_stride, cand_count, low_out, nullptr, stream);
 }

@@ -43,6 +43,7 @@ struct FusedArgs {
   uint32_t score_stride;
   int32_t* cand_count; // nullable
   float* low_out;      // nullable
+  float* surv_probs;   // nullable [rows, idx_stride]: estimated probability of survivor j beside idx
 };
 
 // 8 nibbles of one dword against 8 q values held as 4 half2 pairs (n0,n4),(n1,n5),(n2,n6),(n3,n7);
@@ -230,6 +231,7 @@ __device__ __forceinline__ void estimate_prune_row(const FusedArgs& a, FusedSmem
     }
   }
   int32_t* dst = a.idx + (size_t)row * a.idx_stride;
+  float* wdst = a.surv_probs ? a.surv_probs + (size_t)row * a.idx_stride : nullptr;
 #pragma unroll
   for (int g = 0; g < VPT; ++g) {
     const bool keep = x[g] > low;
@@ -238,7 +240,11 @@ __device__ __forceinline__ void estimate_prune_row(const FusedArgs& a, FusedSmem
       const int r = g / 16;
       // logical page of list entry e0 + 4g + l%4 lives in lane 4*(g%16) + l%4 of my_logical[r]
       const int lp = __builtin_amdgcn_ds_bpermute(4 * (4 * (g % 16) + g4), my_logical[r]);
-      if (keep) dst[pos + __builtin_popcountll(bal & before_mask)] = lp * TWL_PAGE + t;
+      if (keep) {
+        const int at = pos + __builtin_popcountll(bal & before_mask);
+        dst[at] = lp * TWL_PAGE + t;
+        if (wdst) wdst[at] = x[g];
+      }
       pos += __builtin_popcountll(bal);
     }
   }

@@ -268,7 +268,7 @@ static void launch_row(const RowArgs& a, uint32_t rows, hipStream_t s) {
 
 }  // namespace twl
 
-extern "C" int twl_select_estimate_prune(
+int twl::select_estimate_prune_ex(
     const void* q, int dtype, const void* meta, const void* k_int4, const int32_t* kv_page_indices,
     const int32_t* kv_page_indptr, const int32_t* kv_last_page_len, uint32_t batch,
     uint32_t num_q_heads, uint32_t num_kv_heads, uint32_t token_budget,
@@ -276,7 +276,8 @@ extern "C" int twl_select_estimate_prune(
     int32_t* sel_pages, uint32_t sel_stride, int32_t* sel_count, int32_t* idx, uint32_t idx_stride,
     int32_t* count, float* page_scores_out, uint32_t page_score_stride, float* scores_out,
     uint32_t score_stride, int32_t* cand_count, const void* meta_planes,
-    uint32_t plane_cap_pages, const int32_t* plane_slots, uint32_t plane_num_slots, void* stream) {
+    uint32_t plane_cap_pages, const int32_t* plane_slots, uint32_t plane_num_slots,
+    float* surv_probs, void* stream) {
   if (!q || !meta || !k_int4 || !kv_page_indices || !kv_page_indptr || !kv_last_page_len ||
       !sel_pages || !sel_count || !idx || !count)
     return TWL_ENULL;
@@ -307,7 +308,7 @@ extern "C" int twl_select_estimate_prune(
   a.f.num_kv_heads = num_kv_heads; a.f.max_pages = (uint32_t)k; a.f.sm_scale = sm_scale;
   a.f.p_arr = p_arr; a.f.p = p; a.f.high_mode = high_mode; a.f.idx = idx;
   a.f.idx_stride = idx_stride; a.f.count = count; a.f.scores_out = scores_out;
-  a.f.score_stride = score_stride; a.f.cand_count = cand_count;
+  a.f.score_stride = score_stride; a.f.cand_count = cand_count; a.f.surv_probs = surv_probs;
   a.meta = (const uint8_t*)meta; a.token_budget = token_budget;
   a.max_pages_req = max_pages_per_req; a.sel_pages_out = sel_pages; a.sel_count_out = sel_count;
   a.page_scores_out = page_scores_out; a.page_score_stride = page_score_stride;
@@ -333,4 +334,21 @@ extern "C" int twl_select_estimate_prune(
   else TWL_ROW_LAUNCH(TWL_BF16);
 #undef TWL_ROW_LAUNCH
   return hipGetLastError() == hipSuccess ? TWL_OK : TWL_ELAUNCH;
+}
+
+extern "C" int twl_select_estimate_prune(
+    const void* q, int dtype, const void* meta, const void* k_int4, const int32_t* kv_page_indices,
+    const int32_t* kv_page_indptr, const int32_t* kv_last_page_len, uint32_t batch,
+    uint32_t num_q_heads, uint32_t num_kv_heads, uint32_t token_budget,
+    uint32_t max_pages_per_req, float sm_scale, const float* p_arr, float p, int high_mode,
+    int32_t* sel_pages, uint32_t sel_stride, int32_t* sel_count, int32_t* idx, uint32_t idx_stride,
+    int32_t* count, float* page_scores_out, uint32_t page_score_stride, float* scores_out,
+    uint32_t score_stride, int32_t* cand_count, const void* meta_planes,
+    uint32_t plane_cap_pages, const int32_t* plane_slots, uint32_t plane_num_slots, void* stream) {
+  return twl::select_estimate_prune_ex(
+      q, dtype, meta, k_int4, kv_page_indices, kv_page_indptr, kv_last_page_len, batch, num_q_heads,
+      num_kv_heads, token_budget, max_pages_per_req, sm_scale, p_arr, p, high_mode, sel_pages,
+      sel_stride, sel_count, idx, idx_stride, count, page_scores_out, page_score_stride, scores_out,
+      score_stride, cand_count, meta_planes, plane_cap_pages, plane_slots, plane_num_slots, nullptr,
+      stream);
 }

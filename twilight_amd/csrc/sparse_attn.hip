@@ -47,6 +47,7 @@ struct AttnArgs {
   uint32_t rows;
   uint32_t pool;      // workgroups that serve chunks 1.. of long rows
   uint32_t epoch;     // 1..65535, changes with every call: tag of this call's ticket words
+  const float* weights;  // USE_W kernels only: [rows, idx_stride] weight of survivor j (q, K unused)
 };
 
 constexpr int kAttnThreads = 256;
@@ -81,7 +82,11 @@ __device__ __forceinline__ void tag_ticket(int32_t* ticket, uint32_t seen, uint3
 // One chunk (survivors [128*split, 128*split+128) of `row`, which has n > 128*split survivors).
 // Called by all threads of the workgroup.
 // `tok_pre` (chunk 0 only, HAVE_TOK): the chunk's survivor index of this thread, already loaded.
-template <int DT, bool HAVE_TOK>
+// USE_W: the logits are not computed from q and K; survivor j of the row carries the non-negative
+// weight a.weights[row, j] (the estimator's probability, attention.py:295-296) and the output is
+// sum_j w_j V_j / sum_j w_j. No K is read; as a partial result the chunk has maximum 0 and sum
+// sum_j w_j, which the merge below handles unchanged.
+template <int DT, bool HAVE_TOK, bool USE_W>
 __device__ __forceinline__ void attn_chunk(const AttnArgs& a, AttnSmem& sm, uint32_t row,
                                            int split, int n, int tok_pre) {
   int (&slot_id)[kAttnChunk] = sm.slot_id;
@@ -117,7 +122,10 @@ __device__ __forceinline__ void attn_chunk(const AttnArgs& a, AttnSmem& sm, uint
     slot_id[tx] = sid;
   }
   float qf[8];
-  {
+  float e_pre = 0.0f;
+  if (USE_W) {
+    if (tx < cn) e_pre = fmaxf(a.weights[(size_t)row * a.idx_stride + j0 + tx], 0.0f);
+  } else {
     u32x4 v = *(const u32x4*)((const uint16_t*)a.q + (size_t)row * TWL_HEAD_DIM + 8 * sub);
     unpack8<DT>(v, qf);
   }
@@ -138,10 +146,12 @@ __device__ __forceinline__ void attn_chunk(const AttnArgs& a, AttnSmem& sm, uint
   for (int i = 0; i < kAttnSteps; ++i) {
     const int t = i * (4 * kAttnWaves) + wave * 4 + grp;  // local token of this lane group
     tloc[i] = t;
-    const int sid = slot_id[min(t, cn - 1)];
-    const size_t off = (size_t)(sid >> 4) * a.page_stride + (size_t)(sid & 15) * a.token_stride +
-                       head_off;
-    kreg[i] = *(const u32x4*)(kc + off);
+    if (!USE_W) {
+      const int sid = slot_id[min(t, cn - 1)];
+      const size_t off = (size_t)(sid >> 4) * a.page_stride + (size_t)(sid & 15) * a.token_stride +
+                         head_off;
+      kreg[i] = *(const u32x4*)(kc + off);
+    }
   }
 #pragma unroll
   for (int i = 0; i < kAttnSteps; ++i) {
@@ -152,29 +162,36 @@ __device__ __forceinline__ void attn_chunk(const AttnArgs& a, AttnSmem& sm, uint
   }
 
   // ---- logits -------------------------------------------------------------------------------
-  float wmax = -__builtin_inff();
-#pragma unroll
-  for (int i = 0; i < kAttnSteps; ++i) {
-    float kf[8];
-    unpack8<DT>(kreg[i], kf);
-    float acc = 0.0f;
-#pragma unroll
-    for (int d = 0; d < 8; ++d) acc = fmaf(qf[d], kf[d], acc);
-    acc = row16_allreduce<OpSum>(acc) * a.sm_scale;
-    if (tloc[i] < cn) {
-      wmax = fmaxf(wmax, acc);
-      if (sub == 0) w[tloc[i]] = acc;
-    }
-  }
-  if (n_splits > 1 && tx == 0) tag_ticket(&a.tickets[row], ticket_seen, a.epoch);
-  const float m = block_allreduce<OpMax, kAttnWaves>(wmax, red[0]);  // barrier: w[] visible
-
-  // ---- weights ------------------------------------------------------------------------------
+  float m = 0.0f;
   float z = 0.0f;
   float e = 0.0f;
-  if (tx < cn) {
-    e = expf(w[tx] - m);
+  if (USE_W) {
+    if (n_splits > 1 && tx == 0) tag_ticket(&a.tickets[row], ticket_seen, a.epoch);
+    e = e_pre;
     z = e;
+  } else {
+    float wmax = -__builtin_inff();
+#pragma unroll
+    for (int i = 0; i < kAttnSteps; ++i) {
+      float kf[8];
+      unpack8<DT>(kreg[i], kf);
+      float acc = 0.0f;
+#pragma unroll
+      for (int d = 0; d < 8; ++d) acc = fmaf(qf[d], kf[d], acc);
+      acc = row16_allreduce<OpSum>(acc) * a.sm_scale;
+      if (tloc[i] < cn) {
+        wmax = fmaxf(wmax, acc);
+        if (sub == 0) w[tloc[i]] = acc;
+      }
+    }
+    if (n_splits > 1 && tx == 0) tag_ticket(&a.tickets[row], ticket_seen, a.epoch);
+    m = block_allreduce<OpMax, kAttnWaves>(wmax, red[0]);  // barrier: w[] visible
+
+    // ---- weights ----------------------------------------------------------------------------
+    if (tx < cn) {
+      e = expf(w[tx] - m);
+      z = e;
+    }
   }
   z = block_allreduce<OpSum, kAttnWaves>(z, red[1]);
   const bool single = (n_splits == 1);
@@ -302,7 +319,7 @@ __device__ __forceinline__ void attn_chunk(const AttnArgs& a, AttnSmem& sm, uint
 // in row-major order, locating each with a block-wide prefix sum over the rows' chunk counts
 // (a few KB from L2), so a launch never contains more than rows + pool workgroups however long
 // the longest row is.
-template <int DT>
+template <int DT, bool USE_W>
 __global__ __launch_bounds__(kAttnThreads) void sparse_attn_kernel(AttnArgs a) {
   __shared__ AttnSmem sm;
   __shared__ int wave_tot[kAttnWaves];
@@ -319,7 +336,7 @@ __global__ __launch_bounds__(kAttnThreads) void sparse_attn_kernel(AttnArgs a) {
       if (tx == 0 && a.lse_out) a.lse_out[row] = -__builtin_inff();
       return;
     }
-    attn_chunk<DT, true>(a, sm, row, 0, n, tok_pre);
+    attn_chunk<DT, true, USE_W>(a, sm, row, 0, n, tok_pre);
     return;
   }
   const int lane = lane_id();
@@ -352,7 +369,7 @@ __global__ __launch_bounds__(kAttnThreads) void sparse_attn_kernel(AttnArgs a) {
       __syncthreads();
     }
     if (!hit) return;  // j is past the last overflow chunk: nothing left for this workgroup
-    attn_chunk<DT, false>(a, sm, (uint32_t)found[0], found[1], found[2], 0);
+    attn_chunk<DT, false, USE_W>(a, sm, (uint32_t)found[0], found[1], found[2], 0);
     __syncthreads();
   }
 }
@@ -373,8 +390,10 @@ static int launch_sparse_attn(const void* q, void* out, int dtype, const void* k
                               const int32_t* count, const int32_t* kv_page_indices,
                               const int32_t* kv_page_indptr, uint32_t rows, uint32_t num_q_heads,
                               uint32_t num_kv_heads, float sm_scale, float* lse_out,
-                              void* workspace, hipStream_t stream) {
+                              void* workspace, hipStream_t stream,
+                              const float* weights = nullptr) {
   twl::AttnArgs a{};
+  a.weights = weights;
   a.q = q; a.out = out; a.k_cache = k_cache; a.v_cache = v_cache; a.page_stride = page_stride;
   a.token_stride = token_stride; a.head_stride = head_stride; a.idx = idx;
   a.idx_stride = idx_stride; a.count = count; a.kv_page_indices = kv_page_indices;
@@ -394,12 +413,20 @@ static int launch_sparse_attn(const void* q, void* out, int dtype, const void* k
     a.pool = (uint32_t)(overflow_max < 1024 ? overflow_max : 1024);
   }
   dim3 grid(rows + a.pool);
-  if (dtype == TWL_F16)
-    hipLaunchKernelGGL((twl::sparse_attn_kernel<TWL_F16>), grid, dim3(twl::kAttnThreads), 0,
+  if (weights) {
+    if (dtype == TWL_F16)
+      hipLaunchKernelGGL((twl::sparse_attn_kernel<TWL_F16, true>), grid, dim3(twl::kAttnThreads),
+                         0, stream, a);
+    else
+      hipLaunchKernelGGL((twl::sparse_attn_kernel<TWL_BF16, true>), grid, dim3(twl::kAttnThreads),
+                         0, stream, a);
+  } else if (dtype == TWL_F16) {
+    hipLaunchKernelGGL((twl::sparse_attn_kernel<TWL_F16, false>), grid, dim3(twl::kAttnThreads), 0,
                        stream, a);
-  else
-    hipLaunchKernelGGL((twl::sparse_attn_kernel<TWL_BF16>), grid, dim3(twl::kAttnThreads), 0,
+  } else {
+    hipLaunchKernelGGL((twl::sparse_attn_kernel<TWL_BF16, false>), grid, dim3(twl::kAttnThreads), 0,
                        stream, a);
+  }
   return hipGetLastError() == hipSuccess ? TWL_OK : TWL_ELAUNCH;
 }
 
@@ -446,6 +473,34 @@ extern "C" int twl_sparse_attn(const void* q, void* out, int dtype, const void* 
                             head_stride, idx, idx_stride, count, kv_page_indices, kv_page_indptr,
                             rows, num_q_heads, num_kv_heads, sm_scale, lse_out, workspace,
                             (hipStream_t)stream);
+}
+
+// Attention with given weights instead of q.K logits (attention.py:295-296 followed by :299-306):
+// out[row] = sum_j w_j V[idx_j] / sum_j w_j. K and q are not read.
+extern "C" int twl_sparse_attn_weighted(void* out, int dtype, const void* v_cache,
+                                        uint64_t page_stride, uint64_t token_stride,
+                                        uint64_t head_stride, const int32_t* idx,
+                                        uint32_t idx_stride, const int32_t* count,
+                                        const float* weights, const int32_t* kv_page_indices,
+                                        const int32_t* kv_page_indptr, uint32_t batch,
+                                        uint32_t num_q_heads, uint32_t num_kv_heads,
+                                        float* lse_out, void* workspace,
+                                        uint64_t workspace_bytes, void* stream) {
+  if (!workspace || !weights) return TWL_ENULL;
+  if (((uintptr_t)weights) & 3u) return TWL_EALIGN;
+  uint32_t rows = 0;
+  // q and K take no part; the shared check sees V in their place
+  const int rc = check_sparse_attn(v_cache, out, dtype, v_cache, v_cache, page_stride,
+                                   token_stride, head_stride, idx, idx_stride, count,
+                                   kv_page_indices, kv_page_indptr, batch, num_q_heads,
+                                   num_kv_heads, &rows);
+  if (rc != TWL_OK) return rc;
+  if (workspace_bytes < twl_sparse_attn_workspace_bytes(rows, idx_stride)) return TWL_EINVAL;
+  if (((uintptr_t)workspace) & 255u) return TWL_EALIGN;
+  return launch_sparse_attn(nullptr, out, dtype, nullptr, v_cache, page_stride, token_stride,
+                            head_stride, idx, idx_stride, count, kv_page_indices, kv_page_indptr,
+                            rows, num_q_heads, num_kv_heads, 1.0f, lse_out, workspace,
+                            (hipStream_t)stream, weights);
 }
 
 // ---- the same call without a workspace argument -------------------------------------------------

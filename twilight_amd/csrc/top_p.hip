@@ -38,6 +38,7 @@ struct TopPArgs {
   float* probs_out;      // nullable [rows, in_stride] (fused entry only)
   float* low_out;        // nullable [rows]
   int32_t* iters_out;    // nullable [rows]
+  float* surv_probs;     // nullable [rows, idx_stride]: the value of survivor j beside idx
 };
 
 // Element e of the row is held by thread (e/4) % THREADS, slot 4*((e/4)/THREADS) + e%4:
@@ -137,6 +138,7 @@ __global__ __launch_bounds__(THREADS) void top_p_kernel(TopPArgs a) {
   }
   if (a.idx || a.count) {
     int32_t* dst = a.idx ? a.idx + (size_t)row * a.idx_stride : nullptr;
+    float* wdst = (a.idx && a.surv_probs) ? a.surv_probs + (size_t)row * a.idx_stride : nullptr;
     const int32_t* pages = a.sel_pages ? a.sel_pages + (size_t)row * a.sel_stride : nullptr;
     // every chunk's wave totals go to LDS first, so the whole emission needs one barrier
     __shared__ int chunk_tot[CHUNKS][16];
@@ -169,6 +171,7 @@ __global__ __launch_bounds__(THREADS) void top_p_kernel(TopPArgs a) {
         for (int j = 0; j < 4; ++j) {
           if (keep[c] & (1u << j)) {
             const uint32_t e = e0 + j;
+            if (wdst) wdst[pos] = x[4 * c + j];
             dst[pos++] = pages ? (pages[e >> 4] * TWL_PAGE + (int)(e & 15u)) : (int)e;
           }
         }
@@ -229,12 +232,11 @@ extern "C" int twl_top_p_f32(const float* probs, uint8_t* mask, int32_t* idx, in
   return twl::launch_top_p<TWL_F32, false>(a, rows, (hipStream_t)stream);
 }
 
-extern "C" int twl_softmax_top_p_f32(const float* scores, uint32_t score_stride,
-                                     const int32_t* lens, uint32_t rows, uint32_t d,
-                                     const float* p_arr, float p, int high_mode,
-                                     const int32_t* sel_pages, uint32_t sel_stride, int32_t* idx,
-                                     uint32_t idx_stride, int32_t* count, float* probs_out,
-                                     float* low_out, void* stream) {
+int twl::softmax_top_p_ex(const float* scores, uint32_t score_stride, const int32_t* lens,
+                          uint32_t rows, uint32_t d, const float* p_arr, float p, int high_mode,
+                          const int32_t* sel_pages, uint32_t sel_stride, int32_t* idx,
+                          uint32_t idx_stride, int32_t* count, float* probs_out, float* low_out,
+                          float* surv_probs, void* stream) {
   int rc = check_top_p_common(scores, nullptr, idx, count, p, p_arr, rows, d, idx_stride, high_mode);
   if (rc != TWL_OK) return rc;
   if (score_stride < d) return TWL_EINVAL;
@@ -244,6 +246,17 @@ extern "C" int twl_softmax_top_p_f32(const float* scores, uint32_t score_stride,
   a.in = scores; a.in_stride = score_stride; a.lens = lens; a.d = d; a.p_arr = p_arr; a.p = p;
   a.high_mode = high_mode; a.mask = nullptr; a.idx = idx; a.idx_stride = idx_stride;
   a.count = count; a.sel_pages = sel_pages; a.sel_stride = sel_stride; a.probs_out = probs_out;
-  a.low_out = low_out;
+  a.low_out = low_out; a.surv_probs = surv_probs;
   return twl::launch_top_p<TWL_F32, true>(a, rows, (hipStream_t)stream);
+}
+
+extern "C" int twl_softmax_top_p_f32(const float* scores, uint32_t score_stride,
+                                     const int32_t* lens, uint32_t rows, uint32_t d,
+                                     const float* p_arr, float p, int high_mode,
+                                     const int32_t* sel_pages, uint32_t sel_stride, int32_t* idx,
+                                     uint32_t idx_stride, int32_t* count, float* probs_out,
+                                     float* low_out, void* stream) {
+  return twl::softmax_top_p_ex(scores, score_stride, lens, rows, d, p_arr, p, high_mode, sel_pages,
+                               sel_stride, idx, idx_stride, count, probs_out, low_out, nullptr,
+                               stream);
 }

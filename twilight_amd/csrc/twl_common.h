@@ -266,6 +266,31 @@ inline int device_cu_count(int* out) {
   return TWL_OK;
 }
 
+// The exported estimator / pruner entry points with one more output: `surv_probs` (nullable,
+// float [rows, idx_stride]) receives, beside idx[row, j], the softmax probability the estimator
+// gave survivor j. Everything else is the exported function of the same name.
+int gemv_top_p_ex(const void* q, int q_dtype, const void* k_int4, const int32_t* sel_pages,
+                  const int32_t* sel_count, uint32_t sel_stride, const int32_t* kv_page_indices,
+                  const int32_t* kv_page_indptr, const int32_t* kv_last_page_len, uint32_t batch,
+                  uint32_t num_q_heads, uint32_t num_kv_heads, uint32_t max_pages_per_row,
+                  float sm_scale, const float* p_arr, float p, int high_mode, int32_t* idx,
+                  uint32_t idx_stride, int32_t* count, float* scores_out, uint32_t score_stride,
+                  int32_t* cand_count, float* low_out, float* surv_probs, void* stream);
+int select_estimate_prune_ex(
+    const void* q, int dtype, const void* meta, const void* k_int4, const int32_t* kv_page_indices,
+    const int32_t* kv_page_indptr, const int32_t* kv_last_page_len, uint32_t batch,
+    uint32_t num_q_heads, uint32_t num_kv_heads, uint32_t token_budget,
+    uint32_t max_pages_per_req, float sm_scale, const float* p_arr, float p, int high_mode,
+    int32_t* sel_pages, uint32_t sel_stride, int32_t* sel_count, int32_t* idx, uint32_t idx_stride,
+    int32_t* count, float* page_scores_out, uint32_t page_score_stride, float* scores_out,
+    uint32_t score_stride, int32_t* cand_count, const void* meta_planes,
+    uint32_t plane_cap_pages, const int32_t* plane_slots, uint32_t plane_num_slots,
+    float* surv_probs, void* stream);
+int softmax_top_p_ex(const float* scores, uint32_t score_stride, const int32_t* lens,
+                     uint32_t rows, uint32_t d, const float* p_arr, float p, int high_mode,
+                     const int32_t* sel_pages, uint32_t sel_stride, int32_t* idx,
+                     uint32_t idx_stride, int32_t* count, float* probs_out, float* low_out,
+                     float* surv_probs, void* stream);
 
 }  // namespace twl
 #endif  // TWL_COMMON_H_

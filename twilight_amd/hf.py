@@ -281,7 +281,7 @@ def _twilight_attention_forward(self, hidden_states, position_embeddings=None, a
     out = st.layer(q[:, :, 0].contiguous())           # [B, H, 128]
     if st.budget_info is not None and not st.recorded:
         st.budget_info.update(self.layer_idx, st.layer.count)
-        st.budget_info.update_B0(self.layer_idx, min(st.layer.token_budget, st.seq_len))
+        st.budget_info.update_B0(self.layer_idx, min(st.layer._budget(st.seq_len), st.seq_len))
     if st.score_info is not None and not st.recorded:
         st.score_info.update(self.layer_idx, kept_attention_mass(
             st.cache, q[:, :, 0], st.layer.idx, st.layer.count, st.layer.sm_scale))
@@ -312,8 +312,6 @@ def enable_sparse_attention(model, sparse_config: Dict, enable_budget_info: bool
         t = sparse_config.get(part, {}).get("type", "none")
         if str(t).lower() not in ("none", ""):
             raise RuntimeError(f"{part} type {t!r} is not supported")
-    if sparse_config.get("use_estimated_weights_in_attn", False):
-        raise RuntimeError("use_estimated_weights_in_attn is not supported")
     cfg = parse_sparse_config(sparse_config)
     cfg["high"] = high
     skip = 2 if sparse_config.get("skip_first_two_layers", True) else 0
@@ -375,6 +373,10 @@ class GraphedDecodeStep:
                     raise RuntimeError("GraphedDecodeStep needs keep_hf_cache=False")
                 if st.score_info is not None:
                     raise RuntimeError("GraphedDecodeStep cannot record the score diagnostic")
+                if not st.dense and st.cfg.get("sparsity_rate", -1) != -1:
+                    # the budget is a launch argument: a recorded step would keep the first one
+                    raise RuntimeError("GraphedDecodeStep cannot record a selector with "
+                                       "sparsity_rate (its token budget changes every step)")
                 self.states.append((module.layer_idx, st))
         if not self.states:
             raise RuntimeError("no patched attention module")
@@ -432,7 +434,7 @@ class GraphedDecodeStep:
         for lid, st in self.states:
             if st.budget_info is not None and not st.dense:
                 st.budget_info.update(lid, st.layer.count)
-                st.budget_info.update_B0(lid, min(st.layer.token_budget, st.seq_len))
+                st.budget_info.update_B0(lid, min(st.layer._budget(st.seq_len), st.seq_len))
         return self.logits
 
 

@@ -29,6 +29,61 @@ def attention_workspace_bytes(rows: int, idx_stride: int) -> int:
     return int(_lib.lib().twl_sparse_attn_workspace_bytes(rows, idx_stride))
 
 
+def weighted_paged_decode_attention(weights: torch.Tensor, v_cache: torch.Tensor,
+                                    idx: torch.Tensor, count: torch.Tensor,
+                                    kv_page_indices: torch.Tensor, kv_page_indptr: torch.Tensor,
+                                    return_lse: bool = False, out: Optional[torch.Tensor] = None,
+                                    workspace: Optional[torch.Tensor] = None):
+    """Attention over per-row survivor lists with given weights in place of q.K logits
+    (``use_estimated_weights_in_attn``, attention.py:295-296, then :299-306).
+
+    ``weights`` fp32 [B,H,S]: entry j weighs token ``idx[b,h,j]`` (j < ``count[b,h]``);
+    ``v_cache`` [pages,16,Hkv,128] fp16/bf16. Returns ``out`` [B,H,128] in the cache dtype:
+    sum_j w_j V_j / sum_j w_j (and, when asked, log sum_j w_j as ``lse``).
+    """
+    check_input(weights, "weights"); check_dtype(weights, torch.float32, "weights")
+    check_dim(3, weights, "weights")
+    B, H, S = weights.shape
+    vs = _cache_strides(v_cache, "v_cache")
+    Hkv = v_cache.size(2)
+    if v_cache.size(3) != _lib.HEAD_DIM:
+        raise RuntimeError(f"head_dim must be {_lib.HEAD_DIM}, got {v_cache.size(3)}")
+    if H % Hkv != 0:
+        raise RuntimeError(f"num_q_heads {H} must be a multiple of num_kv_heads {Hkv}")
+    check_input(idx, "idx"); check_dtype(idx, torch.int32, "idx"); check_dim(3, idx, "idx")
+    check_input(count, "count"); check_dtype(count, torch.int32, "count")
+    if tuple(idx.shape) != (B, H, S) or count.numel() != B * H:
+        raise RuntimeError("idx must be [B,H,S] like weights and count [B,H]")
+    for name, t in (("kv_page_indices", kv_page_indices), ("kv_page_indptr", kv_page_indptr)):
+        check_input(t, name); check_dtype(t, torch.int32, name)
+    if kv_page_indptr.numel() != B + 1:
+        raise RuntimeError("kv_page_indptr must have B+1 elements")
+    check_same_device(weights, ("v_cache", v_cache), ("idx", idx), ("count", count),
+                      ("kv_page_indices", kv_page_indices), ("kv_page_indptr", kv_page_indptr))
+    dev = weights.device
+    with torch.cuda.device(dev):
+        if out is None:
+            out = torch.empty((B, H, _lib.HEAD_DIM), dtype=v_cache.dtype, device=dev)
+        else:
+            check_input(out, "out")
+            if tuple(out.shape) != (B, H, _lib.HEAD_DIM) or out.dtype != v_cache.dtype:
+                raise RuntimeError("out must be [B,H,128] of the cache dtype")
+        lse = torch.empty((B, H), dtype=torch.float32, device=dev) if return_lse else None
+        need = attention_workspace_bytes(B * H, S)
+        if workspace is None:
+            workspace = torch.empty(need, dtype=torch.uint8, device=dev)
+        else:
+            check_input(workspace, "workspace"); check_dtype(workspace, torch.uint8, "workspace")
+            if workspace.numel() < need or workspace.device != dev:
+                raise RuntimeError(f"workspace must hold {need} bytes on {dev}")
+        rc = _lib.lib().twl_sparse_attn_weighted(
+            ptr(out), dtype_code(v_cache.dtype, "v_cache"), ptr(v_cache), vs[0], vs[1], vs[2],
+            ptr(idx), S, ptr(count), ptr(weights), ptr(kv_page_indices), ptr(kv_page_indptr),
+            B, H, Hkv, ptr(lse), ptr(workspace), workspace.numel(), stream_of(weights))
+    _lib.check(rc, "WeightedPagedDecodeAttention")
+    return (out, lse) if return_lse else out
+
+
 def sparse_paged_decode_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                                   idx: torch.Tensor, count: torch.Tensor,
                                   kv_page_indices: torch.Tensor, kv_page_indptr: torch.Tensor,

@@ -3,7 +3,8 @@
 Mirrors the decode branch of twilight/pyimpl/attention.py:188-306 (selector -> weight estimator
 -> weight pruner -> attention) with the configuration keys of benchmark/configs/*.json:
 ``selector: {type: quest, token_budget, chunk_size}``, ``weight_estimator: {type: min_max_quant,
-quant_bit: 4}``, ``weight_pruner: {type: top_p, threshold}``. All buffers are allocated once; a
+quant_bit: 4}``, ``weight_pruner: {type: top_p, threshold}``, and the optional ``selector.sparsity_rate``
+(quest.py:45-46) and ``use_estimated_weights_in_attn`` (attention.py:295-296). All buffers are allocated once; a
 step is a single call into ``twl_decode_layer`` which enqueues the kernels on the current stream.
 """
 from __future__ import annotations
@@ -34,10 +35,12 @@ def parse_sparse_config(cfg: dict) -> dict:
         raise RuntimeError("weight_estimator must be {type: min_max_quant, quant_bit: 4}")
     if prn.get("type", "top_p") != "top_p":
         raise RuntimeError(f"weight_pruner type {prn.get('type')!r} is not supported (only 'top_p')")
-    if cfg.get("use_estimated_weights_in_attn", False):
-        raise RuntimeError("use_estimated_weights_in_attn=True is not supported")
+    rate = float(sel.get("sparsity_rate", -1))
+    if rate != -1 and not (0.0 <= rate <= 1.0):
+        raise RuntimeError(f"selector sparsity_rate must be -1 (off) or in [0, 1], got {rate}")
     return dict(token_budget=int(sel.get("token_budget", 8192)),
-                top_p=float(prn.get("threshold", 0.85)))
+                top_p=float(prn.get("threshold", 0.85)), sparsity_rate=rate,
+                use_estimated_weights=bool(cfg.get("use_estimated_weights_in_attn", False)))
 
 
 class TwilightDecodeLayer:
@@ -46,7 +49,8 @@ class TwilightDecodeLayer:
     def __init__(self, cache: PagedKVCache, num_q_heads: int, token_budget: int = 8192,
                  top_p: float = 0.85, high: str = "max", sm_scale: Optional[float] = None,
                  fused_estimator: bool = True, keep_scores: bool = False,
-                 reserve_pages: int = 0, group_union: bool = False):
+                 reserve_pages: int = 0, group_union: bool = False,
+                 sparsity_rate: float = -1, use_estimated_weights: bool = False):
         if num_q_heads % cache.num_kv_heads != 0:
             raise RuntimeError("num_q_heads must be a multiple of the cache's kv heads")
         if not (0.0 < top_p <= 1.0):
@@ -69,6 +73,16 @@ class TwilightDecodeLayer:
         self.group_union = bool(group_union)
         if self.group_union and num_q_heads // cache.num_kv_heads not in (1, 2, 4, 8):
             raise RuntimeError("group_union needs 1, 2, 4 or 8 q heads per kv head")
+        # sparsity_rate != -1 replaces token_budget every step by int(longest request * rate), as
+        # quest.py:45-46 does with the sequence length of its padded batch
+        self.sparsity_rate = float(sparsity_rate)
+        if self.sparsity_rate != -1 and not (0.0 <= self.sparsity_rate <= 1.0):
+            raise RuntimeError("sparsity_rate must be -1 (off) or in [0, 1]")
+        # use_estimated_weights: the attention weighs V with the estimator's probabilities of the
+        # survivors (``surv_probs``) instead of computing exact logits from K
+        self.use_estimated_weights = bool(use_estimated_weights)
+        if self.use_estimated_weights and self.group_union:
+            raise RuntimeError("use_estimated_weights and group_union exclude each other")
         self._alloc()
 
     @classmethod
@@ -79,7 +93,7 @@ class TwilightDecodeLayer:
         c = self.cache
         B, H, dev = c.batch, self.H, c.device
         cap = max(c.max_pages_per_req, self.reserve_pages)
-        self.k_pages = quest_num_pages(self.token_budget, cap)
+        self.k_pages = quest_num_pages(self._budget(cap * _lib.PAGE), cap)
         M = self.k_pages * _lib.PAGE
         if M > _lib.MAX_CANDIDATES:
             raise RuntimeError(f"token budget {M} exceeds the supported maximum {_lib.MAX_CANDIDATES}")
@@ -94,6 +108,8 @@ class TwilightDecodeLayer:
         self.out = torch.zeros((B, H, _lib.HEAD_DIM), dtype=c.dtype, device=dev)
         ws = int(_lib.lib().twl_sparse_attn_workspace_bytes(B * H, M))
         self.attn_workspace = torch.zeros(ws, dtype=torch.uint8, device=dev)
+        self.surv_probs = torch.zeros((B, H, M), dtype=f32, device=dev) \
+            if self.use_estimated_weights else None
         self.group_idx = self.group_count = self.group_workspace = None
         if self.group_union:
             Hkv = c.num_kv_heads
@@ -104,6 +120,15 @@ class TwilightDecodeLayer:
             self.group_workspace = torch.empty(gws, dtype=torch.uint8, device=dev)
         self._shape = (B, cap)
         self._args, self._args_key = None, None
+
+    def _budget(self, seq_len: int) -> int:
+        """Token budget of a step whose longest request holds ``seq_len`` tokens."""
+        if self.sparsity_rate == -1:
+            return self.token_budget
+        # quest.py:45-46, then :91-93: a budget of 0 still keeps one chunk, which is what a budget
+        # of one whole chunk asks for
+        budget = int(seq_len * self.sparsity_rate)
+        return budget if budget > 0 else _lib.PAGE
 
     def _build_args(self, q: torch.Tensor) -> "_lib.LayerArgs":
         c = self.cache
@@ -126,7 +151,7 @@ class TwilightDecodeLayer:
         a.kv_page_indices, a.kv_page_indptr = ptr(c.kv_page_indices), ptr(c.kv_page_indptr)
         a.kv_last_page_len = ptr(c.kv_last_page_len)
         a.batch, a.num_q_heads, a.num_kv_heads = c.batch, self.H, c.num_kv_heads
-        a.max_pages_per_req, a.token_budget = c.max_pages_per_req, self.token_budget
+        a.max_pages_per_req, a.token_budget = c.max_pages_per_req, self._budget(c.max_seq_len)
         a.top_p, a.high_mode, a.sm_scale = self.top_p, self.high_mode, self.sm_scale
         a.sel_pages, a.sel_stride = ptr(self.sel_pages), self.sel_pages.size(2)
         a.sel_count = ptr(self.sel_count)
@@ -144,6 +169,8 @@ class TwilightDecodeLayer:
             a.group_count = ptr(self.group_count)
             a.group_workspace = ptr(self.group_workspace)
             a.group_workspace_bytes = self.group_workspace.numel()
+        if self.use_estimated_weights:
+            a.surv_probs, a.use_estimated_weights = ptr(self.surv_probs), 1
         return a
 
     def forward(self, q: torch.Tensor) -> torch.Tensor:
@@ -167,6 +194,8 @@ class TwilightDecodeLayer:
         if self._args_key != key:
             self._args, self._args_key = self._build_args(q), key
         a = self._args
+        if self.sparsity_rate != -1:
+            a.token_budget = self._budget(c.max_seq_len)
         with torch.cuda.device(c.device):
             rc = _lib.lib().twl_decode_layer(ctypes.byref(a), stream_of(q))
         _lib.check(rc, "TwilightDecodeLayer")
