@@ -577,6 +577,37 @@ def measure_shape(L, dev, B, H, Hkv, N, dt, budget, top_p, n_layers, steps, warm
     if H != Hkv:
         out["layer_bytes_shared_candidate_lists"] = shared
         out["frac_of_hbm_peak_shared_candidate_lists"] = gb(shared)
+    if H != Hkv and H // Hkv in (2, 4, 8):
+        # the option that realises the shared count: one Quest selection per kv head, metadata and
+        # INT4 records read once per kv head, five launches (scores, top-k, group GEMV, pruner,
+        # attention)
+        glayers = [TwilightDecodeLayer(l.cache, H, token_budget=budget, top_p=top_p, high="max",
+                                       group_select=True) for l in layers]
+        for i in range(warmup):
+            glayers[i % n_layers].forward(qs[i % n_layers])
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(steps):
+            glayers[i % n_layers].forward(qs[i % n_layers])
+        torch.cuda.synchronize()
+        g_us = (time.perf_counter() - t0) * 1e6 / steps
+        for i in range(n_layers):
+            glayers[i].forward(qs[i])
+        torch.cuda.synchronize()
+        g_bar = float(torch.stack([l.count for l in glayers]).float().mean())
+        gemv_us = _time_calls(rot(lambda l, c, q: lambda: L.twl_gemv_int4_group(
+            p(q), qcode, p(l.scores), M, p(l.cand_count), p(c.k_int4), p(l.sel_pages),
+            p(l.sel_count), kp, p(c.kv_page_indices), p(c.kv_page_indptr), p(c.kv_last_page_len),
+            B, H, Hkv, kp, sm, stream)), max(steps, 40), 2 * n_layers)
+        gemv_bytes = B * Hkv * M * 80 + rows * M * 4
+        out["group_select"] = {
+            "what": "TwilightDecodeLayer(group_select=True): one candidate list per kv head "
+                    "(largest q-head page score), not the reference's per-q-head selection",
+            "us_per_layer": round(g_us, 2), "survivors_mean": round(g_bar, 1),
+            "frac_of_hbm_peak_shared_candidate_lists": round(shared / g_us / 1e3 / HBM_PEAK_GBS, 4),
+            "gemv_int4_group_us": round(gemv_us, 2), "gemv_int4_group_bytes": gemv_bytes,
+            "gemv_int4_group_frac_of_hbm_peak": round(gemv_bytes / gemv_us / 1e3 / HBM_PEAK_GBS, 4)}
+        del glayers
     if dense:
         gws = torch.empty(int(L.twl_group_attn_workspace_bytes(B, H, Hkv, N, 0)), dtype=torch.uint8,
                           device=dev)

@@ -201,6 +201,22 @@ int twl_gemv_int4(const void* q, int q_dtype, float* out, uint32_t out_stride, i
                   uint32_t num_q_heads, uint32_t num_kv_heads, uint32_t max_pages_per_row,
                   float sm_scale, void* stream);
 
+/* twl_gemv_int4 for q heads that share kv heads AND one page list per kv head: the list of a
+ * group's first q head (sel_pages / sel_count row b * num_q_heads + kvh * G, required) serves the
+ * G = num_q_heads / num_kv_heads heads of the group (G in {2, 4, 8}), every INT4 record is
+ * fetched once per group and out / out_count are written for every q head. A head's scores are
+ * bit-identical to twl_gemv_int4 over the same list.
+ * Replaces: the same estimator matmul (attention.py:252-255) when the candidate set is chosen per
+ * kv head (the reference repeats K per q head, attention.py:124-126, and selects per q head; see
+ * twl_layer_args.group_select). */
+int twl_gemv_int4_group(const void* q, int q_dtype, float* out, uint32_t out_stride,
+                        int32_t* out_count, const void* k_int4, const int32_t* sel_pages,
+                        const int32_t* sel_count, uint32_t sel_stride,
+                        const int32_t* kv_page_indices, const int32_t* kv_page_indptr,
+                        const int32_t* kv_last_page_len, uint32_t batch, uint32_t num_q_heads,
+                        uint32_t num_kv_heads, uint32_t max_pages_per_row, float sm_scale,
+                        void* stream);
+
 /* ---------------------------------------------------------------------------------------------
  * Token-granular paged score GEMVs in the tensor layouts (and call shapes) of the absent
  * ftka.cuda_ops.gemv module, as used by benchmark/efficiency/bench_gemv.py. K cache
@@ -541,6 +557,15 @@ typedef struct twl_layer_args {
    * Not available together with group_idx. */
   float* surv_probs;
   int use_estimated_weights;
+  /* group_select != 0 (G = num_q_heads / num_kv_heads in {2, 4, 8}): the Quest selection is made
+   * per kv head — a page's score is the largest of its group's q-head scores — so the q heads of
+   * a group share one candidate list, the metadata and the INT4 records are read once per kv head
+   * (twl_quest_page_scores per group, twl_quest_topk_pages, twl_gemv_int4_group,
+   * twl_softmax_top_p_f32), and every q head still prunes and attends on its own scores. Not the
+   * reference's per-q-head selection (attention.py:124-126 repeats K per q head): an option, as
+   * group_idx is. sel_pages / sel_count hold the group's list in each of its q-head rows;
+   * `scores` and `page_scores` (required) are always written. */
+  int group_select;
 } twl_layer_args;
 
 int twl_decode_layer(const twl_layer_args* args, void* stream);

@@ -17,6 +17,9 @@ How each function is pinned (tests/test_oracle_*.py):
                          also with given logits (use_estimated_weights_in_attn); a K the 4-bit
                          grid holds exactly makes both attention modes of decode_layer_dense meet
   sparsity_rate          closed forms of the budget rule: rate 1 keeps all, rate 0 one chunk
+  quest_selector_group_dense
+                         group 1 is quest_selector_dense; identical queries inside a group give
+                         the per-head selection; brute force over the group maxima on 25 chunks
   get_label_tensor_ref, bgemv_int8_ref
                          the reference's own torch checks (channel.py:82-110, bgemv_int8.py:78-93),
                          i.e. a gather and a matmul
@@ -148,6 +151,26 @@ def quest_selector_dense(q: torch.Tensor, k: torch.Tensor, chunk_size: int, toke
     mask = torch.zeros((B, H, 1, padded), dtype=torch.bool)        # quest.py:111-118
     mask.scatter_(-1, tok, True)
     return mask[..., :N], topk                                     # quest.py:121-122
+
+
+def quest_selector_group_dense(q: torch.Tensor, k: torch.Tensor, chunk_size: int,
+                               token_budget: int, group: int):
+    """Selection per kv head (an option of this build, not in the reference, which selects per q
+    head): the chunk scores of quest.py:36-84 per q head, the largest of each group of ``group``
+    consecutive q heads per chunk, then the top-k of quest.py:93-122 on those, the same for every
+    q head of the group. Returns (token mask [B,H,1,N] bool, group scores [B,H,1,chunks])."""
+    B, H, _, _ = q.shape
+    N = k.shape[-2]
+    est = quest_chunk_scores_dense(q, k, chunk_size)
+    n_chunks = est.shape[-1]
+    gmax = est.reshape(B, H // group, group, 1, n_chunks).amax(dim=2, keepdim=True)
+    gmax = gmax.expand(B, H // group, group, 1, n_chunks).reshape(B, H, 1, n_chunks)
+    kc = quest_chunk_budget(token_budget, chunk_size, n_chunks)
+    order = torch.sort(gmax.double(), dim=-1, descending=True, stable=True).indices
+    tok = order[..., :kc].unsqueeze(-1) * chunk_size + torch.arange(chunk_size)
+    mask = torch.zeros((B, H, 1, n_chunks * chunk_size), dtype=torch.bool)
+    mask.scatter_(-1, tok.reshape(B, H, 1, -1), True)
+    return mask[..., :N], gmax
 
 
 def quest_page_meta(k_pages: torch.Tensor, valid_len: Optional[torch.Tensor] = None):

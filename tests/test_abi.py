@@ -93,6 +93,11 @@ def test_c_level_validation_without_gpu(hip_lib):
     assert L.twl_sparse_attn_workspace_bytes(512, 8192) <= _lib.STATIC_SCRATCH_BYTES
     assert L.twl_sparse_attn_static(fake, fake, 0, fake, fake, 4096, 256, 128, fake, 8192, fake,
                                     fake, fake, 128, 32, 32, 1.0, 0, 0) == -7   # 4096 rows: too big
+    # the group GEMV: a page list is required, 2 / 4 / 8 q heads per kv head
+    gg = lambda **kw: L.twl_gemv_int4_group(
+        fake, 0, fake, kw.get("os", 64), 0, fake, kw.get("sel", fake), 0, 4, fake, fake, fake, 1,
+        kw.get("hq", 4), kw.get("hkv", 1), 4, 1.0, 0)
+    assert gg(sel=0) == -1 and gg(hq=3) == -2 and gg(hq=4, hkv=4) == -2 and gg(os=63) == -2
     # attention on given weights: weights and workspace required, V strides and sizes as above
     wat = lambda **kw: L.twl_sparse_attn_weighted(
         kw.get("out", fake), 0, fake, 4096, 256, kw.get("hs", 128), fake, kw.get("stride", 8), fake,

@@ -149,6 +149,37 @@ def test_gemv_selected_pages_and_ragged_counts(dev):
             assert np.all(got[b, h, n * 16:] == 123.0)      # nothing written past the row's pages
 
 
+@pytest.mark.parametrize("H,Hkv,qdt", [(8, 2, torch.float16), (8, 4, torch.bfloat16), (8, 1, torch.float16)])
+def test_gemv_group_lists_equal_per_head_gemv(dev, H, Hkv, qdt):
+    """One page list per kv head, records fetched once per group: every q head's scores are those
+    of the per-head GEMV over the same list, bit for bit (ragged counts, partial last page)."""
+    B, npg, S = 3, 90, 70
+    G = H // Hkv
+    rec = synth.int4_records_random(B * npg, Hkv, seed=16)
+    ids, indptr, last = synth.identity_page_table(B, npg, last_len=5, shuffle_seed=17)
+    g = torch.Generator().manual_seed(18)
+    q = torch.randn((B, H, 128), generator=g).to(qdt)
+    lists = torch.stack([torch.sort(torch.randperm(npg, generator=g)[:S]).values
+                         for _ in range(B * Hkv)]).reshape(B, Hkv, S).to(torch.int32)
+    first = torch.cat([torch.randperm(npg - 1, generator=g)[:S - 1], torch.tensor([npg - 1])])
+    lists[0, 0] = torch.sort(first).values.to(torch.int32)       # the partial last page is a candidate
+    cnt_kv = torch.randint(1, S + 1, (B, Hkv), generator=g).to(torch.int32)
+    cnt_kv[0, 0] = S; cnt_kv[1, 0] = 1; cnt_kv[2, 0] = 33
+    sel = lists.repeat_interleave(G, dim=1).contiguous()
+    cnt = cnt_kv.repeat_interleave(G, dim=1).contiguous()
+    # the group kernel only looks at the first q head's list: the other rows may hold anything
+    junk = sel.clone()
+    junk.reshape(B, Hkv, G, S)[:, :, 1:] = 0
+    args = (q.to(dev), rec.to(dev), ids.to(dev), indptr.to(dev), last.to(dev))
+    want, wc = K.sparse_gemv_int4(*args, sel_pages=sel.to(dev), sel_count=cnt.to(dev),
+                                  out=torch.full((B, H, S * 16), 7.0, device=dev))
+    got, gc = K.sparse_gemv_int4(*args, sel_pages=junk.to(dev), sel_count=cnt.to(dev),
+                                 out=torch.full((B, H, S * 16), 7.0, device=dev), group_lists=True)
+    assert torch.equal(gc, wc)
+    assert torch.equal(got.view(torch.int32), want.view(torch.int32))
+    assert torch.isneginf(want).any()                             # the partial page was exercised
+
+
 def test_gemv_constant_case_of_the_reference_bench(dev):
     # benchmark/efficiency/bench_gemv.py:390-422: q = 1, nibbles 3, scale 1, zero 0 -> 3*128 = 384
     npg = 8

@@ -47,7 +47,7 @@ def _assert_selection_ties(page_scores, gpu_pages, ora_mask0, npg):
 
 
 def _run_case(dev, B, H, Hkv, N, budget, p, dt, seed, shuffle=True, n_heavy=16, fused=True,
-              planes=False, rate=-1, use_est=False):
+              planes=False, rate=-1, use_est=False, group_select=False):
     q, k, v = synth.heavy_hitter_qkv(B, H, N, n_heavy=n_heavy, mass=0.6, seed=seed, dtype=dt)
     group = H // Hkv
     kk, vv = k[:, ::group].contiguous(), v[:, ::group].contiguous()        # one K/V per kv head
@@ -57,7 +57,7 @@ def _run_case(dev, B, H, Hkv, N, budget, p, dt, seed, shuffle=True, n_heavy=16, 
                                     plane_pages=npg if planes else None)
     layer = TwilightDecodeLayer(cache, H, token_budget=budget, top_p=p, high="max",
                                 fused_estimator=fused, keep_scores=True, sparsity_rate=rate,
-                                use_estimated_weights=use_est)
+                                use_estimated_weights=use_est, group_select=group_select)
     if rate != -1:
         budget = int(N * rate)                                              # quest.py:45-46
     out = layer(q[:, :, 0].to(dt).to(dev)).cpu().float()
@@ -66,6 +66,14 @@ def _run_case(dev, B, H, Hkv, N, budget, p, dt, seed, shuffle=True, n_heavy=16, 
     ref = P.decode_layer_dense(q, krep, vrep, top_p=p, token_budget=budget if budget < N else None,
                                high_mode=native.HIGH_MAX, quant="storage", prob_dtype=dt,
                                sparsity_rate=rate, use_estimated_weights=use_est)
+    est_pg = None
+    if group_select:
+        # one candidate list per kv head: the oracle's group selection replaces the per-head one
+        gmask, gsc = P.quest_selector_group_dense(q.float(), krep.float(), 16, budget, group)
+        est_pg = gsc[:, :, 0].reshape(B * H, -1)
+        ref = P.decode_layer_dense(q, krep, vrep, top_p=p, token_budget=budget, high_mode=native.HIGH_MAX,
+                                   quant="storage", prob_dtype=dt, use_estimated_weights=use_est,
+                                   mask0=gmask)
     rows = B * H
     # 1. selector: the oracle's pages, except pages whose score ties the k-th within rounding
     #    (checked on the oracle's own page scores); the later stages are then followed on the
@@ -75,8 +83,11 @@ def _run_case(dev, B, H, Hkv, N, budget, p, dt, seed, shuffle=True, n_heavy=16, 
     mask0 = ref["mask0"].reshape(rows, N).numpy()
     gmask0 = _pages_to_mask(sel, selc, npg)[:, :N]
     differ = np.nonzero((gmask0 != mask0).any(-1))[0]
+    if group_select:
+        assert (sel.reshape(B, Hkv, group, -1) == sel.reshape(B, Hkv, group, -1)[:, :, :1]).all()
     if differ.size:
-        est_pg = P.quest_chunk_scores_dense(q.float(), krep.float(), 16)[:, :, 0].reshape(rows, -1)
+        if est_pg is None:
+            est_pg = P.quest_chunk_scores_dense(q.float(), krep.float(), 16)[:, :, 0].reshape(rows, -1)
         for r in differ:
             _assert_selection_ties(est_pg[r], sel[r, :selc[r]], mask0[r], npg)
         ref = P.decode_layer_dense(q, krep, vrep, top_p=p, token_budget=budget, high_mode=native.HIGH_MAX,
@@ -180,6 +191,19 @@ def test_layer_estimated_weights_long_rows(dev):
     layer, _ = _run_case(dev, 2, 8, 8, 4096, 2048, 0.99, torch.float16, seed=5, n_heavy=0,
                          use_est=True)
     assert int(layer.count.max()) > 256
+
+
+@pytest.mark.parametrize("B,H,Hkv,N,budget,dt", [
+    (2, 8, 2, 2048, 512, torch.bfloat16),     # Llama-3 grouping in the small
+    (8, 32, 8, 1024, 256, torch.float16),     # 256 rows
+    (3, 8, 4, 1000, 250, torch.float16),      # two q heads per kv head, ragged
+    (1, 8, 1, 600, 100, torch.bfloat16),      # eight q heads on one kv head
+    (2, 4, 4, 512, 128, torch.float16),       # no grouping: the option changes nothing
+])
+def test_layer_group_select(dev, B, H, Hkv, N, budget, dt):
+    """group_select: one Quest selection per kv head (largest q-head score per page), records read
+    once per kv head; every later stage per q head as before."""
+    _run_case(dev, B, H, Hkv, N, budget, 0.9, dt, seed=3 * B + H + Hkv, n_heavy=6, group_select=True)
 
 
 @pytest.mark.parametrize("N,rate,planes", [(2048, 0.25, False), (1000, 0.13, True), (300, 0.0, False),

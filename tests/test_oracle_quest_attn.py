@@ -68,6 +68,35 @@ def test_quest_meta_form_equals_dense_form():
             assert torch.allclose(s.float(), dense[b, h, 0], rtol=1e-5, atol=1e-4)
 
 
+def test_group_selection_reduces_to_the_per_head_selection():
+    g = torch.Generator().manual_seed(11)
+    B, H, N = 2, 8, 400
+    q = torch.randn((B, H, 1, 128), generator=g)
+    k = torch.randn((B, H, N, 128), generator=g)
+    per_head, _ = P.quest_selector_dense(q, k, 16, 96)
+    m1, _ = P.quest_selector_group_dense(q, k, 16, 96, 1)
+    assert torch.equal(m1, per_head)
+    # identical queries (and keys) inside a group: the group's choice is every head's own choice
+    q4 = q[:, ::4].repeat_interleave(4, dim=1)
+    k4 = k[:, ::4].repeat_interleave(4, dim=1)
+    m4, _ = P.quest_selector_group_dense(q4, k4, 16, 96, 4)
+    assert torch.equal(m4, P.quest_selector_dense(q4, k4, 16, 96)[0])
+    # different queries over shared keys: one mask per group, of the budget's size; brute force:
+    # no chunk outside it has a larger group score than a chunk inside it
+    kk = k[:, ::4].repeat_interleave(4, dim=1)
+    mg, _ = P.quest_selector_group_dense(q, kk, 16, 96, 4)
+    assert mg.sum(-1).unique().tolist() == [96]
+    mgr = mg.reshape(B, 2, 4, N)
+    assert (mgr == mgr[:, :, :1]).all()
+    sc = P.quest_chunk_scores_dense(q, kk, 16)[:, :, 0]                       # [B, H, 25]
+    for b in range(B):
+        for kv in range(2):
+            gsc = [max(float(sc[b, 4 * kv + j, c]) for j in range(4)) for c in range(25)]
+            chosen = [c for c in range(25) if mg[b, 4 * kv, 0, c * 16]]
+            assert len(chosen) == 6
+            assert min(gsc[c] for c in chosen) >= max(gsc[c] for c in range(25) if c not in chosen)
+
+
 def test_estimator_scores_is_a_matmul():
     g = torch.Generator().manual_seed(2)
     q = torch.randn((1, 4, 1, 128), generator=g).half().float()

@@ -28,7 +28,7 @@ EXPORTS = (
     "twl_strerror", "twl_abi_version", "twl_device_count", "twl_top_p_f32", "twl_top_p_f16",
     "twl_softmax_top_p_f32", "twl_gemv_top_p", "twl_select_estimate_prune", "twl_gemv_int4", "twl_gemv_int4_nhd",
     "twl_gemv_int8_nhd", "twl_gemv_f16_nhd", "twl_gemv_f16_single", "twl_sparse_attn",
-    "twl_sparse_attn_workspace_bytes", "twl_sparse_attn_static", "twl_sparse_attn_weighted",
+    "twl_sparse_attn_workspace_bytes", "twl_sparse_attn_static", "twl_sparse_attn_weighted", "twl_gemv_int4_group",
     "twl_group_attn",
     "twl_group_attn_workspace_bytes",
     "twl_group_union", "twl_rope_qk", "twl_quest_select",
@@ -63,6 +63,7 @@ class LayerArgs(ctypes.Structure):
         ("group_count", c_void_p),
         ("group_workspace", c_void_p), ("group_workspace_bytes", c_uint64),
         ("surv_probs", c_void_p), ("use_estimated_weights", c_int),
+        ("group_select", c_int),
     ]
 
 
@@ -100,6 +101,7 @@ def lib() -> ctypes.CDLL:
                                             vp, u32, vp, vp, u32, vp, u32, vp]
     L.twl_gemv_int4.argtypes = [vp, i32, vp, u32, vp, vp, vp, vp, u32, vp, vp, vp, u32, u32, u32,
                                 u32, f32, vp]
+    L.twl_gemv_int4_group.argtypes = L.twl_gemv_int4.argtypes
     L.twl_gemv_int4_nhd.argtypes = [vp, vp, u32, vp, vp, vp, vp, vp, vp, u32, u32, u32, u32, f32, vp]
     L.twl_gemv_int8_nhd.argtypes = L.twl_gemv_int4_nhd.argtypes
     L.twl_gemv_f16_nhd.argtypes = [vp, vp, u32, vp, vp, vp, vp, u32, u32, u32, u32, f32, vp]

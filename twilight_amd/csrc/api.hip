@@ -27,6 +27,10 @@ extern "C" int twl_device_count(void) {
   return n;
 }
 
+namespace twl {
+int layer_attention(const twl_layer_args* a, void* stream);
+}
+
 // twilight/pyimpl/attention.py:188-306 for q_len == 1: selector -> estimator -> pruner -> attention.
 extern "C" int twl_decode_layer(const twl_layer_args* a, void* stream) {
   if (!a) return TWL_ENULL;
@@ -49,6 +53,30 @@ extern "C" int twl_decode_layer(const twl_layer_args* a, void* stream) {
   if (k * TWL_PAGE > TWL_MAX_CANDIDATES) return TWL_EINVAL;
 
   int rc;
+  if (a->group_select && a->num_q_heads != a->num_kv_heads) {
+    // one candidate list per kv head: scores (group maximum) -> top-k -> group GEMV -> pruner
+    if (!a->page_scores || !a->meta || !a->k_int4) return TWL_ENULL;
+    rc = twl::quest_page_scores_ex(a->q, a->dtype, a->meta, a->kv_page_indices,
+                                   a->kv_page_indptr, a->batch, a->num_q_heads, a->num_kv_heads,
+                                   a->max_pages_per_req, a->page_scores, a->page_score_stride, 1,
+                                   stream);
+    if (rc != TWL_OK) return rc;
+    rc = twl_quest_topk_pages(a->page_scores, a->page_score_stride, a->kv_page_indptr, a->batch,
+                              a->num_q_heads, a->token_budget, a->max_pages_per_req,
+                              a->sel_pages, a->sel_stride, a->sel_count, stream);
+    if (rc != TWL_OK) return rc;
+    rc = twl_gemv_int4_group(a->q, a->dtype, a->scores, a->score_stride, a->cand_count, a->k_int4,
+                             a->sel_pages, a->sel_count, a->sel_stride, a->kv_page_indices,
+                             a->kv_page_indptr, a->kv_last_page_len, a->batch, a->num_q_heads,
+                             a->num_kv_heads, k, a->sm_scale, stream);
+    if (rc != TWL_OK) return rc;
+    rc = twl::softmax_top_p_ex(a->scores, a->score_stride, a->cand_count, rows, k * TWL_PAGE,
+                               nullptr, a->top_p, a->high_mode, a->sel_pages, a->sel_stride,
+                               a->idx, a->idx_stride, a->count, nullptr, nullptr, a->surv_probs,
+                               stream);
+    if (rc != TWL_OK) return rc;
+    return twl::layer_attention(a, stream);
+  }
   int cus = 0;
   const bool have_cus = twl::device_cu_count(&cus) == TWL_OK;
   // Fewer rows than half the compute units: a workgroup per row leaves most of the chip idle while
@@ -130,7 +158,12 @@ extern "C" int twl_decode_layer(const twl_layer_args* a, void* stream) {
       if (rc != TWL_OK) return rc;
     }
   }
-  // 4. exact attention over the survivors: per q head, or per kv head over the group's union
+  return twl::layer_attention(a, stream);
+}
+
+// 4. exact attention over the survivors: per q head, or per kv head over the group's union
+int twl::layer_attention(const twl_layer_args* a, void* stream) {
+  int rc;
   if (a->group_idx) {
     if (!a->group_count || !a->group_workspace) return TWL_ENULL;
     rc = twl_group_union(a->idx, a->idx_stride, a->count, a->batch, a->num_q_heads,

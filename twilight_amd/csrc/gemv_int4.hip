@@ -198,6 +198,134 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_int4_kernel(GemvArgs a) {
     if (grp * U + (lane >> 4) < np) orow[grp * U * TWL_PAGE + lane] = held[grp];
 }
 
+// The q heads of a kv head over ONE page list (that of the group's first q head): every INT4
+// record is fetched once and multiplied with the GROUP queries. The unpacked nibbles are shared;
+// per head the dot products, the scale / zero step and the quad reduction are those of
+// gemv_int4_kernel in the same order, so a head's scores equal what that kernel gives it over the
+// same list bit for bit.
+template <int QDT, int GROUP, int PW>
+__global__ __launch_bounds__(kGemvThreads) void gemv_int4_group_kernel(GemvArgs a) {
+  constexpr int U = kGemvUnroll;
+  constexpr int G = PW / U;
+  static_assert(PW % U == 0 && PW <= 64, "one lane per page id, whole groups");
+  const uint32_t b = blockIdx.y / a.num_kv_heads;
+  const uint32_t kvh = blockIdx.y - b * a.num_kv_heads;
+  const uint32_t row0 = b * a.num_q_heads + kvh * GROUP;  // the group's first q-head row
+  const int lane = lane_id();
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int p0 = (blockIdx.x * (kGemvThreads / kWave) + wave) * PW;
+
+  const int pg_begin = a.kv_page_indptr[b];
+  const int pg_end = a.kv_page_indptr[b + 1];
+  const int last_len = a.kv_last_page_len[b];
+  const int sel_n = a.sel_count ? a.sel_count[row0] : (int)a.sel_stride;
+  int my_logical = (lane < PW && (uint32_t)(p0 + lane) < a.sel_stride)
+                       ? a.sel_pages[(size_t)row0 * a.sel_stride + p0 + lane] : 0;
+  const int g4 = lane & 3;
+  const int t = lane >> 2;
+  const int req_pages = pg_end - pg_begin;
+  int n_pages = min(max(sel_n, 0), (int)a.max_pages);
+  if (req_pages <= 0) n_pages = 0;
+  if (blockIdx.x == 0 && threadIdx.x < GROUP && a.out_count)
+    a.out_count[row0 + threadIdx.x] = n_pages * TWL_PAGE;
+  if (p0 >= n_pages) return;
+  const int np = min(PW, n_pages - p0);
+  my_logical = min(max(my_logical, 0), req_pages - 1);
+  int my_phys = 0;
+  if (lane < np) my_phys = a.kv_page_indices[pg_begin + my_logical];
+
+  half2_t qp[GROUP][16];
+  float qsum[GROUP];
+#pragma unroll
+  for (int h = 0; h < GROUP; ++h) {
+    const uint16_t* qrow = (const uint16_t*)a.q + (size_t)(row0 + h) * TWL_HEAD_DIM + 32 * g4;
+    float qf[32];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const u32x4 v = *(const u32x4*)(qrow + 8 * i);
+      const uint32_t ws[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        qf[8 * i + 2 * j] = bits16_to_f32<QDT>(ws[j] & 0xFFFFu);
+        qf[8 * i + 2 * j + 1] = bits16_to_f32<QDT>(ws[j] >> 16);
+      }
+    }
+#pragma unroll
+    for (int w = 0; w < 4; ++w)
+#pragma unroll
+      for (int s2 = 0; s2 < 4; ++s2) {
+        half2_t pr = {q_to_half(qf[8 * w + s2]), q_to_half(qf[8 * w + s2 + 4])};
+        qp[h][4 * w + s2] = pr;
+      }
+    float qs = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 32; ++i) qs += (float)q_to_half(qf[i]);
+    qsum[h] = qs;
+  }
+
+  const size_t rec_stride = (size_t)a.num_kv_heads * TWL_INT4_RECORD_BYTES;
+  const uint8_t* base = a.k_int4 + (size_t)kvh * TWL_INT4_RECORD_BYTES + 16 * lane;
+  const float ninf = -__builtin_inff();
+  const int src_lane4 = 4 * (4 * (lane & 15) + (lane >> 4));
+  const uint32_t m = 0x00F000F0u, one = 0x3C003C00u;
+  u32x4 nib[U];
+  uint32_t sz[U];
+  float held[GROUP][G];
+#pragma unroll
+  for (int grp = 0; grp < G; ++grp) {
+    if (grp * U < np) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int i = grp * U + u;
+        const int phys = __builtin_amdgcn_readlane(my_phys, (i < np) ? i : 0);
+        const uint8_t* rec = base + (size_t)phys * rec_stride;
+        nib[u] = __builtin_nontemporal_load((const u32x4*)rec);
+        sz[u] = __builtin_nontemporal_load((const uint32_t*)(rec + 1024 - 12 * lane));
+      }
+      float mine[GROUP];
+#pragma unroll
+      for (int h = 0; h < GROUP; ++h) mine[h] = 0.0f;
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int i = grp * U + u;
+        // the page's 32 nibbles of this lane as 16 fp16 pairs, once for all heads
+        half2_t nb[16];
+        const uint32_t ws[4] = {nib[u].x, nib[u].y, nib[u].z, nib[u].w};
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          nb[4 * w + 0] = __builtin_bit_cast(half2_t, and_or(ws[w] << 4, m, one));
+          nb[4 * w + 1] = __builtin_bit_cast(half2_t, and_or(ws[w], m, one));
+          nb[4 * w + 2] = __builtin_bit_cast(half2_t, and_or(ws[w] >> 4, m, one));
+          nb[4 * w + 3] = __builtin_bit_cast(half2_t, and_or(ws[w] >> 8, m, one));
+        }
+        const float scale64 = f16_bits_to_f32(sz[u] & 0xFFFFu) * 64.0f;
+        const float zero = f16_bits_to_f32(sz[u] >> 16);
+        const int logical = __builtin_amdgcn_readlane(my_logical, (i < np) ? i : 0);
+        const int valid = (logical == req_pages - 1) ? last_len : TWL_PAGE;
+#pragma unroll
+        for (int h = 0; h < GROUP; ++h) {
+          float acc = 0.0f;
+#pragma unroll
+          for (int j = 0; j < 16; ++j) acc = __builtin_amdgcn_fdot2(nb[j], qp[h][j], acc, false);
+          const float part = quad_allreduce<OpSum>(fmaf(scale64, acc - qsum[h], zero * qsum[h]));
+          const float val = (t < valid) ? part * a.sm_scale : ninf;
+          mine[h] = (g4 == u) ? val : mine[h];
+        }
+      }
+#pragma unroll
+      for (int h = 0; h < GROUP; ++h)
+        held[h][grp] = as_f32(__builtin_amdgcn_ds_bpermute(src_lane4, as_i32(mine[h])));
+    }
+  }
+#pragma unroll
+  for (int h = 0; h < GROUP; ++h) {
+    float* orow = a.out + (size_t)(row0 + h) * a.out_stride + (size_t)p0 * TWL_PAGE;
+#pragma unroll
+    for (int grp = 0; grp < G; ++grp)
+      if (grp * U + (lane >> 4) < np) orow[grp * U * TWL_PAGE + lane] = held[h][grp];
+  }
+}
+
 // One workgroup of 16 wavefronts per (batch, head) row, the row's scores parked in LDS and written
 // out in one burst when the row is done. With about one row per compute unit (the stand-alone
 // benchmark shape: 256 rows of 2048 pages) every compute unit streams for the whole kernel and
@@ -391,3 +519,50 @@ extern "C" int twl_gemv_int4(const void* q, int q_dtype, float* out, uint32_t ou
   return hipGetLastError() == hipSuccess ? TWL_OK : TWL_ELAUNCH;
 }
 
+
+extern "C" int twl_gemv_int4_group(const void* q, int q_dtype, float* out, uint32_t out_stride,
+                                   int32_t* out_count, const void* k_int4,
+                                   const int32_t* sel_pages, const int32_t* sel_count,
+                                   uint32_t sel_stride, const int32_t* kv_page_indices,
+                                   const int32_t* kv_page_indptr, const int32_t* kv_last_page_len,
+                                   uint32_t batch, uint32_t num_q_heads, uint32_t num_kv_heads,
+                                   uint32_t max_pages_per_row, float sm_scale, void* stream) {
+  if (!q || !out || !k_int4 || !sel_pages || !kv_page_indices || !kv_page_indptr ||
+      !kv_last_page_len)
+    return TWL_ENULL;
+  if (q_dtype != TWL_F16 && q_dtype != TWL_BF16) return TWL_EDTYPE;
+  if (batch == 0 || num_q_heads == 0 || num_kv_heads == 0 || num_q_heads % num_kv_heads != 0)
+    return TWL_EINVAL;
+  const uint32_t group = num_q_heads / num_kv_heads;
+  if (group != 2 && group != 4 && group != 8) return TWL_EINVAL;
+  if (max_pages_per_row == 0 || (uint64_t)max_pages_per_row * TWL_PAGE > out_stride)
+    return TWL_EINVAL;
+  if (sel_stride < max_pages_per_row) return TWL_EINVAL;
+  if ((uint64_t)batch * num_q_heads > 65535u) return TWL_EINVAL;
+  if ((((uintptr_t)q) & 15u) || (((uintptr_t)k_int4) & 15u) || (((uintptr_t)out) & 3u))
+    return TWL_EALIGN;
+  twl::GemvArgs a{};
+  a.q = q; a.out = out; a.out_stride = out_stride; a.out_count = out_count;
+  a.k_int4 = (const uint8_t*)k_int4; a.sel_pages = sel_pages; a.sel_count = sel_count;
+  a.sel_stride = sel_stride; a.kv_page_indices = kv_page_indices; a.kv_page_indptr = kv_page_indptr;
+  a.kv_last_page_len = kv_last_page_len; a.num_q_heads = num_q_heads;
+  a.num_kv_heads = num_kv_heads; a.max_pages = max_pages_per_row; a.sm_scale = sm_scale;
+  hipStream_t st = (hipStream_t)stream;
+  // 16 pages per wavefront (measured at 8 x 8 kv heads x 512 pages: 8 pages 19.4 us, 16 pages
+  // 18.3, 32 pages 20.0): a kv head's list is short (the budget) and, besides batch x kv heads,
+  // the only source of parallelism, while every wavefront first converts the group's queries
+  constexpr int PW = 16;
+  const uint32_t per_block = PW * (twl::kGemvThreads / twl::kWave);
+  const dim3 grid((max_pages_per_row + per_block - 1) / per_block, batch * num_kv_heads);
+  const dim3 blk(twl::kGemvThreads);
+#define TWL_GEMV_GROUP(DT)                                                                        \
+  do {                                                                                            \
+    if (group == 2) hipLaunchKernelGGL((twl::gemv_int4_group_kernel<DT, 2, PW>), grid, blk, 0, st, a); \
+    else if (group == 4) hipLaunchKernelGGL((twl::gemv_int4_group_kernel<DT, 4, PW>), grid, blk, 0, st, a); \
+    else hipLaunchKernelGGL((twl::gemv_int4_group_kernel<DT, 8, PW>), grid, blk, 0, st, a);        \
+  } while (0)
+  if (q_dtype == TWL_F16) TWL_GEMV_GROUP(TWL_F16);
+  else TWL_GEMV_GROUP(TWL_BF16);
+#undef TWL_GEMV_GROUP
+  return hipGetLastError() == hipSuccess ? TWL_OK : TWL_ELAUNCH;
+}

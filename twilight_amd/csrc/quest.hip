@@ -31,6 +31,7 @@ struct QuestArgs {
   int32_t* sel_pages;
   uint32_t sel_stride;
   int32_t* sel_count;
+  int group_max;  // GROUP > 1: every q head of a group receives the group's largest score per page
 };
 
 constexpr int kQsThreads = 256;
@@ -146,6 +147,13 @@ __global__ __launch_bounds__(kQsThreads) void quest_score_kernel(QuestArgs a) {
       }
     }
   }
+  if (GROUP > 1 && a.group_max) {
+    float mx = keep[0];
+#pragma unroll
+    for (int g = 1; g < GROUP; ++g) mx = fmaxf(mx, keep[g]);
+#pragma unroll
+    for (int g = 0; g < GROUP; ++g) keep[g] = mx;
+  }
   // one store per wave and q head: 32 consecutive scores
   if (lane < np) {
 #pragma unroll
@@ -200,12 +208,15 @@ static void launch_score(int q_dtype, uint32_t batch, hipStream_t s, const twl::
   else launch_score_g<1>(q_dtype, dim3(gx, batch * a.num_q_heads), s, a);
 }
 
-extern "C" int twl_quest_page_scores(const void* q, int q_dtype, const void* meta,
-                                     const int32_t* kv_page_indices,
-                                     const int32_t* kv_page_indptr, uint32_t batch,
-                                     uint32_t num_q_heads, uint32_t num_kv_heads,
-                                     uint32_t max_pages_per_req, float* page_scores,
-                                     uint32_t score_stride, void* stream) {
+int twl::quest_page_scores_ex(const void* q, int q_dtype, const void* meta,
+                              const int32_t* kv_page_indices, const int32_t* kv_page_indptr,
+                              uint32_t batch, uint32_t num_q_heads, uint32_t num_kv_heads,
+                              uint32_t max_pages_per_req, float* page_scores,
+                              uint32_t score_stride, int group_max, void* stream) {
+  if (group_max) {
+    const uint32_t group = num_kv_heads ? num_q_heads / num_kv_heads : 0;
+    if (group != 2 && group != 4 && group != 8) return TWL_EINVAL;
+  }
   int rc = check_quest_common(q, q_dtype, meta, kv_page_indices, kv_page_indptr, batch,
                               num_q_heads, num_kv_heads, max_pages_per_req, page_scores,
                               score_stride);
@@ -214,8 +225,20 @@ extern "C" int twl_quest_page_scores(const void* q, int q_dtype, const void* met
   a.q = q; a.meta = (const uint8_t*)meta; a.kv_page_indices = kv_page_indices;
   a.kv_page_indptr = kv_page_indptr; a.num_q_heads = num_q_heads; a.num_kv_heads = num_kv_heads;
   a.max_pages = max_pages_per_req; a.page_scores = page_scores; a.score_stride = score_stride;
+  a.group_max = group_max;
   launch_score(q_dtype, batch, (hipStream_t)stream, a);
   return hipGetLastError() == hipSuccess ? TWL_OK : TWL_ELAUNCH;
+}
+
+extern "C" int twl_quest_page_scores(const void* q, int q_dtype, const void* meta,
+                                     const int32_t* kv_page_indices,
+                                     const int32_t* kv_page_indptr, uint32_t batch,
+                                     uint32_t num_q_heads, uint32_t num_kv_heads,
+                                     uint32_t max_pages_per_req, float* page_scores,
+                                     uint32_t score_stride, void* stream) {
+  return twl::quest_page_scores_ex(q, q_dtype, meta, kv_page_indices, kv_page_indptr, batch,
+                                   num_q_heads, num_kv_heads, max_pages_per_req, page_scores,
+                                   score_stride, 0, stream);
 }
 
 extern "C" int twl_quest_topk_pages(const float* page_scores, uint32_t score_stride,

@@ -286,6 +286,13 @@ int select_estimate_prune_ex(
     uint32_t score_stride, int32_t* cand_count, const void* meta_planes,
     uint32_t plane_cap_pages, const int32_t* plane_slots, uint32_t plane_num_slots,
     float* surv_probs, void* stream);
+// twl_quest_page_scores; with group_max every q head of a kv head's group receives the largest
+// of the group's scores for each page (2, 4 or 8 q heads per kv head)
+int quest_page_scores_ex(const void* q, int q_dtype, const void* meta,
+                         const int32_t* kv_page_indices, const int32_t* kv_page_indptr,
+                         uint32_t batch, uint32_t num_q_heads, uint32_t num_kv_heads,
+                         uint32_t max_pages_per_req, float* page_scores, uint32_t score_stride,
+                         int group_max, void* stream);
 int softmax_top_p_ex(const float* scores, uint32_t score_stride, const int32_t* lens,
                      uint32_t rows, uint32_t d, const float* p_arr, float p, int high_mode,
                      const int32_t* sel_pages, uint32_t sel_stride, int32_t* idx,

@@ -16,18 +16,23 @@ def sparse_gemv_int4(q: torch.Tensor, k_int4: torch.Tensor, kv_page_indices: tor
                      sel_pages: Optional[torch.Tensor] = None,
                      sel_count: Optional[torch.Tensor] = None,
                      max_pages: Optional[int] = None, sm_scale: Optional[float] = None,
-                     out: Optional[torch.Tensor] = None, out_count: Optional[torch.Tensor] = None):
+                     out: Optional[torch.Tensor] = None, out_count: Optional[torch.Tensor] = None,
+                     group_lists: bool = False):
     """``scores[b,h,c] = sm_scale * q[b,h,:] . dequant(K_int4[candidate c])`` in fp32.
 
     ``q`` [B,H,128] fp16/bf16; ``k_int4`` uint8 [pages, Hkv, 1280] INT4 shadow records;
     the CSR page table of the batch; ``sel_pages`` int32 [B,H,S] per-row ascending logical page
     lists with ``sel_count`` int32 [B,H] (both None: every page of the request, ``max_pages``
     = the longest request's page count). Candidate slots past a request's length are ``-inf``.
+    ``group_lists``: the q heads of a kv head share the page list of the group's first q head
+    (``twl_gemv_int4_group``: every record fetched once per kv head; 2, 4 or 8 q heads per kv head).
     Returns ``(scores fp32 [B,H,16*max_pages], cand_count int32 [B,H])``.
     """
     check_input(q, "q")
     check_dim(3, q, "q")
     B, H, D = q.shape
+    if group_lists and sel_pages is None:
+        raise RuntimeError("group_lists needs sel_pages")
     if D != _lib.HEAD_DIM:
         raise RuntimeError(f"head_dim must be {_lib.HEAD_DIM}, got {D}")
     check_input(k_int4, "k_int4")
@@ -77,7 +82,8 @@ def sparse_gemv_int4(q: torch.Tensor, k_int4: torch.Tensor, kv_page_indices: tor
         if out_count is None:
             out_count = torch.empty((B, H), dtype=torch.int32, device=dev)
         scale = 1.0 / math.sqrt(D) if sm_scale is None else float(sm_scale)
-        rc = _lib.lib().twl_gemv_int4(
+        entry = _lib.lib().twl_gemv_int4_group if group_lists else _lib.lib().twl_gemv_int4
+        rc = entry(
             ptr(q), dtype_code(q.dtype, "q"), ptr(out), out.size(2), ptr(out_count), ptr(k_int4),
             ptr(sel_pages), ptr(sel_count), sel_stride, ptr(kv_page_indices), ptr(kv_page_indptr),
             ptr(kv_last_page_len), B, H, Hkv, max_pages, scale, stream_of(q))

@@ -50,7 +50,8 @@ class TwilightDecodeLayer:
                  top_p: float = 0.85, high: str = "max", sm_scale: Optional[float] = None,
                  fused_estimator: bool = True, keep_scores: bool = False,
                  reserve_pages: int = 0, group_union: bool = False,
-                 sparsity_rate: float = -1, use_estimated_weights: bool = False):
+                 sparsity_rate: float = -1, use_estimated_weights: bool = False,
+                 group_select: bool = False):
         if num_q_heads % cache.num_kv_heads != 0:
             raise RuntimeError("num_q_heads must be a multiple of the cache's kv heads")
         if not (0.0 < top_p <= 1.0):
@@ -83,6 +84,12 @@ class TwilightDecodeLayer:
         self.use_estimated_weights = bool(use_estimated_weights)
         if self.use_estimated_weights and self.group_union:
             raise RuntimeError("use_estimated_weights and group_union exclude each other")
+        # group_select: one candidate list per kv head (a page scores the largest of its group's
+        # q-head scores), metadata and INT4 records read once per kv head; every q head still
+        # prunes and attends on its own scores. Not the reference's per-q-head selection.
+        self.group_select = bool(group_select) and num_q_heads != cache.num_kv_heads
+        if self.group_select and num_q_heads // cache.num_kv_heads not in (2, 4, 8):
+            raise RuntimeError("group_select needs 2, 4 or 8 q heads per kv head")
         self._alloc()
 
     @classmethod
@@ -171,6 +178,7 @@ class TwilightDecodeLayer:
             a.group_workspace_bytes = self.group_workspace.numel()
         if self.use_estimated_weights:
             a.surv_probs, a.use_estimated_weights = ptr(self.surv_probs), 1
+        a.group_select = 1 if self.group_select else 0
         return a
 
     def forward(self, q: torch.Tensor) -> torch.Tensor:
