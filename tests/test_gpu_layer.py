@@ -400,6 +400,81 @@ def test_full_size_layer_sampled_rows_and_properties(dev, B, H, Hkv, dt, p, plan
         assert e2e < 5 * tol, (r, e2e)
 
 
+def test_full_size_options_every_row(dev):
+    """The optional forms of the layer at the Llama-3 shape's full size (B=8, 32 q / 8 kv heads,
+    bf16, ctx 32768, budget 8192), every row, through properties that need no dense oracle:
+    use_estimated_weights (same lists, the survivors' estimator probabilities, out = sum w V /
+    sum w against a torch gather) and group_select (one list per kv head = the top pages of the
+    group's largest page scores; kept mass >= p on its own scores)."""
+    B, H, Hkv, N, budget, p, dt = 8, 32, 8, 32768, 8192, 0.9, torch.bfloat16
+    G, npg, rows = H // Hkv, N // 16, B * H
+    q, k, v, (ids, indptr, last) = synth.layer_inputs_device(B, H, Hkv, N, dt, dev, seed=4)
+    cache = PagedKVCache(B * npg, Hkv, dt, dev)
+    cache.k_cache, cache.v_cache = k, v
+    cache.set_page_table(ids, indptr, last)
+    cache.rebuild_shadow()
+    cache.enable_planes()
+    base = TwilightDecodeLayer(cache, H, token_budget=budget, top_p=p, keep_scores=True)
+    base(q)
+    est = TwilightDecodeLayer(cache, H, token_budget=budget, top_p=p, use_estimated_weights=True)
+    out = est(q).float()
+    assert torch.equal(est.count, base.count) and torch.isfinite(out).all()
+    cnt = base.count.reshape(rows)
+    pos = torch.arange(base.idx.shape[-1], device=dev)[None, :]
+    valid = pos < cnt[:, None]
+    assert torch.equal(torch.where(valid, est.idx.reshape(rows, -1), 0),
+                       torch.where(valid, base.idx.reshape(rows, -1), 0))
+    # the emitted weights are the softmax of the candidate scores at the survivors' slots
+    sel = base.sel_pages.reshape(rows, -1).long().contiguous()
+    idx = base.idx.reshape(rows, -1).long()
+    slot = torch.searchsorted(sel, (idx // 16).clamp(min=0).contiguous()).clamp(max=sel.shape[1] - 1)
+    cand = slot * 16 + idx % 16
+    probs = torch.softmax(base.scores.reshape(rows, -1), dim=-1)
+    want_w = torch.gather(probs, 1, cand.clamp(0, probs.shape[1] - 1))
+    got_w = est.surv_probs.reshape(rows, -1)
+    assert torch.allclose(torch.where(valid, got_w, 0), torch.where(valid, want_w, 0), rtol=1e-4, atol=1e-10)
+    # out = sum w V / sum w, for every row of at most 1024 survivors (all but a handful)
+    cap = 1024
+    short = (cnt <= cap).nonzero().squeeze(-1)
+    assert short.numel() >= rows * 0.9
+    r_b, r_kv = short // H, (short % H) // G
+    tok = idx[short, :cap].clamp(min=0)
+    phys = ids.long()[(r_b * npg)[:, None] + tok // 16]                       # physical page
+    vv = v[phys, tok % 16, r_kv[:, None]].float()                             # [rows', cap, 128]
+    w = torch.where(valid[short, :cap], got_w[short, :cap], 0.0)
+    wn = w / w.sum(-1, keepdim=True)
+    wn = torch.where((cnt[short] <= 128)[:, None], wn.to(dt).float(), wn)     # attention.py:302-304
+    ref = torch.einsum("rc,rcd->rd", wn, vv)
+    assert torch.allclose(out.reshape(rows, 128)[short], ref, rtol=8e-3, atol=8e-3)
+    del vv, est
+
+    grp = TwilightDecodeLayer(cache, H, token_budget=budget, top_p=p, group_select=True)
+    gout = grp(q)
+    assert torch.isfinite(gout.float()).all() and bool((grp.sel_count == 512).all())
+    gs = grp.sel_pages.reshape(B, Hkv, G, -1)
+    assert bool((gs == gs[:, :, :1]).all())
+    # the group's list = the 512 pages with the largest group score; the row kernel of `base`
+    # scores the same pages from the plane layout (another summation order): pages at the
+    # boundary may differ within rounding
+    gmax = base.page_scores.reshape(B, Hkv, G, -1)[..., :npg].amax(dim=2)     # [B, Hkv, npg]
+    kth = torch.sort(gmax, dim=-1, descending=True).values[..., 511]
+    chosen = torch.zeros_like(gmax, dtype=torch.bool)
+    chosen.scatter_(-1, gs[:, :, 0].long(), True)
+    tolr = 1e-3 * kth.abs().clamp(min=1.0)[..., None]
+    assert bool((gmax[chosen].reshape(B, Hkv, 512) >= (kth[..., None] - tolr)).all())
+    assert bool((torch.where(chosen, torch.full_like(gmax, -1e30), gmax) <= kth[..., None] + tolr).all())
+    # kept mass on the group layer's own scores
+    gcnt = grp.count.reshape(rows)
+    gvalid = pos < gcnt[:, None]
+    gsel = grp.sel_pages.reshape(rows, -1).long().contiguous()
+    gidx = grp.idx.reshape(rows, -1).long()
+    gslot = torch.searchsorted(gsel, (gidx // 16).clamp(min=0).contiguous()).clamp(max=gsel.shape[1] - 1)
+    assert bool(((torch.gather(gsel, 1, gslot) == gidx // 16) | ~gvalid).all())
+    gprobs = torch.softmax(grp.scores.reshape(rows, -1), dim=-1)
+    gkept = torch.where(gvalid, torch.gather(gprobs, 1, (gslot * 16 + gidx % 16).clamp(0, gprobs.shape[1] - 1)), 0.0)
+    assert float(gkept.sum(-1).min()) >= p - 1e-5
+
+
 @pytest.mark.parametrize("H,Hkv", [(8, 8), (8, 2)])
 def test_layer_step_replays_from_a_hip_graph(dev, H, Hkv):
     # a serving loop captures the decode step: every replay, with eager work and synchronisations
