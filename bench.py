@@ -660,6 +660,8 @@ def main() -> int:
                     help="keep the Quest metadata in the 512-byte record layout only")
     ap.add_argument("--group-union", action="store_true",
                     help="attention over the union of each kv head's survivor lists (GQA)")
+    ap.add_argument("--group-select", action="store_true",
+                    help="one Quest selection per kv head, INT4 records read once per group (GQA)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra-shapes", action="store_true",
                     help="default workload: skip the B=16 and the Llama-3-shape sections")
@@ -718,7 +720,8 @@ def main() -> int:
             cache.enable_planes()      # metadata also in plane layout: the row kernel reads half
         layers.append(TwilightDecodeLayer(cache, H, token_budget=args.budget, top_p=args.top_p,
                                           high="max", fused_estimator=not args.split_estimator,
-                                          group_union=args.group_union))
+                                          group_union=args.group_union,
+                                          group_select=args.group_select))
         qs.append(q)
     torch.cuda.synchronize()
     nl = len(layers)
@@ -999,7 +1002,8 @@ def main() -> int:
                                 f"(group 32), top-p {args.top_p}"),
                    "batch": B, "context": N, "budget": args.budget, "top_p": args.top_p,
                    "layers_rotated": nl, "survivors_mean": round(n_bar, 1),
-                   "survivors_max": n_max},
+                   "survivors_max": n_max,
+                   **({"group_select": True} if args.group_select else {})},
         "us_per_step_graph_replay": None if graph_us is None else round(graph_us, 2),
         "layer_bytes": layer_bytes,
         "layer_frac_of_hbm_peak": (round(layer_bytes / wall_us / 1e3 / HBM_PEAK_GBS, 4)
