@@ -216,6 +216,8 @@ def test_one_launch_row_kernel_equals_three_launches(dev, N, lens, budget, H, Hk
     (65536 + 48, 8192, 2, 2, torch.float16), # 4099 pages: three pages beyond two plane passes
     (1600, 320, 16, 4, torch.float16),       # GQA 4:1, 32 rows: a group's rows share an XCD
     (1000, 100, 4, 2, torch.bfloat16),       # GQA 2:1, 8 rows: rows in launch order
+    (1600, 320, 8, 1, torch.float16),        # eight q heads on one kv head
+    (34832, 8192, 8, 2, torch.bfloat16),     # GQA 4:1 with a second plane pass and a record tail
 ])
 def test_row_kernel_with_plane_metadata(dev, N, budget, H, Hkv, dt):
     """The plane layout (minima / maxima of all pages of a request contiguous per channel) against
