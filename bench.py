@@ -114,7 +114,7 @@ def cpu_baseline_cfg1(warmups: int = 3, repeats: int = 20):
 
 
 def cpu_baseline(N: int, H: int, budget: int, top_p: float, batch_scale: int, dev, seed: int = 0,
-                 warmups: int = 1, repeats: int = 3):
+                 warmups: int = 1, repeats: int = 3, survivors=None):
     """Times the CPU oracle (torch fp32 + the C quantiser and top-p restatement) on one batch
     element drawn by the generator the GPU workload uses (same planted heavy hitters), un-paged to
     dense K / V: one warm-up, the median of three runs, scaled by the batch size. The reference's
@@ -123,7 +123,9 @@ def cpu_baseline(N: int, H: int, budget: int, top_p: float, batch_scale: int, de
     from twilight_amd import synth
     torch.set_num_threads(os.cpu_count() or 1)
     threads = torch.get_num_threads()
-    qd, kd, vd, (ids, _, _) = synth.layer_inputs_device(1, H, H, N, torch.float16, dev, seed=seed)
+    qd, kd, vd, (ids, _, _) = synth.layer_inputs_device(1, H, H, N, torch.float16, dev, seed=seed,
+                                                        survivors=survivors, top_p=top_p,
+                                                        budget=budget)
     order = ids.long()
     q = qd.float().cpu().reshape(1, H, 1, 128)
     k = kd[order].reshape(N, H, 128).permute(1, 0, 2).float().cpu().reshape(1, H, N, 128).contiguous()
@@ -150,6 +152,7 @@ def cpu_baseline(N: int, H: int, budget: int, top_p: float, batch_scale: int, de
                    f"not (variant B); torch uses {threads} threads "
                    f"(os.cpu_count() = {os.cpu_count()}), the C quantiser / top-p one"),
         "survivors_mean": float(ra["mask"].sum(-1).float().mean()),
+        "survivors_median": float(ra["mask"].sum(-1).float().median()),
         "cfg1": cpu_baseline_cfg1(),
     }
 
@@ -500,8 +503,15 @@ class _Timed:
         return getattr(self._layer, name)
 
 
+def _planted_name(survivors) -> str:
+    return ("peaked (a fixed shift of 0.9 q, slots with replacement: most rows hold one "
+            "dominant token)" if survivors is None else
+            f"calibrated (shift solved per row for a top-p nucleus of {survivors[0]}-{survivors[1]} "
+            "tokens over the row's candidates)")
+
+
 def measure_shape(L, dev, B, H, Hkv, N, dt, budget, top_p, n_layers, steps, warmup,
-                  dense: bool = False):
+                  dense: bool = False, survivors=None):
     """One more shape of the same layer, measured the way the headline figure is: ``n_layers``
     independent caches visited round-robin, wall time per ``twl_decode_layer`` step, and the two
     kernels of the step timed alone with events. Returns a dict for the JSON line."""
@@ -512,7 +522,9 @@ def measure_shape(L, dev, B, H, Hkv, N, dt, budget, top_p, n_layers, steps, warm
     qcode = 1 if dt == torch.bfloat16 else 0
     layers, qs = [], []
     for li in range(n_layers):
-        q, k, v, (ids, indptr, last) = synth.layer_inputs_device(B, H, Hkv, N, dt, dev, seed=500 + 10 * li)
+        q, k, v, (ids, indptr, last) = synth.layer_inputs_device(
+            B, H, Hkv, N, dt, dev, seed=500 + 10 * li, survivors=survivors, top_p=top_p,
+            budget=budget)
         cache = PagedKVCache(B * npg, Hkv, dt, dev)
         cache.k_cache, cache.v_cache = k, v
         cache.set_page_table(ids, indptr, last)
@@ -532,7 +544,8 @@ def measure_shape(L, dev, B, H, Hkv, N, dt, budget, top_p, n_layers, steps, warm
     for i in range(n_layers):
         layers[i].forward(qs[i])
     torch.cuda.synchronize()
-    n_bar = float(torch.stack([l.count for l in layers]).float().mean())
+    cnts = torch.stack([l.count for l in layers]).float()
+    n_bar = float(cnts.mean())
     rows, kp = B * H, layers[0].k_pages
     M = kp * 16
     stream = torch.cuda.current_stream().cuda_stream
@@ -571,7 +584,8 @@ def measure_shape(L, dev, B, H, Hkv, N, dt, budget, top_p, n_layers, steps, warm
                        f"budget {budget}, p {top_p}, {n_layers} caches rotated",
            "us_per_layer": round(wall_us, 2), "steps": steps,
            "select_estimate_prune_us": round(row_us, 2), "sparse_attn_us": round(attn_us, 2),
-           "survivors_mean": round(n_bar, 1),
+           "survivors_mean": round(n_bar, 1), "survivors_median": float(cnts.median()),
+           "survivors_max": int(cnts.max()), "planted": _planted_name(survivors),
            "layer_bytes_per_q_head_lists": per_head, "frac_of_hbm_peak_per_q_head_lists": gb(per_head),
            "layer_bytes_read_by_design": by_design, "frac_of_hbm_peak_read_by_design": gb(by_design)}
     if H != Hkv:
@@ -662,6 +676,9 @@ def main() -> int:
                     help="attention over the union of each kv head's survivor lists (GQA)")
     ap.add_argument("--group-select", action="store_true",
                     help="one Quest selection per kv head, INT4 records read once per group (GQA)")
+    ap.add_argument("--planted", choices=["calibrated", "peaked"], default="calibrated",
+                    help="planted heavy hitters: calibrated = K shift solved per row so that top-p "
+                         "keeps 100-400 tokens; peaked = one fixed shift (median 2 kept tokens)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra-shapes", action="store_true",
                     help="default workload: skip the B=16 and the Llama-3-shape sections")
@@ -692,6 +709,7 @@ def main() -> int:
     if args.workload == "llama3-model":
         return bench_llama3_model(args, dev)
     llama = args.workload == "llama3"
+    survivors = (100, 400) if args.planted == "calibrated" else None
     B, H, Hkv, N, D = args.batch, 32, (8 if llama else 32), args.context, 128
     npg = N // 16
     dt = torch.bfloat16 if llama else torch.float16
@@ -711,7 +729,9 @@ def main() -> int:
     # left in the 256 MB last-level cache by the previous step.
     layers, qs = [], []
     for li in range(args.layers):
-        q, k, v, (ids, indptr, last) = synth.layer_inputs_device(B, H, Hkv, N, dt, dev, seed=10 * li)
+        q, k, v, (ids, indptr, last) = synth.layer_inputs_device(
+            B, H, Hkv, N, dt, dev, seed=10 * li, survivors=survivors, top_p=args.top_p,
+            budget=args.budget)
         cache = PagedKVCache(B * npg, Hkv, dt, dev)
         cache.k_cache, cache.v_cache = k, v
         cache.set_page_table(ids, indptr, last)
@@ -971,10 +991,24 @@ def main() -> int:
     if (not llama and not args.no_extra_shapes and not args.split_estimator and not args.no_planes
             and (B, N, args.budget) == (8, 32768, 8192)):
         es, ew = max(20, min(args.steps, 60)), max(4, min(args.warmup, 10))
+        # the same layer on the other planted workload (the headline of earlier runs)
+        other = None if survivors is not None else (100, 400)
+        extra["b8_" + ("peaked" if other is None else "calibrated")] = measure_shape(
+            L, dev, 8, 32, 32, N, torch.float16, args.budget, args.top_p, 4, es, ew, survivors=other)
         extra["cfg4_b16"] = measure_shape(L, dev, 16, 32, 32, N, torch.float16, args.budget,
-                                          args.top_p, 2, es, ew)
+                                          args.top_p, 2, es, ew, survivors=survivors)
+        # the rest of the batch axis of the reference's latency figure (figures/kernels.png)
+        free_b = torch.cuda.mem_get_info()[0]
+        for bb, ncache in ((32, 2), (64, 1)):
+            need = ncache * bb * N * 32 * 128 * 2 * 2 * 1.45   # K, V, INT4 shadow, metadata twice
+            if need > free_b * 0.9:
+                extra[f"cfg4_b{bb}"] = {"skipped": f"needs about {need / 2**30:.0f} GiB, "
+                                                   f"{free_b / 2**30:.0f} GiB free"}
+                continue
+            extra[f"cfg4_b{bb}"] = measure_shape(L, dev, bb, 32, 32, N, torch.float16, args.budget,
+                                                 args.top_p, ncache, 20, 4, survivors=survivors)
         extra["cfg5_layer"] = measure_shape(L, dev, 8, 32, 8, N, torch.bfloat16, args.budget, 0.9,
-                                            4, es, ew, dense=True)
+                                            4, es, ew, dense=True, survivors=survivors)
         # the whole model at that shape (32 layers, random weights), a few decode steps: tokens/s
         # of the patched model replayed from one HIP graph against the model's own dense decode
         margs = argparse.Namespace(**vars(args))
@@ -987,7 +1021,7 @@ def main() -> int:
 
     cpu = None
     if not args.no_cpu_baseline and not llama:
-        cpu = cpu_baseline(N, H, args.budget, args.top_p, B, dev)
+        cpu = cpu_baseline(N, H, args.budget, args.top_p, B, dev, survivors=survivors)
 
     line = {
         "metric": "\u00b5s/decode-layer at 32k ctx (select+prune+attn); GEMV & attn HBM GB/s vs peak",
@@ -1001,7 +1035,8 @@ def main() -> int:
                                 f"(page 16), context {N}, Quest budget {args.budget}, INT4 K estimate "
                                 f"(group 32), top-p {args.top_p}"),
                    "batch": B, "context": N, "budget": args.budget, "top_p": args.top_p,
-                   "layers_rotated": nl, "survivors_mean": round(n_bar, 1),
+                   "layers_rotated": nl, "planted": _planted_name(survivors),
+                   "survivors_mean": round(n_bar, 1), "survivors_median": float(counts.median()),
                    "survivors_max": n_max,
                    **({"group_select": True} if args.group_select else {})},
         "us_per_step_graph_replay": None if graph_us is None else round(graph_us, 2),

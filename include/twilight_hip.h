@@ -260,8 +260,10 @@ int twl_gemv_f16_single(const void* q, void* o, const void* k, uint32_t num_head
  * (page, token, kv_head, d) lives at page*page_stride + token*token_stride + kv_head*head_stride + d.
  * Rows longer than 128 survivors are split over several workgroups that meet in `workspace`
  * (256-byte aligned, at least twl_sparse_attn_workspace_bytes(rows, idx_stride) bytes, no initial
- * contents required: its first rows*4 bytes are ticket words tagged with a per-call number, so a
- * word left by a call that never finished counts as zero; a finished call leaves them zero).
+ * contents required: its first rows*8 bytes are 64-bit ticket words that carry a 48-bit tag of
+ * the call, drawn from a per-process random sequence, so a word left by a call that never
+ * finished, or memory that was never cleared, counts as zero unless it happens to hold the
+ * call's tag, a 2^-48 event per split row; a finished call leaves the words zero).
  * Two calls that share a workspace must not overlap in time. In a split row the
  * softmax weights are not rounded to the q dtype before the V product (the partial sums are
  * merged in fp32); a row of at most 128 survivors follows the reference rounding exactly.
@@ -280,8 +282,10 @@ int twl_sparse_attn(const void* q, void* out, int dtype, const void* k_cache, co
  * part of the library's device image (every GPU the library runs on holds it until the process
  * ends). The call allocates and frees nothing. Returns TWL_ETOOBIG when
  * twl_sparse_attn_workspace_bytes(batch * num_q_heads, idx_stride) exceeds that size (24 MiB hold
- * 512 rows of up to 8192 survivors). The first call on a device looks up the array's address
- * there and should happen outside graph capture. All calls on one GPU share the array: calls that
+ * 512 rows of up to 8192 survivors). The array used is the current device's: TWL_EINVAL when q
+ * does not live on the current device. The first call on a device looks up the array's address
+ * there and must happen outside stream capture (TWL_EINVAL on a capturing stream; later calls
+ * may be captured). All calls on one GPU share the array: calls that
  * overlap in time on one GPU (two streams, two threads) race. Nothing in the array has to be
  * cleared between calls (the ticket words are tagged per call), so the call is one launch. */
 #define TWL_STATIC_SCRATCH_BYTES (24u << 20)

@@ -74,7 +74,7 @@ def test_c_level_validation_without_gpu(hip_lib):
     assert L.twl_gemv_int4(fake, 0, fake, 8, 0, fake, 0, 0, 0, fake, fake, fake, 1, 1, 1, 1, 1.0, 0) == -2
     assert L.twl_gemv_int4(fake + 4, 0, fake, 16, 0, fake, 0, 0, 0, fake, fake, fake, 1, 1, 1, 1, 1.0, 0) == -4
     ws = L.twl_sparse_attn_workspace_bytes(1, 8)
-    assert ws == 256 + 130 * 4 and L.twl_sparse_attn_workspace_bytes(256, 8192) == 1024 + 256 * 64 * 520
+    assert ws == 256 + 130 * 4 and L.twl_sparse_attn_workspace_bytes(256, 8192) == 2048 + 256 * 64 * 520
     assert L.twl_sparse_attn(fake, fake, 0, fake, fake, 4096, 256, 128, 0, 8, fake, fake, fake,
                              1, 1, 1, 1.0, 0, fake, ws, 0) == -1
     assert L.twl_sparse_attn(fake, fake, 0, fake, fake, 4096, 256, 130, fake, 8, fake, fake, fake,

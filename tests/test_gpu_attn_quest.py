@@ -174,18 +174,20 @@ def test_sparse_attention_split_rows_share_a_workspace(dev):
             cache.kv_page_indptr, workspace=ws)
         ref = P.masked_attention(q.float(), k.float(), v.float(), mask, prob_dtype=torch.float16)[:, :, 0]
         assert torch.allclose(out.cpu().float(), ref, rtol=1e-3, atol=1e-3), trial
-        assert int(ws[:B * H * 4].view(torch.int32).abs().sum()) == 0
+        assert int(ws[:B * H * 8].view(torch.int64).abs().sum()) == 0
     # ticket words that are not zero when the call starts (a call that never finished, memory that
-    # was never cleared) carry another call's tag or none: they count as zero
-    ws[:B * H * 4].view(torch.int32).copy_(torch.tensor([2, 0x00070003, 0x7FFF0001, 1, -1, 0x12340017, 9, 3]))
+    # was never cleared) carry another call's 48-bit tag or none: they count as zero. Small
+    # counts, words shaped like (small tag << 16) | count, all ones, and arbitrary bits.
+    ws[:B * H * 8].view(torch.int64).copy_(torch.tensor(
+        [2, 0x00070003, 0x7FFF0001, 1, -1, (0x1234 << 16) | 0x17, 0x0123456789ABCDEF, 3 << 32]))
     out = K.sparse_paged_decode_attention(
         q[:, :, 0].contiguous().to(dev), cache.k_cache, cache.v_cache,
         torch.from_numpy(np.maximum(idx, 0)).reshape(B, H, N).to(dev),
         torch.from_numpy(count).reshape(B, H).to(dev), cache.kv_page_indices,
         cache.kv_page_indptr, workspace=ws)
     assert torch.allclose(out.cpu().float(), ref, rtol=1e-3, atol=1e-3)
-    split = torch.from_numpy(count).reshape(-1) > 128     # the rows that used their ticket
-    assert int(ws[:B * H * 4].view(torch.int32)[split].abs().sum()) == 0
+    split = torch.from_numpy(count).reshape(-1) > 512     # rows that used their ticket for sure
+    assert int(ws[:B * H * 8].view(torch.int64)[split].abs().sum()) == 0
 
 
 def test_attention_folds_positions_outside_the_request(dev):

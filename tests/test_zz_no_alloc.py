@@ -31,10 +31,11 @@ def _case(dev, B, H, N, lens, seed, dtype):
     return q.to(dev), cache, idx.to(dev), cnt.to(dev)
 
 
-def _run(L, static, q, cache, idx, cnt, ws=None):
+def _run(L, static, q, cache, idx, cnt, ws=None, out=None, lse=None):
     B, H, _ = q.shape
-    out = torch.full_like(q, float("nan"))
-    lse = torch.full((B, H), float("nan"), dtype=torch.float32, device=q.device)
+    if out is None:
+        out = torch.full_like(q, float("nan"))
+        lse = torch.full((B, H), float("nan"), dtype=torch.float32, device=q.device)
     ks = cache.k_cache.stride()
     code = _lib.TWL_F16 if q.dtype == torch.float16 else _lib.TWL_BF16
     head = (ptr(q), ptr(out), code, ptr(cache.k_cache), ptr(cache.v_cache), ks[0], ks[1], ks[2],
@@ -63,12 +64,17 @@ def test_static_scratch_entry_equals_workspace_entry(dev):
         ws = torch.zeros(int(L.twl_sparse_attn_workspace_bytes(B * H, N)), dtype=torch.uint8,
                          device=dev)
         ref_out, ref_lse = _run(L, False, q, cache, idx, cnt, ws)
+        # one untimed call first: the address lookup of the first call on a device is set-up
+        _run(L, True, q, cache, idx, cnt)
+        out = torch.full_like(q, float("nan"))
+        lse = torch.full((B, H), float("nan"), dtype=torch.float32, device=dev)
         torch.cuda.synchronize()
         free0 = torch.cuda.mem_get_info()[0]
         reserved0 = torch.cuda.memory_reserved()
-        # out / lse are allocated by the test before the call, as a caller's would be
-        out, lse = _run(L, True, q, cache, idx, cnt)
-        assert torch.cuda.memory_reserved() == reserved0 or torch.cuda.mem_get_info()[0] <= free0
+        out, lse = _run(L, True, q, cache, idx, cnt, out=out, lse=lse)
+        # neither torch's allocator nor the device lost memory to the call
+        assert torch.cuda.memory_reserved() == reserved0
+        assert torch.cuda.mem_get_info()[0] >= free0
         assert torch.equal(out.view(torch.int16), ref_out.view(torch.int16)), (B, H, N)
         assert torch.equal(lse.view(torch.int32), ref_lse.view(torch.int32)), (B, H, N)
         assert torch.isfinite(out.float()).all()

@@ -105,10 +105,22 @@ def identity_page_table(B: int, pages_per_req: int, last_len: int = PAGE, device
 
 def layer_inputs_device(B: int, H: int, Hkv: int, N: int, dtype: torch.dtype, device,
                         seed: int = 0, heavy_pages: int = 8, alpha: float = 0.9,
-                        shuffle_pages: bool = True):
+                        shuffle_pages: bool = True,
+                        survivors: Optional[Tuple[int, int]] = None, top_p: float = 0.95,
+                        budget: int = 8192):
     """Decode-layer inputs built on the GPU: q [B,H,128], paged K, V [B*N/16, 16, Hkv, 128]
-    ~ N(0,1) in ``dtype``; per (batch, q head) ``heavy_pages`` random pages get ``K += alpha*q`` on
-    3 of their tokens (planted heavy hitters). Returns (q, k_pages, v_pages, page table tuple)."""
+    ~ N(0,1) in ``dtype``; per (batch, q head) ``heavy_pages`` random pages get ``K += a*q`` on
+    3 of their tokens (planted heavy hitters). Returns (q, k_pages, v_pages, page table tuple).
+
+    ``survivors=None`` ("peaked" workload): ``a = alpha`` for every row and the 3 token slots of a
+    page are drawn with replacement, so most rows hold a token planted twice that takes nearly
+    all of the softmax mass (a top-p of 0.95 keeps 2 tokens at the median, thousands in the few
+    rows without such a token).
+
+    ``survivors=(lo, hi)`` ("calibrated" workload): the slots are distinct and ``a`` is solved per
+    row, by bisection on the row's own logits, so that a nucleus of mass ``top_p`` over the row's
+    ``budget`` Quest candidates (whole pages by the min/max upper bound, the planted pages among
+    them) holds a target number of tokens drawn log-uniformly from [lo, hi]."""
     assert N % PAGE == 0
     dev = torch.device(device)
     g = torch.Generator(device=dev)
@@ -127,6 +139,9 @@ def layer_inputs_device(B: int, H: int, Hkv: int, N: int, dtype: torch.dtype, de
     ids_d = ids.to(dev).long()
     group = H // Hkv
     gp = _gen(seed + 1)
+    if survivors is not None:
+        _plant_calibrated(q, k, ids_d, B, H, Hkv, npg, heavy_pages, gp, survivors, top_p, budget)
+        return q, k, v, (ids.to(dev), indptr.to(dev), last.to(dev))
     for b in range(B):
         for h in range(H):
             lp = torch.randperm(npg, generator=gp)[:heavy_pages]
@@ -137,3 +152,64 @@ def layer_inputs_device(B: int, H: int, Hkv: int, N: int, dtype: torch.dtype, de
                 cur = k[phys, slots[:, j], kvh].float()
                 k[phys, slots[:, j], kvh] = (cur + alpha * q[b, h].float()).to(dtype)
     return q, k, v, (ids.to(dev), indptr.to(dev), last.to(dev))
+
+
+def nucleus_size(logits: torch.Tensor, top_p: float) -> torch.Tensor:
+    """Size of the smallest set of entries of each row of ``logits`` [R, M] whose softmax mass
+    reaches ``top_p`` (sort descending, cumulative sum)."""
+    pr = torch.softmax(logits.double(), dim=-1)
+    cs = torch.cumsum(torch.sort(pr, dim=-1, descending=True).values, dim=-1)
+    return (cs < top_p).sum(-1) + 1
+
+
+def _plant_calibrated(q, k, ids_d, B, H, Hkv, npg, heavy_pages, gp, survivors, top_p, budget):
+    """Plants 3 distinct tokens in each of ``heavy_pages`` pages per (batch, q head) with
+    ``K += a*q``, ``a`` solved per row for a target nucleus size (see layer_inputs_device)."""
+    dev, dtype, D = q.device, q.dtype, HEAD_DIM
+    group = H // Hkv
+    kpages = min(npg, max(1, budget // PAGE) + (1 if budget % PAGE else 0))
+    lo_t, hi_t = survivors
+    hrow = torch.arange(H, device=dev)
+    kvh_of = hrow // group
+    for b in range(B):
+        phys_b = ids_d[b * npg:(b + 1) * npg]
+        kk = k[phys_b].float()                                       # [npg, 16, Hkv, D]
+        qf = q[b].float()                                            # [H, D]
+        logits = torch.einsum("pthd,hgd->hgpt", kk, qf.view(Hkv, group, D)).reshape(H, npg, PAGE)
+        logits /= math.sqrt(D)
+        pmax = kk.amax(1).permute(1, 0, 2)[kvh_of]                   # [H, npg, D]
+        pmin = kk.amin(1).permute(1, 0, 2)[kvh_of]
+        bound = torch.maximum(qf[:, None, :] * pmax, qf[:, None, :] * pmin).sum(-1)   # [H, npg]
+        del kk, pmax, pmin
+        lps, sls, tgt = [], [], []
+        for _ in range(H):
+            lps.append(torch.randperm(npg, generator=gp)[:heavy_pages])
+            sls.append(torch.stack([torch.randperm(PAGE, generator=gp)[:3]
+                                    for _ in range(heavy_pages)]))
+            u = float(torch.rand((), generator=gp))
+            tgt.append(math.exp(math.log(lo_t) + u * (math.log(hi_t) - math.log(lo_t))))
+        lp = torch.stack(lps).to(dev)                                # [H, heavy_pages]
+        sl = torch.stack(sls).to(dev)                                # [H, heavy_pages, 3]
+        target = torch.tensor(tgt, device=dev)
+        heavy = torch.zeros((H, npg, PAGE), dtype=torch.bool, device=dev)
+        hi_ = hrow[:, None, None].expand_as(sl)
+        heavy[hi_, lp[:, :, None].expand_as(sl), sl] = True
+        bound.scatter_(1, lp, float("inf"))                          # planted pages are selected
+        sel = torch.topk(bound, kpages, dim=1).indices               # [H, kpages]
+        take = sel[:, :, None].expand(-1, -1, PAGE)
+        cand = torch.gather(logits, 1, take).reshape(H, -1)
+        hm = torch.gather(heavy, 1, take).reshape(H, -1).float()
+        qq = (qf * qf).sum(-1) / math.sqrt(D)
+        a_lo = torch.zeros(H, device=dev)
+        a_hi = torch.full((H,), 4.0, device=dev)
+        for _ in range(28):
+            a = 0.5 * (a_lo + a_hi)
+            n = nucleus_size(cand + (a * qq)[:, None] * hm, top_p)
+            more = n.float() > target                                # too many kept: plant harder
+            a_lo = torch.where(more, a, a_lo)
+            a_hi = torch.where(more, a_hi, a)
+        a = 0.5 * (a_lo + a_hi)
+        pg = phys_b[lp][:, :, None].expand_as(sl)                    # [H, heavy_pages, 3] physical
+        hh = kvh_of[:, None, None].expand_as(sl)
+        cur = k[pg, sl, hh].float()                                  # [H, heavy_pages, 3, D]
+        k[pg, sl, hh] = (cur + a[:, None, None, None] * qf[:, None, None, :]).to(dtype)
