@@ -73,7 +73,14 @@ enum twl_dtype { TWL_F16 = 0, TWL_BF16 = 1, TWL_F32 = 2 };
 
 /* how the top-p bisection initialises its upper bound */
 enum twl_top_p_high {
-  TWL_HIGH_FIRST = 0, /* probs[row][0], as csrc/include/sampling.cuh:156-159 does */
+  TWL_HIGH_FIRST = 0, /* probs[row][0], as csrc/include/sampling.cuh:156-159 does: the
+                       * probability of token 0 of the context. Entry points that prune a
+                       * candidate list (page lists: twl_softmax_top_p_f32 with sel_pages,
+                       * twl_gemv_top_p, twl_select_estimate_prune, twl_decode_layer) take the
+                       * first candidate's probability when logical page 0 heads the list and
+                       * 0 otherwise (a token outside the selection has probability 0 on the
+                       * reference's full-length row): the search then ends at once and every
+                       * candidate with a positive probability is kept */
   TWL_HIGH_MAX = 1    /* the row maximum (paper Algorithm 1) */
 };
 

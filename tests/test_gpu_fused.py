@@ -79,11 +79,28 @@ def _case(dev, B, H, Hkv, npg, S, last_len, p, high, qdt, seed, ragged=True, per
     # 2. the pruned lists against the oracle run on the GPU's own scores
     x = torch.from_numpy(sc).masked_fill(torch.from_numpy(np.isinf(sc)), torch.finfo(torch.float32).min)
     hm = native.HIGH_MAX if high == "max" else native.HIGH_FIRST
+    if high == "first":
+        # The reference's bound is the probability of TOKEN 0 of the context on a full-length row
+        # (csrc/include/sampling.cuh:156-159 after attention.py:255,274-278): when logical page 0
+        # is not the list's first page the oracle sees an extra leading entry of probability 0
+        # (dropped again below), otherwise the candidate row as it is.
+        lead = torch.full((rows, 1), torch.finfo(torch.float32).min)
+        no0 = (sel.reshape(rows, S)[:, 0] != 0) | (cnt_in.reshape(rows) == 0)
+        xs = [torch.cat([lead[r], x[r]]) if no0[r] else torch.cat([x[r], lead[r]]) for r in range(rows)]
+        x = torch.stack(xs)
     p_np = top_p.numpy().astype(np.float32) if per_row_p else p
     live = np.nonzero(cnt_in.reshape(-1).numpy() > 0)[0]
-    om, oprobs, ol, _ = P.top_p_unnormalized(x.reshape(rows, 1, 1, M)[live], p_np[live] if per_row_p else p_np, hm)
-    pn = oprobs.reshape(len(live), M).numpy()
+    Mx = x.shape[1]
+    om, oprobs, ol, _ = P.top_p_unnormalized(x.reshape(rows, 1, 1, Mx)[live], p_np[live] if per_row_p else p_np, hm)
+    pn = oprobs.reshape(len(live), Mx).numpy()
     _, _, _, og = native.top_p_mask_f32(pn, p_np[live] if per_row_p else p_np, hm, return_margin=True)
+    om = om.reshape(len(live), Mx)
+    if high == "first":
+        # back to candidate positions (the padding entry has probability 0 and is never kept)
+        keep = [slice(1, Mx) if no0[r] else slice(0, M) for r in live]
+        assert not any(bool(om[i, 0]) for i, r in enumerate(live) if no0[r])
+        pn = np.stack([pn[i, k] for i, k in enumerate(keep)])
+        om = torch.stack([om[i, k] for i, k in enumerate(keep)])
     selr = sel.reshape(rows, S).numpy()
     gm = np.zeros((rows, M), dtype=bool)
     for r in range(rows):

@@ -47,15 +47,19 @@ def _assert_selection_ties(page_scores, gpu_pages, ora_mask0, npg):
 
 
 def _run_case(dev, B, H, Hkv, N, budget, p, dt, seed, shuffle=True, n_heavy=16, fused=True,
-              planes=False, rate=-1, use_est=False, group_select=False):
+              planes=False, rate=-1, use_est=False, group_select=False, high="max", sink=None):
     q, k, v = synth.heavy_hitter_qkv(B, H, N, n_heavy=n_heavy, mass=0.6, seed=seed, dtype=dt)
     group = H // Hkv
+    if sink is not None:
+        # an attention sink: token 0 of every kv head leans towards its group's first query
+        k[:, :, 0] = (k[:, :, 0] + sink * q[:, ::group, 0].repeat_interleave(group, dim=1)).to(dt).float()
+    HM = native.HIGH_FIRST if high == "first" else native.HIGH_MAX
     kk, vv = k[:, ::group].contiguous(), v[:, ::group].contiguous()        # one K/V per kv head
     npg = (N + 15) // 16
     perm = torch.randperm(B * npg, generator=torch.Generator().manual_seed(seed)) if shuffle else None
     cache = PagedKVCache.from_dense(kk.to(dt), vv.to(dt), dev, page_perm=perm,
                                     plane_pages=npg if planes else None)
-    layer = TwilightDecodeLayer(cache, H, token_budget=budget, top_p=p, high="max",
+    layer = TwilightDecodeLayer(cache, H, token_budget=budget, top_p=p, high=high,
                                 fused_estimator=fused, keep_scores=True, sparsity_rate=rate,
                                 use_estimated_weights=use_est, group_select=group_select)
     if rate != -1:
@@ -64,14 +68,14 @@ def _run_case(dev, B, H, Hkv, N, budget, p, dt, seed, shuffle=True, n_heavy=16, 
     krep = kk.repeat_interleave(group, dim=1)                               # attention.py:124-126
     vrep = vv.repeat_interleave(group, dim=1)
     ref = P.decode_layer_dense(q, krep, vrep, top_p=p, token_budget=budget if budget < N else None,
-                               high_mode=native.HIGH_MAX, quant="storage", prob_dtype=dt,
+                               high_mode=HM, quant="storage", prob_dtype=dt,
                                sparsity_rate=rate, use_estimated_weights=use_est)
     est_pg = None
     if group_select:
         # one candidate list per kv head: the oracle's group selection replaces the per-head one
         gmask, gsc = P.quest_selector_group_dense(q.float(), krep.float(), 16, budget, group)
         est_pg = gsc[:, :, 0].reshape(B * H, -1)
-        ref = P.decode_layer_dense(q, krep, vrep, top_p=p, token_budget=budget, high_mode=native.HIGH_MAX,
+        ref = P.decode_layer_dense(q, krep, vrep, top_p=p, token_budget=budget, high_mode=HM,
                                    quant="storage", prob_dtype=dt, use_estimated_weights=use_est,
                                    mask0=gmask)
     rows = B * H
@@ -90,7 +94,7 @@ def _run_case(dev, B, H, Hkv, N, budget, p, dt, seed, shuffle=True, n_heavy=16, 
             est_pg = P.quest_chunk_scores_dense(q.float(), krep.float(), 16)[:, :, 0].reshape(rows, -1)
         for r in differ:
             _assert_selection_ties(est_pg[r], sel[r, :selc[r]], mask0[r], npg)
-        ref = P.decode_layer_dense(q, krep, vrep, top_p=p, token_budget=budget, high_mode=native.HIGH_MAX,
+        ref = P.decode_layer_dense(q, krep, vrep, top_p=p, token_budget=budget, high_mode=HM,
                                    quant="storage", prob_dtype=dt, use_estimated_weights=use_est,
                                    mask0=torch.from_numpy(gmask0).reshape(B, H, 1, N))
     # 2. estimator scores on the selected candidates (1e-3 relative)
@@ -108,7 +112,7 @@ def _run_case(dev, B, H, Hkv, N, budget, p, dt, seed, shuffle=True, n_heavy=16, 
     cnt = layer.count.cpu().numpy().reshape(rows)
     gm = _lists_to_mask(idx, cnt, N)
     probs = ref["probs"].reshape(rows, N).numpy()
-    _, _, _, margin = native.top_p_mask_f32(probs, p, native.HIGH_MAX, return_margin=True)
+    _, _, _, margin = native.top_p_mask_f32(probs, p, HM, return_margin=True)
     assert_top_p_parity(probs, p, gm, ref["mask"].reshape(rows, N).numpy(), ref["low"], margin,
                         margin_tol=5e-6)
     # 4. attention: exact over the GPU's own survivors, and end to end against the oracle
@@ -144,6 +148,41 @@ def test_cfg1_full_context(dev, fused):
 @pytest.mark.parametrize("fused", [True, False])
 def test_small_layer_configs(dev, B, H, Hkv, N, budget, p, dt, fused):
     _run_case(dev, B, H, Hkv, N, budget, p, dt, seed=B * 100 + H, n_heavy=8, fused=fused)
+
+
+@pytest.mark.parametrize("B,H,Hkv,N,budget,dt,fused,planes", [
+    (2, 8, 8, 2048, 512, torch.float16, True, False),     # estimator + pruner in one launch
+    (2, 8, 8, 2048, 512, torch.float16, False, False),    # every stage its own launch
+    (8, 32, 32, 1024, 256, torch.float16, True, True),    # the one-launch row kernel
+    (2, 8, 2, 2048, 512, torch.bfloat16, True, False),    # GQA
+])
+@pytest.mark.parametrize("sink", [None, 0.6, 1.5])
+def test_layer_high_first_is_the_reference_bound(dev, B, H, Hkv, N, budget, dt, fused, planes, sink):
+    """high="first": the bisection starts from the probability of TOKEN 0 of the context, as
+    csrc/include/sampling.cuh:156-159 does on the full-length row that attention.py:274-278 hands
+    it. Without a sink page 0 is rarely among the selected pages: token 0 then has probability 0,
+    the loop ends at once and every candidate with a positive probability is kept. With a sink
+    token 0 is a candidate; a moderate one (0.6, about as heavy as the planted tokens) is often
+    not the row maximum, so the result is a superset of the minimal set; a strong one (1.5) is
+    the maximum. With q heads sharing kv heads the sink leans towards the group's first query."""
+    layer, ref = _run_case(dev, B, H, Hkv, N, budget, 0.9, dt, seed=11 * B + H, n_heavy=8, fused=fused,
+                           planes=planes, high="first", sink=sink)
+    rows = B * H
+    sel = layer.sel_pages.cpu().numpy().reshape(rows, -1)
+    cnt = layer.count.cpu().numpy().reshape(rows)
+    cand = layer.cand_count.cpu().numpy().reshape(rows)
+    no_page0 = sel[:, 0] != 0
+    if sink is None:
+        assert no_page0.any()
+        # nothing is pruned in those rows (probabilities that underflow to 0 aside)
+        probs = ref["probs"].reshape(rows, N).numpy()
+        assert np.array_equal(cnt[no_page0], (probs[no_page0] > 0).sum(-1))
+        assert (cnt[no_page0] >= 0.9 * np.minimum(cand[no_page0], N)).all()
+    else:
+        lead = (np.arange(rows) % H) % (H // Hkv) == 0      # the rows the sink was planted for
+        with0 = lead & ~no_page0
+        assert with0.sum() >= 0.5 * lead.sum()      # the sink page is selected in most rows
+        assert (cnt[with0] < cand[with0]).all()     # and there the search prunes
 
 
 @pytest.mark.parametrize("B,H,Hkv,N,budget", [
@@ -315,18 +354,23 @@ def test_append_kernel_records_equal_bulk_build(dev, dt):
         assert torch.equal(getattr(cache, name)[ia], getattr(full, name)[ib]), name
 
 
-@pytest.mark.parametrize("B,H,Hkv,dt,p,planes", [
-    (16, 32, 32, torch.float16, 0.95, False),   # Longchat-7B shape (32 MHA heads, fp16), records
-    (16, 32, 32, torch.float16, 0.95, True),    # the same through the plane-layout metadata
-    (8, 32, 8, torch.bfloat16, 0.90, True),     # Llama-3-8B shape (32 q / 8 kv heads, bf16)
+@pytest.mark.parametrize("B,H,Hkv,dt,p,planes,survivors", [
+    (16, 32, 32, torch.float16, 0.95, False, None),       # Longchat-7B shape (32 MHA heads, fp16), records
+    (16, 32, 32, torch.float16, 0.95, True, (100, 400)),  # through the plane-layout metadata, on the
+                                                          # benchmark's calibrated heavy hitters
+    (8, 32, 8, torch.bfloat16, 0.90, True, None),         # Llama-3-8B shape (32 q / 8 kv heads, bf16)
+    (8, 32, 8, torch.bfloat16, 0.90, True, (100, 400)),
 ])
-def test_full_size_layer_sampled_rows_and_properties(dev, B, H, Hkv, dt, p, planes):
+def test_full_size_layer_sampled_rows_and_properties(dev, B, H, Hkv, dt, p, planes, survivors):
     # The two model shapes of the headline benchmark at their full size: ctx 32768, paged KV (shuffled pages), Quest
-    # budget 8192. The oracle (dense, CPU) checks a sample of (batch, head) rows end to end;
+    # budget 8192, on both planted workloads of the benchmark. The oracle (dense, CPU) checks 32
+    # (batch, head) rows end to end: the longest, the shortest and 30 drawn at random;
     # size-independent properties check every row.
     N, budget = 32768, 8192
     npg = N // 16
-    q, k, v, (ids, indptr, last) = synth.layer_inputs_device(B, H, Hkv, N, dt, dev, seed=3)
+    q, k, v, (ids, indptr, last) = synth.layer_inputs_device(B, H, Hkv, N, dt, dev, seed=3,
+                                                             survivors=survivors, top_p=p,
+                                                             budget=budget)
     cache = PagedKVCache(B * npg, Hkv, dt, dev)
     cache.k_cache, cache.v_cache = k, v
     cache.set_page_table(ids, indptr, last)
@@ -362,8 +406,14 @@ def test_full_size_layer_sampled_rows_and_properties(dev, B, H, Hkv, dt, p, plan
     # sampled rows against the dense oracle
     ids_c = ids.cpu().long()
     rng = np.random.default_rng(0)
-    long_row = int(np.argmax(cnt))
-    picks = sorted(set([long_row] + [int(r) for r in rng.integers(0, rows, 5)]))
+    picks = [int(np.argmax(cnt)), int(np.argmin(cnt))]
+    while len(picks) < 32:
+        r = int(rng.integers(0, rows))
+        if r not in picks:
+            picks.append(r)
+    if survivors is not None:
+        # the generator's target: a nucleus of 100-400 tokens per row
+        assert survivors[0] * 0.8 <= np.median(cnt) <= survivors[1] * 1.2, np.median(cnt)
     tol = 1e-3 if dt == torch.float16 else 8e-3
     for r in picks:
         b, h = divmod(r, H)

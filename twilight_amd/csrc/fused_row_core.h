@@ -194,7 +194,12 @@ __device__ __forceinline__ void estimate_prune_row(const FusedArgs& a, FusedSmem
   const float p = a.p_arr ? a.p_arr[row] : a.p;
   float high;
   if (a.high_mode == TWL_HIGH_FIRST) {
-    if (tx == 0) first = x[0];  // candidate 0 = wave 0, lane 0, group 0
+    // csrc/include/sampling.cuh:156-159 reads probs[row, 0], the probability of TOKEN 0 of the
+    // context, on a full-length row in which tokens outside the selection have probability 0
+    // (attention.py:255,274-278). Candidate 0 (wave 0, lane 0, group 0) is token 0 exactly when
+    // logical page 0 heads the ascending page list; otherwise the bound is 0, the loop ends at
+    // once and every candidate with a positive probability is kept.
+    if (tx == 0) first = (n_pages > 0 && my_logical[0] == 0) ? x[0] : 0.0f;
     __syncthreads();
     high = first;
   } else {

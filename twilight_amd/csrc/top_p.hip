@@ -97,9 +97,14 @@ __global__ __launch_bounds__(THREADS) void top_p_kernel(TopPArgs a) {
   const float p = round_to<DT>(a.p_arr ? a.p_arr[row] : a.p);
   float high;
   if (a.high_mode == TWL_HIGH_FIRST) {
-    // element 0 lives in thread 0, slot 0
+    // element 0 lives in thread 0, slot 0. With a page list it stands for token 0 of the context
+    // (what csrc/include/sampling.cuh:156-159 reads on its full-length row) only when logical
+    // page 0 heads the ascending list; a token outside the list has probability 0 there.
     __shared__ float first;
-    if (tx == 0) first = (len > 0) ? x[0] : 0.0f;
+    if (tx == 0) {
+      const bool is_token0 = !a.sel_pages || a.sel_pages[(size_t)row * a.sel_stride] == 0;
+      first = (len > 0 && is_token0) ? x[0] : 0.0f;
+    }
     __syncthreads();
     high = first;
   } else if (FUSED_SOFTMAX) {
