@@ -195,14 +195,17 @@ def bench_topp(args, L, dev) -> int:
            for i in range(4)]
     masks = {}
     mask = torch.empty((rows, M), dtype=torch.uint8, device=dev)
-    for name, dt in (("fp32", torch.float32), ("fp16", torch.float16), ("bf16", torch.bfloat16)):
+    for name, dt in (("fp32", torch.float32), ("fp32_exact", torch.float32), ("fp16", torch.float16),
+                     ("bf16", torch.bfloat16)):
         ps = [torch.softmax(x, -1).to(dt).contiguous() for x in xs1]
         state = {"i": 0}
 
         def call_mask():
             pr = ps[state["i"] % 4]
             state["i"] += 1
-            if dt == torch.float32:
+            if name == "fp32_exact":
+                L.twl_top_p_f32_exact(pr.data_ptr(), mask.data_ptr(), 0, 0, 0, 0.95, rows, M, M, 0, 0, 0, stream)
+            elif dt == torch.float32:
                 L.twl_top_p_f32(pr.data_ptr(), mask.data_ptr(), 0, 0, 0, 0.95, rows, M, M, 0, 0, 0, stream)
             else:
                 L.twl_top_p_f16(pr.data_ptr(), 0 if dt == torch.float16 else 1, mask.data_ptr(), 0, 0, 0,
@@ -216,9 +219,10 @@ def bench_topp(args, L, dev) -> int:
                                    "sets of 1-512 tokens per row, high = row max"},
             "per_p": res,
             "mask_ops_us_p095": masks,
-            "mask_ops_what": "twl_top_p_f32 / twl_top_p_f16 on [8, 32, 8192] probabilities writing "
-                             "the byte mask; the 16-bit forms run the reference's 16-bit arithmetic "
-                             "in cub::BlockReduce's order (1024 threads per row)"}
+            "mask_ops_what": "twl_top_p_f32 / twl_top_p_f32_exact / twl_top_p_f16 on [8, 32, 8192] "
+                             "probabilities writing the byte mask; fp32_exact and the 16-bit forms "
+                             "run the reference's arithmetic in cub::BlockReduce's order (1024 "
+                             "threads per row)"}
     print(json.dumps(line))
     return 0
 

@@ -87,7 +87,7 @@ enum twl_top_p_high {
 const char* twl_strerror(int status);
 /* ABI version of this header; bumps when a signature changes. twl_abi_version() returns the
  * version the library was built with: a caller compares the two before anything else. */
-#define TWL_ABI_VERSION 9
+#define TWL_ABI_VERSION 10
 int twl_abi_version(void);
 /* Number of HIP devices visible, or a negative twl_status. */
 int twl_device_count(void);
@@ -120,6 +120,17 @@ int twl_top_p_f32(const float* probs, uint8_t* mask, int32_t* idx, int32_t* coun
 int twl_top_p_f16(const void* probs, int dtype, uint8_t* mask, int32_t* idx, int32_t* count,
                   const float* p_arr, float p, uint32_t rows, uint32_t d, uint32_t idx_stride,
                   int high_mode, float* low_out, int32_t* iters_out, void* stream);
+/* twl_top_p_f32 with the additions of the reference's DType = float instantiation
+ * (csrc/src/sampling.cu:45-63) in the order of cub::BlockReduce<float, 1024,
+ * BLOCK_REDUCE_WARP_REDUCTIONS> (sampling.cuh:54; VEC = gcd(4, d)), as twl_top_p_f16 has them for
+ * the 16-bit types: masks, low_out and iters_out equal the reference kernel's on every row, also
+ * where a partial sum meets p within a rounding error (there twl_top_p_f32, which adds in an
+ * order of its own and is about three times faster, may decide an iteration the other way and
+ * keep a set that differs by tokens within 1e-5 of the pivot). Same arguments as twl_top_p_f32. */
+int twl_top_p_f32_exact(const float* probs, uint8_t* mask, int32_t* idx, int32_t* count,
+                        const float* p_arr, float p, uint32_t rows, uint32_t d,
+                        uint32_t idx_stride, int high_mode, float* low_out, int32_t* iters_out,
+                        void* stream);
 
 /* ---------------------------------------------------------------------------------------------
  * Fused softmax + top-p + stream compaction over raw (un-normalised) scores.

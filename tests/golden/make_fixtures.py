@@ -15,7 +15,7 @@ cross-checked against the literal it is expected to equal:
   ``high`` = the first element) is followed by hand: 3 iterations, final low 0.25.
 * ``top_p_dyadic`` — rows of powers of two, whose bisection is exact in every arithmetic width: the
   one vector that pins the 16-bit entry point independently of how its sums are ordered.
-* ``top_p_cub_order`` — rows for TopPReturnMaskKernel instantiated with a 16-bit DType
+* ``top_p_cub_order`` — rows for TopPReturnMaskKernel instantiated with a 16-bit DType or float
   (csrc/src/sampling.cu:22-43), where p, the pivots, the width test and every partial sum live in
   half / bfloat16 and the order of the additions is that of cub::BlockReduce with
   BLOCK_REDUCE_WARP_REDUCTIONS (csrc/include/sampling.cuh:54,171-217): each of the 1024 threads
@@ -116,7 +116,7 @@ def top_p_dyadic():
 
 
 # ---- the 16-bit instantiation in CUB's order ------------------------------------------------------
-FORMATS = {"f16": (11, -14), "bf16": (8, -126)}     # significand bits (with the hidden one), e_min
+FORMATS = {"f16": (11, -14), "bf16": (8, -126), "f32": (24, -126)}   # significand bits (with the hidden one), e_min
 
 
 def rne(x, fmt):
@@ -145,6 +145,9 @@ def bits_to_frac(b, fmt):
     if fmt == "f16":
         e, m = (b >> 10) & 31, b & 1023
         return F(m, 1 << 24) if e == 0 else F(1024 + m, 1024) * F(2) ** (e - 15)
+    if fmt == "f32":
+        e, m = (b >> 23) & 255, b & ((1 << 23) - 1)
+        return F(m, 1 << 23) * F(2) ** -126 if e == 0 else F((1 << 23) + m, 1 << 23) * F(2) ** (e - 127)
     e, m = (b >> 7) & 255, b & 127
     return F(m, 128) * F(2) ** -126 if e == 0 else F(128 + m, 128) * F(2) ** (e - 127)
 
@@ -181,6 +184,7 @@ def _check_rounding():
         b = (u + 0x7FFF + ((u >> 16) & 1)) >> 16
         f32 = F(struct.unpack("<f", struct.pack("<f", v))[0])
         assert rne(f32, "bf16") == bits_to_frac(b, "bf16") and frac_to_bits(rne(f32, "bf16"), "bf16") == b
+        assert rne(F(v), "f32") == f32 and bits_to_frac(u, "f32") == f32 and frac_to_bits(f32, "f32") == u
     assert rne(F(1, 100000), "f16") == F(168, 1 << 24) and rne(F(3, 1 << 25), "f16") == F(2, 1 << 24)
 
 
@@ -202,7 +206,7 @@ def cub_block_sums(kept, d, fmt, alt=None):
     from math import gcd
     R = (lambda x: x) if alt == "exact_sums" else (lambda x: rne(x, fmt))
     add = lambda x, y: y if x == 0 else (x if y == 0 else R(x + y))   # adding 0 is exact
-    vec = gcd(8, d)
+    vec = gcd(4 if fmt == "f32" else 8, d)            # 16 / sizeof(DType), sampling.cuh:239
     if alt == "flat_sum":                       # one running sum over the row
         return reduce(add, [kept[i] for i in sorted(kept)], F(0))
     by_chunk = {}
@@ -274,6 +278,8 @@ def _random_row(rng, fmt, d, nnz):
 def _targeted_rows(fmt):
     """Rows built for the mistakes a random search rarely meets."""
     from fractions import Fraction as F
+    if fmt == "f32":
+        return []      # the 16-bit rows below live on the grid of binary16 subnormals
     u = F(1, 1 << 24)
     rows = []
     # width of the final bracket exactly fmt(1e-5) = 168 * 2^-24: the loop stops; with an
@@ -294,9 +300,11 @@ def top_p_cub_order():
     from fractions import Fraction as F
     _check_rounding()
     out = []
-    for fmt in ("f16", "bf16"):
-        rng = random.Random(7 if fmt == "f16" else 8)
-        missing = set(ALTS)
+    for fmt in ("f16", "bf16", "f32"):
+        rng = random.Random({"f16": 7, "bf16": 8, "f32": 9}[fmt])
+        # float: 1e-5 and its float rounding have no float between them, so a bracket width is
+        # on the same side of both: that mistake cannot show, the other six can
+        missing = set(ALTS) - ({"exact_eps"} if fmt == "f32" else set())
         shapes = [(16, 16), (320, 70), (2048, 90), (12, 12), (8 * 1024 + 24, 140), (10, 10), (7, 7),
                   (3 * 8 * 1024, 200)]
         cands = [(r, d, hf, None) for r, d, hf in _targeted_rows(fmt)]
@@ -342,8 +350,8 @@ def top_p_cub_order():
                             "differs_under": hit})
                 break
         assert not missing and min(per_shape.values()) > 0, (fmt, missing, per_shape)
-    return {"source": "csrc/include/sampling.cuh:119-231 with DType = half / nv_bfloat16 "
-                      "(csrc/src/sampling.cu:22-43), sums in the order of cub::BlockReduce "
+    return {"source": "csrc/include/sampling.cuh:119-231 with DType = half / nv_bfloat16 / float "
+                      "(csrc/src/sampling.cu:22-63), sums in the order of cub::BlockReduce "
                       "BLOCK_REDUCE_WARP_REDUCTIONS, exact rational arithmetic + explicit rounding",
             "rows": out}
 

@@ -66,16 +66,20 @@ def test_oracle_top_p_on_the_dyadic_rows_in_every_width():
 
 def _cub_row(r):
     """(bits uint16 [1, d], dtype code, high mode) of one ``top_p_cub_order`` fixture row."""
-    bits = np.zeros((1, r["d"]), np.uint16)
+    code = {"f16": 0, "bf16": 1, "f32": 2}[r["dtype"]]
+    bits = np.zeros((1, r["d"]), np.uint32 if code == 2 else np.uint16)
     for i, b in r["nonzero"]:
         bits[0, i] = b
-    return bits, (0 if r["dtype"] == "f16" else 1), \
-        (native.HIGH_FIRST if r["high"] == "first" else native.HIGH_MAX)
+    if code == 2:
+        bits = bits.view(np.float32)          # the float oracle takes the values themselves
+    return bits, code, (native.HIGH_FIRST if r["high"] == "first" else native.HIGH_MAX)
 
 
 def _low_bits(low: float, code: int) -> int:
     if code == 0:
         return int(np.float32(low).astype(np.float16).view(np.uint16))
+    if code == 2:
+        return int(np.float32(low).view(np.uint32))
     return int(np.float32(low).view(np.uint32) >> 16)
 
 
@@ -90,10 +94,11 @@ def test_oracle_top_p_in_16_bit_arithmetic_and_cub_order():
         assert np.nonzero(mask[0])[0].tolist() == r["kept"], (r["dtype"], r["d"])
         assert _low_bits(low[0], code) == r["low_bits"] and iters[0] == r["iterations"]
         seen |= {(r["dtype"], a) for a in r["differs_under"]}
-    for fmt in ("f16", "bf16"):
+    for fmt in ("f16", "bf16", "f32"):
         for alt in ("exact_sums", "flat_sum", "thread_tree", "warp_tree", "chunks_merged",
                     "exact_mid", "exact_eps"):
-            assert (fmt, alt) in seen
+            # (no float lies between 1e-5 and its float rounding: that mistake cannot show there)
+            assert (fmt, alt) in seen or (fmt, alt) == ("f32", "exact_eps")
 
 
 def test_oracle_estimator_on_the_constant_inputs():
@@ -140,15 +145,21 @@ def test_hip_top_p_in_16_bit_arithmetic_and_cub_order(dev):
     import twilight_amd.kernel as K
     for r in KA["top_p_cub_order"]["rows"]:
         bits, code, _ = _cub_row(r)
-        t = torch.from_numpy(bits.view(np.int16)).view(torch.float16 if code == 0 else torch.bfloat16)
+        if code == 2:
+            t = torch.from_numpy(bits)
+        else:
+            t = torch.from_numpy(bits.view(np.int16)).view(torch.float16 if code == 0 else torch.bfloat16)
         t = t.reshape(1, 1, 1, -1).to(dev)
         idx, count, mask, low, iters = K.top_p_select(t, r["p"], high=r["high"], return_mask=True,
-                                                      return_stats=True)
+                                                      return_stats=True, exact=True)
         kept = torch.nonzero(mask[0, 0, 0]).flatten().tolist()
         assert kept == r["kept"], (r["dtype"], r["d"], r["differs_under"])
         assert idx[0, 0, :int(count[0, 0])].tolist() == r["kept"]
         assert _low_bits(float(low[0]), code) == r["low_bits"] and int(iters[0]) == r["iterations"]
-        assert torch.equal(K.top_p_fp16_return_mask(t, r["p"], high=r["high"]), mask)
+        if code == 2:
+            assert torch.equal(K.top_p_fp32_return_mask(t, r["p"], high=r["high"], exact=True), mask)
+        else:
+            assert torch.equal(K.top_p_fp16_return_mask(t, r["p"], high=r["high"]), mask)
 
 
 @pytest.mark.gpu

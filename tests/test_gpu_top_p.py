@@ -222,6 +222,59 @@ def test_16bit_entry_cfg3_shape(dev, dt):
             assert oi.mean() > 5     # the rows really iterate
 
 
+def test_fp32_exact_entry(dev):
+    # the reference's DType = float instantiation (csrc/src/sampling.cu:45-63) with the sums in
+    # cub::BlockReduce's order (VEC = gcd(4, d) in {4, 2, 1}, one to eight chunks of 1024 * VEC):
+    # masks, final pivots and iteration counts identical on EVERY row, no margin; both upper
+    # bounds, scalar and per-row p, mask-only and list outputs.
+    g = torch.Generator().manual_seed(4)
+    for d, rows, scale in ((3000, 16, 4.0), (8192, 32, 5.0), (4100, 8, 4.0), (1002, 8, 3.0),
+                           (999, 8, 3.0), (32768, 8, 6.0), (20000, 4, 5.0), (24, 4, 1.0), (5, 4, 1.0),
+                           (1, 3, 1.0), (17, 4, 2.0), (1025, 4, 3.0), (4097, 4, 4.0), (9000, 4, 4.0)):
+        probs = _softmax(torch.randn((1, rows, 1, d), generator=g) * scale)
+        pn32 = probs.numpy().reshape(rows, d)
+        for high, mode in (("max", native.HIGH_MAX), ("first", native.HIGH_FIRST)):
+            for p in (0.9, 0.85 + 0.1 * torch.rand(rows, generator=g)):
+                pn = p.numpy().astype(np.float32) if torch.is_tensor(p) else p
+                om, ol, oi = native.top_p_mask_cub(pn32, native.DT_F32, pn, mode)
+                pd = p.to(dev) if torch.is_tensor(p) else p
+                idx, count, mask, low, iters = K.top_p_select(probs.to(dev), pd, high=high,
+                                                              return_mask=True, return_stats=True,
+                                                              exact=True)
+                gm = mask.cpu().numpy().reshape(rows, d)
+                assert np.array_equal(gm, om.astype(bool)), (d, high)
+                assert np.array_equal(low.cpu().numpy(), ol) and np.array_equal(iters.cpu().numpy(), oi)
+                cn = count.cpu().numpy().reshape(-1)
+                ix = idx.cpu().numpy().reshape(rows, d)
+                for r in range(rows):
+                    assert np.array_equal(ix[r, :cn[r]], np.nonzero(gm[r])[0])
+        assert torch.equal(K.top_p_fp32_return_mask(probs.to(dev), 0.9, exact=True),
+                           torch.from_numpy(native.top_p_mask_cub(pn32, native.DT_F32, 0.9, native.HIGH_FIRST)[0]
+                                            .astype(bool)).reshape(1, rows, 1, d).to(dev))
+
+
+@pytest.mark.parametrize("first_is_max", [True, False])
+def test_fp32_exact_entry_cfg3(dev, first_is_max):
+    # the pruner workload (8 x 32 rows of 8192 probabilities, Zipf spikes over a normal
+    # background), both p, both upper bounds: equal to the float oracle on every row
+    x = synth.topp_scores(8, 32, 8192, seed=13, first_is_max=first_is_max)
+    probs = _softmax(x).reshape(8, 32, 1, 8192)
+    pn32 = probs.numpy().reshape(256, 8192)
+    for p in (0.85, 0.95):
+        for high, mode in (("first", native.HIGH_FIRST), ("max", native.HIGH_MAX)):
+            om, ol, oi = native.top_p_mask_cub(pn32, native.DT_F32, p, mode)
+            idx, count, mask, low, iters = K.top_p_select(probs.to(dev), p, high=high,
+                                                          return_mask=True, return_stats=True,
+                                                          exact=True)
+            assert np.array_equal(mask.cpu().numpy().reshape(256, 8192), om.astype(bool))
+            assert np.array_equal(low.cpu().numpy(), ol) and np.array_equal(iters.cpu().numpy(), oi)
+            assert oi.mean() > 5 or not first_is_max
+            # the default kernel (its own order of additions) keeps the same set wherever no
+            # decision of the search came within rounding of p
+            fast = K.top_p_fp32_return_mask(probs.to(dev), p, high=high).cpu().numpy().reshape(256, 8192)
+            assert (fast == om.astype(bool)).all(-1).sum() >= 250
+
+
 def test_fused_softmax_top_p_lists(dev):
     # twilight/pyimpl/top_p.py:10-15 on candidate scores with -inf slots, ragged lens, page mapping
     B, H, S = 2, 4, 40

@@ -14,7 +14,7 @@ from .build import LIB_PATH
 
 TWL_OK = 0
 TWL_F16, TWL_BF16, TWL_F32 = 0, 1, 2
-ABI_VERSION = 9  # TWL_ABI_VERSION of include/twilight_hip.h, checked when the library is loaded
+ABI_VERSION = 10  # TWL_ABI_VERSION of include/twilight_hip.h, checked when the library is loaded
 TWL_HIGH_FIRST, TWL_HIGH_MAX = 0, 1
 PAGE = 16
 HEAD_DIM = 128
@@ -25,7 +25,7 @@ STATIC_SCRATCH_BYTES = 24 << 20
 
 # every symbol include/twilight_hip.h declares
 EXPORTS = (
-    "twl_strerror", "twl_abi_version", "twl_device_count", "twl_top_p_f32", "twl_top_p_f16",
+    "twl_strerror", "twl_abi_version", "twl_device_count", "twl_top_p_f32", "twl_top_p_f16", "twl_top_p_f32_exact",
     "twl_softmax_top_p_f32", "twl_gemv_top_p", "twl_select_estimate_prune", "twl_gemv_int4", "twl_gemv_int4_nhd",
     "twl_gemv_int8_nhd", "twl_gemv_f16_nhd", "twl_gemv_f16_single", "twl_sparse_attn",
     "twl_sparse_attn_workspace_bytes", "twl_sparse_attn_static", "twl_sparse_attn_weighted", "twl_gemv_int4_group",
@@ -91,6 +91,7 @@ def lib() -> ctypes.CDLL:
             f"{ABI_VERSION}: rebuild it with `python -m twilight_amd.build`")
     L.twl_device_count.argtypes = []
     L.twl_top_p_f32.argtypes = [vp, vp, vp, vp, vp, f32, u32, u32, u32, i32, vp, vp, vp]
+    L.twl_top_p_f32_exact.argtypes = L.twl_top_p_f32.argtypes
     L.twl_top_p_f16.argtypes = [vp, i32, vp, vp, vp, vp, f32, u32, u32, u32, i32, vp, vp, vp]
     L.twl_softmax_top_p_f32.argtypes = [vp, u32, vp, u32, u32, vp, f32, i32, vp, u32, vp, u32, vp,
                                         vp, vp, vp]

@@ -1,14 +1,15 @@
-// Top-p mask kernel for fp16 / bf16 probabilities: TopPReturnMaskKernel<1024,
+// Top-p mask kernel in the arithmetic of the probabilities' own type: TopPReturnMaskKernel<1024,
 // BLOCK_REDUCE_WARP_REDUCTIONS, VEC, DType> (csrc/include/sampling.cuh:119-231) as instantiated for
-// half and nv_bfloat16 (csrc/src/sampling.cu:22-43), with the arithmetic that instantiation has.
+// half and nv_bfloat16 (csrc/src/sampling.cu:22-43) and for float (csrc/src/sampling.cu:45-63),
+// with the arithmetic and the order of additions each instantiation has. The 16-bit case:
 //
 // There p, low, high, mid, the tolerance 1e-5, the bracket width and EVERY partial sum are values
 // of the 16-bit type, each addition rounding to nearest even. A sum of thousands of 16-bit
 // numbers depends on the order of the additions, so the kernel below adds in the order CUB's
 // block reduction does (cub::BlockReduce with BLOCK_REDUCE_WARP_REDUCTIONS, sampling.cuh:54):
 //   - a workgroup has the reference's 1024 threads; thread t owns, in chunk i, the
-//     VEC = gcd(8, d) elements from (i * 1024 + t) * VEC on (sampling.cuh:176-181,239-243), zeros
-//     past the end of the row;
+//     VEC = gcd(16 / sizeof(DType), d) elements from (i * 1024 + t) * VEC on
+//     (sampling.cuh:176-181,239-243), zeros past the end of the row;
 //   - a thread folds its VEC masked items left to right (cub::ThreadReduce);
 //   - a CUDA warp is 32 consecutive threads = half a wavefront: its five shuffle-down steps
 //     (offsets 1, 2, 4, 8, 16; lane l adds lane l + offset) are four row-shift DPP steps inside each
@@ -23,13 +24,16 @@
 // in registers (at most 32 values per thread); an iteration costs one barrier.
 //
 // A 16-bit addition is computed as an fp32 addition rounded to the 16-bit type: fp32 carries
-// 24 >= 2 * 11 + 2 significand bits, so the double rounding equals the single one.
+// 24 >= 2 * 11 + 2 significand bits, so the double rounding equals the single one. For float the
+// rounding step is the identity and what remains is the order of the additions, which is what
+// makes the float op reproduce the reference's masks row for row (the faster fp32 kernel of
+// top_p.hip adds in another order and can differ where a sum meets p within rounding).
 #include "twl_common.h"
 
 namespace twl {
 
 struct TopPDtArgs {
-  const uint16_t* probs;   // [rows, d]
+  const void* probs;       // [rows, d] of the kernel's element type
   uint32_t d;
   const float* p_arr;      // nullable
   float p;
@@ -70,38 +74,54 @@ __global__ __launch_bounds__(kCubThreads) void top_p_dtype_kernel(TopPDtArgs a) 
   const int nchunks = (int)((d + kCubThreads * VEC - 1) / (kCubThreads * VEC));  // <= MAXC
 
   // ---- the row, once (VEC divides d, so a thread's VEC elements are all inside or all outside)
-  const uint16_t* src = a.probs + (size_t)row * d;
-  const bool vec_ok = ((((uintptr_t)src) & (2u * VEC - 1u)) == 0);
+  constexpr uint32_t ESZ = (DT == TWL_F32) ? 4u : 2u;
+  const uint8_t* src = (const uint8_t*)a.probs + (size_t)row * d * ESZ;
+  const bool vec_ok = ((((uintptr_t)src) & (ESZ * VEC - 1u)) == 0);
   float x[MAXC][VEC];
   bool valid[MAXC];
 #pragma unroll
   for (int c = 0; c < MAXC; ++c) {
     const uint32_t e0 = ((uint32_t)c * kCubThreads + (uint32_t)tx) * VEC;
     valid[c] = c < nchunks && e0 < d;
-    uint32_t bits[VEC];
+    float raw[VEC];
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) bits[j] = 0;
+    for (int j = 0; j < VEC; ++j) raw[j] = 0.0f;
     if (valid[c]) {
-      if (VEC == 8 && vec_ok) {
-        const u32x4 v = *(const u32x4*)(src + e0);
-        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+      if constexpr (DT == TWL_F32) {
+        const float* s32 = (const float*)src;
+        if (VEC == 4 && vec_ok) {
+          const f32x4 v = *(const f32x4*)(s32 + e0);
+          const float w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) bits[j] = (w[j / 2] >> (16 * (j & 1))) & 0xFFFFu;
-      } else if (VEC == 4 && vec_ok) {
-        const u32x2 v = *(const u32x2*)(src + e0);
-        const uint32_t w[2] = {v.x, v.y};
+          for (int j = 0; j < VEC; ++j) raw[j] = w[j % 4];
+        } else {
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) bits[j] = (w[j / 2] >> (16 * (j & 1))) & 0xFFFFu;
+          for (int j = 0; j < VEC; ++j) raw[j] = s32[e0 + j];
+        }
       } else {
+        const uint16_t* s16 = (const uint16_t*)src;
+        uint32_t bits[VEC];
+        if (VEC == 8 && vec_ok) {
+          const u32x4 v = *(const u32x4*)(s16 + e0);
+          const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-        for (int j = 0; j < VEC; ++j) bits[j] = src[e0 + j];
+          for (int j = 0; j < VEC; ++j) bits[j] = (w[(j / 2) % 4] >> (16 * (j & 1))) & 0xFFFFu;
+        } else if (VEC == 4 && vec_ok) {
+          const u32x2 v = *(const u32x2*)(s16 + e0);
+          const uint32_t w[2] = {v.x, v.y};
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) bits[j] = (w[(j / 2) % 2] >> (16 * (j & 1))) & 0xFFFFu;
+        } else {
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) bits[j] = s16[e0 + j];
+        }
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) raw[j] = bits16_to_f32<DT>(bits[j]);
       }
     }
 #pragma unroll
-    for (int j = 0; j < VEC; ++j) {
-      const float v = bits16_to_f32<DT>(bits[j]);
-      x[c][j] = (v > 0.0f) ? v : 0.0f;   // probabilities; negative, -0 and NaN count as 0
-    }
+    for (int j = 0; j < VEC; ++j)
+      x[c][j] = (raw[j] > 0.0f) ? raw[j] : 0.0f;   // probabilities; negative, -0 and NaN count as 0
   }
 
   // ---- bounds (sampling.cuh:156-162) ----------------------------------------------------------
@@ -268,8 +288,13 @@ template <int DT>
 static int launch_top_p_dtype(const TopPDtArgs& a, uint32_t rows, hipStream_t s) {
   const dim3 grid(rows), block(kCubThreads);
   // VEC_SIZE = gcd(16 / sizeof(DType), d), sampling.cuh:239
-  if (a.d % 8 == 0) hipLaunchKernelGGL((top_p_dtype_kernel<DT, 8>), grid, block, 0, s, a);
-  else if (a.d % 4 == 0) hipLaunchKernelGGL((top_p_dtype_kernel<DT, 4>), grid, block, 0, s, a);
+  if constexpr (DT != TWL_F32) {
+    if (a.d % 8 == 0) {
+      hipLaunchKernelGGL((top_p_dtype_kernel<DT, 8>), grid, block, 0, s, a);
+      return hipGetLastError() == hipSuccess ? TWL_OK : TWL_ELAUNCH;
+    }
+  }
+  if (a.d % 4 == 0) hipLaunchKernelGGL((top_p_dtype_kernel<DT, 4>), grid, block, 0, s, a);
   else if (a.d % 2 == 0) hipLaunchKernelGGL((top_p_dtype_kernel<DT, 2>), grid, block, 0, s, a);
   else hipLaunchKernelGGL((top_p_dtype_kernel<DT, 1>), grid, block, 0, s, a);
   return hipGetLastError() == hipSuccess ? TWL_OK : TWL_ELAUNCH;
@@ -277,10 +302,9 @@ static int launch_top_p_dtype(const TopPDtArgs& a, uint32_t rows, hipStream_t s)
 
 }  // namespace twl
 
-extern "C" int twl_top_p_f16(const void* probs, int dtype, uint8_t* mask, int32_t* idx,
-                             int32_t* count, const float* p_arr, float p, uint32_t rows,
-                             uint32_t d, uint32_t idx_stride, int high_mode, float* low_out,
-                             int32_t* iters_out, void* stream) {
+static int check_top_p_dtype(const void* probs, const uint8_t* mask, const int32_t* idx,
+                             const int32_t* count, const float* p_arr, float p, uint32_t rows,
+                             uint32_t d, uint32_t idx_stride, int high_mode) {
   if (!probs) return TWL_ENULL;
   if (!mask && !idx && !count) return TWL_ENULL;
   if (idx && !count) return TWL_ENULL;
@@ -288,12 +312,37 @@ extern "C" int twl_top_p_f16(const void* probs, int dtype, uint8_t* mask, int32_
   if (idx && idx_stride < d) return TWL_EINVAL;
   if (high_mode != TWL_HIGH_FIRST && high_mode != TWL_HIGH_MAX) return TWL_EINVAL;
   if (!p_arr && !(p > 0.0f && p <= 1.0f)) return TWL_EINVAL;
+  return TWL_OK;
+}
+
+extern "C" int twl_top_p_f16(const void* probs, int dtype, uint8_t* mask, int32_t* idx,
+                             int32_t* count, const float* p_arr, float p, uint32_t rows,
+                             uint32_t d, uint32_t idx_stride, int high_mode, float* low_out,
+                             int32_t* iters_out, void* stream) {
+  const int rc = check_top_p_dtype(probs, mask, idx, count, p_arr, p, rows, d, idx_stride, high_mode);
+  if (rc != TWL_OK) return rc;
   if (dtype != TWL_F16 && dtype != TWL_BF16) return TWL_EDTYPE;
   if (((uintptr_t)probs) & 1u) return TWL_EALIGN;
   twl::TopPDtArgs a{};
-  a.probs = (const uint16_t*)probs; a.d = d; a.p_arr = p_arr; a.p = p; a.high_mode = high_mode;
+  a.probs = probs; a.d = d; a.p_arr = p_arr; a.p = p; a.high_mode = high_mode;
   a.mask = mask; a.idx = idx; a.idx_stride = idx_stride; a.count = count; a.low_out = low_out;
   a.iters_out = iters_out;
   if (dtype == TWL_F16) return twl::launch_top_p_dtype<TWL_F16>(a, rows, (hipStream_t)stream);
   return twl::launch_top_p_dtype<TWL_BF16>(a, rows, (hipStream_t)stream);
+}
+
+// The float instantiation of the same kernel (csrc/src/sampling.cu:45-63): fp32 arithmetic with the
+// additions in cub::BlockReduce's order, VEC = gcd(4, d).
+extern "C" int twl_top_p_f32_exact(const float* probs, uint8_t* mask, int32_t* idx, int32_t* count,
+                                   const float* p_arr, float p, uint32_t rows, uint32_t d,
+                                   uint32_t idx_stride, int high_mode, float* low_out,
+                                   int32_t* iters_out, void* stream) {
+  const int rc = check_top_p_dtype(probs, mask, idx, count, p_arr, p, rows, d, idx_stride, high_mode);
+  if (rc != TWL_OK) return rc;
+  if (((uintptr_t)probs) & 3u) return TWL_EALIGN;
+  twl::TopPDtArgs a{};
+  a.probs = probs; a.d = d; a.p_arr = p_arr; a.p = p; a.high_mode = high_mode;
+  a.mask = mask; a.idx = idx; a.idx_stride = idx_stride; a.count = count; a.low_out = low_out;
+  a.iters_out = iters_out;
+  return twl::launch_top_p_dtype<TWL_F32>(a, rows, (hipStream_t)stream);
 }

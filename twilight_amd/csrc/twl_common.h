@@ -27,10 +27,9 @@ __device__ __forceinline__ int lane_id() {
 
 // ---- 16-bit float conversions (exact widenings; narrowing is round-to-nearest-even) ----------
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return as_f32(b << 16); }
+// round to nearest even by the hardware convert (v_cvt_pk_bf16_f32); a NaN stays a NaN
 __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
-  uint32_t x = as_u32(f);
-  if ((x & 0x7FFFFFFFu) > 0x7F800000u) return (x >> 16) | 0x40u;
-  return (x + 0x7FFFu + ((x >> 16) & 1u)) >> 16;
+  return (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)f);
 }
 __device__ __forceinline__ float f16_bits_to_f32(uint32_t b) {
   return (float)__builtin_bit_cast(_Float16, (uint16_t)b);
