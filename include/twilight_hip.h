@@ -222,8 +222,11 @@ int twl_gemv_int4(const void* q, int q_dtype, float* out, uint32_t out_stride, i
 /* twl_gemv_int4 for q heads that share kv heads AND one page list per kv head: the list of a
  * group's first q head (sel_pages / sel_count row b * num_q_heads + kvh * G, required) serves the
  * G = num_q_heads / num_kv_heads heads of the group (G in {2, 4, 8}), every INT4 record is
- * fetched once per group and out / out_count are written for every q head. A head's scores are
- * bit-identical to twl_gemv_int4 over the same list.
+ * fetched once per group and out / out_count are written for every q head. The group's
+ * products run on the matrix cores (v_mfma_f32_16x16x32_f16 on the exact fp16 values of the
+ * nibbles, fp32 accumulation): a head's scores equal twl_gemv_int4's over the same list up to
+ * the fp32 rounding of sums taken in another order (within 2e-5 of the row's typical score in
+ * the tests), not bit for bit.
  * Replaces: the same estimator matmul (attention.py:252-255) when the candidate set is chosen per
  * kv head (the reference repeats K per q head, attention.py:124-126, and selects per q head; see
  * twl_layer_args.group_select). */
@@ -586,7 +589,8 @@ typedef struct twl_layer_args {
    * twl_softmax_top_p_f32), and every q head still prunes and attends on its own scores. Not the
    * reference's per-q-head selection (attention.py:124-126 repeats K per q head): an option, as
    * group_idx is. sel_pages / sel_count hold the group's list in each of its q-head rows;
-   * `scores` and `page_scores` (required) are always written. */
+   * `scores`, `cand_count` and `page_scores` (all required: TWL_ENULL before anything is
+   * launched) are always written. */
   int group_select;
 } twl_layer_args;
 

@@ -54,8 +54,20 @@ extern "C" int twl_decode_layer(const twl_layer_args* a, void* stream) {
 
   int rc;
   if (a->group_select && a->num_q_heads != a->num_kv_heads) {
-    // one candidate list per kv head: scores (group maximum) -> top-k -> group GEMV -> pruner
-    if (!a->page_scores || !a->meta || !a->k_int4) return TWL_ENULL;
+    // one candidate list per kv head: scores (group maximum) -> top-k -> group GEMV -> pruner.
+    // Everything the four launches need is checked before the first one: the score matrix and
+    // the candidate counts travel through memory between them (requests shorter than the budget
+    // leave score slots unwritten, which only cand_count tells the pruner).
+    if (!a->page_scores || !a->meta || !a->k_int4 || !a->scores || !a->cand_count ||
+        !a->sel_pages || !a->sel_count || !a->q || !a->kv_page_indices || !a->kv_page_indptr ||
+        !a->kv_last_page_len)
+      return TWL_ENULL;
+    {
+      const uint32_t g = a->num_kv_heads ? a->num_q_heads / a->num_kv_heads : 0;
+      if (a->num_kv_heads == 0 || a->num_q_heads % a->num_kv_heads != 0 ||
+          (g != 2 && g != 4 && g != 8))
+        return TWL_EINVAL;
+    }
     rc = twl::quest_page_scores_ex(a->q, a->dtype, a->meta, a->kv_page_indices,
                                    a->kv_page_indptr, a->batch, a->num_q_heads, a->num_kv_heads,
                                    a->max_pages_per_req, a->page_scores, a->page_score_stride, 1,

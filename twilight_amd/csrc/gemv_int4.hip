@@ -199,21 +199,38 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_int4_kernel(GemvArgs a) {
 }
 
 // The q heads of a kv head over ONE page list (that of the group's first q head): every INT4
-// record is fetched once and multiplied with the GROUP queries. The unpacked nibbles are shared;
-// per head the dot products, the scale / zero step and the quad reduction are those of
-// gemv_int4_kernel in the same order, so a head's scores equal what that kernel gives it over the
-// same list bit for bit.
-template <int QDT, int GROUP, int PW>
+// record is fetched once and meets the group's queries on the matrix cores. Per page and per
+// quantisation group the estimator is a [heads x 32] x [32 x 16 tokens] product; four of them
+// (the page's four quantisation groups) share one v_mfma_f32_16x16x32_f16 by giving each
+// (head, group) pair a ROW of the A operand that is zero outside its own group:
+//   A (16 x 32)  row 4*h + c', k-block c (lanes 16c..16c+15): q[h, 32c + 8j .. +8] if c == c', else 0
+//   B (32 x 16)  column t (token), k-block c: the 8 nibbles of dword j of group c, as the exact
+//                fp16 values 1 + n/64 (one shift and one v_and_or per two nibbles)
+//   C (16 x 16)  lane (r, t) holds rows 4r .. 4r+3 = (head r, groups 0..3) of token t
+// accumulated over the group's four dwords j. A lane (r, t) therefore ends with the four per-group
+// dot products of ONE (head, token) pair: scale and zero (four fp16 pairs = one 16-byte load per
+// token) are applied and summed inside the lane, no cross-lane step at all:
+//     score = sm_scale * sum_c' ( 64 scale[t,c'] (C[c'] - qsum[h,c']) + zero[t,c'] qsum[h,c'] )
+// About 55 vector instructions and 4 matrix instructions per page for up to four heads (the
+// per-head arithmetic on the vector unit took about 130), eight heads take two A operands. The
+// products are exact and accumulate in fp32 as before, in the matrix unit's order: scores agree
+// with twl_gemv_int4 within fp32 rounding of the sums, not bit for bit.
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+
+template <int QDT, int GROUP, int PW, int U>
 __global__ __launch_bounds__(kGemvThreads) void gemv_int4_group_kernel(GemvArgs a) {
-  constexpr int U = kGemvUnroll;
   constexpr int G = PW / U;
+  constexpr int SETS = (GROUP + 3) / 4;          // A operands of four heads each
+  constexpr int NW = kGemvThreads / kWave;
   static_assert(PW % U == 0 && PW <= 64, "one lane per page id, whole groups");
+  __shared__ float qs_lds[NW][SETS][4][4];                // [wave][set][head of set][group]
+  __shared__ __align__(16) float sc_lds[NW][4 * SETS][PW * TWL_PAGE];
   const uint32_t b = blockIdx.y / a.num_kv_heads;
   const uint32_t kvh = blockIdx.y - b * a.num_kv_heads;
   const uint32_t row0 = b * a.num_q_heads + kvh * GROUP;  // the group's first q-head row
   const int lane = lane_id();
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-  const int p0 = (blockIdx.x * (kGemvThreads / kWave) + wave) * PW;
+  const int p0 = (blockIdx.x * NW + wave) * PW;
 
   const int pg_begin = a.kv_page_indptr[b];
   const int pg_end = a.kv_page_indptr[b + 1];
@@ -221,56 +238,68 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_int4_group_kernel(GemvArgs 
   const int sel_n = a.sel_count ? a.sel_count[row0] : (int)a.sel_stride;
   int my_logical = (lane < PW && (uint32_t)(p0 + lane) < a.sel_stride)
                        ? a.sel_pages[(size_t)row0 * a.sel_stride + p0 + lane] : 0;
-  const int g4 = lane & 3;
-  const int t = lane >> 2;
   const int req_pages = pg_end - pg_begin;
   int n_pages = min(max(sel_n, 0), (int)a.max_pages);
   if (req_pages <= 0) n_pages = 0;
   if (blockIdx.x == 0 && threadIdx.x < GROUP && a.out_count)
     a.out_count[row0 + threadIdx.x] = n_pages * TWL_PAGE;
-  if (p0 >= n_pages) return;
-  const int np = min(PW, n_pages - p0);
-  my_logical = min(max(my_logical, 0), req_pages - 1);
+  const int np = max(0, min(PW, n_pages - p0));            // 0: this wavefront only keeps the barriers
+  my_logical = min(max(my_logical, 0), max(req_pages - 1, 0));
   int my_phys = 0;
   if (lane < np) my_phys = a.kv_page_indices[pg_begin + my_logical];
 
-  half2_t qp[GROUP][16];
-  float qsum[GROUP];
+  const int c = lane >> 4;          // k-block of both operands; as a C lane: head of the set
+  const int t = lane & 15;          // B column / C column: token of the page
+  const int hl = t >> 2, cq = t & 3;  // as an A lane: head of the set, quantisation group of the row
+
+  // ---- A operands: lane = (k-block c, row 4*hl + c') ------------------------------------------
+  half8_t aop[SETS][4];
 #pragma unroll
-  for (int h = 0; h < GROUP; ++h) {
-    const uint16_t* qrow = (const uint16_t*)a.q + (size_t)(row0 + h) * TWL_HEAD_DIM + 32 * g4;
-    float qf[32];
+  for (int st = 0; st < SETS; ++st) {
+    const int h = 4 * st + hl;
+    const bool live = (c == cq) && h < GROUP;
+    float qsum = 0.0f;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const u32x4 v = *(const u32x4*)(qrow + 8 * i);
-      const uint32_t ws[4] = {v.x, v.y, v.z, v.w};
+    for (int j = 0; j < 4; ++j) {
+      u32x4 v = {0u, 0u, 0u, 0u};
+      if (live)
+        v = *(const u32x4*)((const uint16_t*)a.q + (size_t)(row0 + h) * TWL_HEAD_DIM + 32 * c + 8 * j);
+      float qf[8];
+      unpack8<QDT>(v, qf);
+      _Float16 qh[8];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        qf[8 * i + 2 * j] = bits16_to_f32<QDT>(ws[j] & 0xFFFFu);
-        qf[8 * i + 2 * j + 1] = bits16_to_f32<QDT>(ws[j] >> 16);
+      for (int i = 0; i < 8; ++i) {
+        qh[i] = q_to_half(qf[i]);
+        qsum += (float)qh[i];
       }
+      // element order of the unpacked nibbles: n0 n4 n1 n5 n2 n6 n3 n7
+      aop[st][j] = half8_t{qh[0], qh[4], qh[1], qh[5], qh[2], qh[6], qh[3], qh[7]};
     }
-#pragma unroll
-    for (int w = 0; w < 4; ++w)
-#pragma unroll
-      for (int s2 = 0; s2 < 4; ++s2) {
-        half2_t pr = {q_to_half(qf[8 * w + s2]), q_to_half(qf[8 * w + s2 + 4])};
-        qp[h][4 * w + s2] = pr;
-      }
-    float qs = 0.0f;
-#pragma unroll
-    for (int i = 0; i < 32; ++i) qs += (float)q_to_half(qf[i]);
-    qsum[h] = qs;
+    if (live) qs_lds[wave][st][hl][cq] = qsum;
+    else if (c == cq) qs_lds[wave][st][hl][cq] = 0.0f;
   }
+  __syncthreads();
+  float qs[SETS][4];                // as a C lane (head c of the set): sum of q over each group
+#pragma unroll
+  for (int st = 0; st < SETS; ++st)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) qs[st][i] = qs_lds[wave][st][c][i];
 
   const size_t rec_stride = (size_t)a.num_kv_heads * TWL_INT4_RECORD_BYTES;
-  const uint8_t* base = a.k_int4 + (size_t)kvh * TWL_INT4_RECORD_BYTES + 16 * lane;
+  // B lane (k-block c, token t): the 16 bytes of token t's quantisation group c; C lane (head c,
+  // token t): the token's four (scale, zero) pairs
+  const uint8_t* base = a.k_int4 + (size_t)kvh * TWL_INT4_RECORD_BYTES;
+  const uint32_t nib_off = 64u * (uint32_t)t + 16u * (uint32_t)c;
+  const uint32_t sz_off = 1024u + 16u * (uint32_t)t;
   const float ninf = -__builtin_inff();
-  const int src_lane4 = 4 * (4 * (lane & 15) + (lane >> 4));
-  const uint32_t m = 0x00F000F0u, one = 0x3C003C00u;
-  u32x4 nib[U];
-  uint32_t sz[U];
-  float held[GROUP][G];
+  // the mask in a scalar register and the exponent pattern in a vector register, both opaque to
+  // the compiler, so that (x & m) | one is one v_and_or_b32 (it cannot carry two literals)
+  uint32_t m = 0x00F000F0u, one = 0x3C003C00u;
+  asm volatile("" : "+s"(m));
+  asm volatile("" : "+v"(one));
+  // (Requesting the first pages before the queries are converted was measured: 12.9 against
+  // 12.1 us; the wavefronts of a compute unit are not in step, so the phases overlap anyway.)
+  u32x4 nib[U], sz[U];
 #pragma unroll
   for (int grp = 0; grp < G; ++grp) {
     if (grp * U < np) {
@@ -279,50 +308,67 @@ __global__ __launch_bounds__(kGemvThreads) void gemv_int4_group_kernel(GemvArgs 
         const int i = grp * U + u;
         const int phys = __builtin_amdgcn_readlane(my_phys, (i < np) ? i : 0);
         const uint8_t* rec = base + (size_t)phys * rec_stride;
-        nib[u] = __builtin_nontemporal_load((const u32x4*)rec);
-        sz[u] = __builtin_nontemporal_load((const uint32_t*)(rec + 1024 - 12 * lane));
+        nib[u] = __builtin_nontemporal_load((const u32x4*)(rec + nib_off));
+        sz[u] = __builtin_nontemporal_load((const u32x4*)(rec + sz_off));
       }
-      float mine[GROUP];
-#pragma unroll
-      for (int h = 0; h < GROUP; ++h) mine[h] = 0.0f;
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const int i = grp * U + u;
-        // the page's 32 nibbles of this lane as 16 fp16 pairs, once for all heads
-        half2_t nb[16];
         const uint32_t ws[4] = {nib[u].x, nib[u].y, nib[u].z, nib[u].w};
+        const uint32_t sw[4] = {sz[u].x, sz[u].y, sz[u].z, sz[u].w};
+        half8_t bop[4];
 #pragma unroll
-        for (int w = 0; w < 4; ++w) {
-          nb[4 * w + 0] = __builtin_bit_cast(half2_t, and_or(ws[w] << 4, m, one));
-          nb[4 * w + 1] = __builtin_bit_cast(half2_t, and_or(ws[w], m, one));
-          nb[4 * w + 2] = __builtin_bit_cast(half2_t, and_or(ws[w] >> 4, m, one));
-          nb[4 * w + 3] = __builtin_bit_cast(half2_t, and_or(ws[w] >> 8, m, one));
+        for (int j = 0; j < 4; ++j) {
+          // plain C here, not the and_or() helper: the matrix instruction that reads these
+          // registers needs wait states after a vector write, which the compiler inserts for
+          // instructions it knows and cannot for the text of an asm statement
+          const u32x4 e = {((ws[j] << 4) & m) | one, (ws[j] & m) | one,
+                           ((ws[j] >> 4) & m) | one, ((ws[j] >> 8) & m) | one};
+          bop[j] = __builtin_bit_cast(half8_t, e);
         }
-        const float scale64 = f16_bits_to_f32(sz[u] & 0xFFFFu) * 64.0f;
-        const float zero = f16_bits_to_f32(sz[u] >> 16);
         const int logical = __builtin_amdgcn_readlane(my_logical, (i < np) ? i : 0);
         const int valid = (logical == req_pages - 1) ? last_len : TWL_PAGE;
 #pragma unroll
-        for (int h = 0; h < GROUP; ++h) {
-          float acc = 0.0f;
+        for (int st = 0; st < SETS; ++st) {
+          f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-          for (int j = 0; j < 16; ++j) acc = __builtin_amdgcn_fdot2(nb[j], qp[h][j], acc, false);
-          const float part = quad_allreduce<OpSum>(fmaf(scale64, acc - qsum[h], zero * qsum[h]));
-          const float val = (t < valid) ? part * a.sm_scale : ninf;
-          mine[h] = (g4 == u) ? val : mine[h];
+          for (int j = 0; j < 4; ++j)
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(aop[st][j], bop[j], acc, 0, 0, 0);
+          const float cv[4] = {acc.x, acc.y, acc.z, acc.w};
+          float v = 0.0f;
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const float scale64 = f16_bits_to_f32(sw[g] & 0xFFFFu) * 64.0f;
+            const float zero = f16_bits_to_f32(sw[g] >> 16);
+            v = fmaf(scale64, cv[g] - qs[st][g], v);
+            v = fmaf(zero, qs[st][g], v);
+          }
+          sc_lds[wave][4 * st + c][i * TWL_PAGE + t] = (t < valid) ? v * a.sm_scale : ninf;
         }
       }
-#pragma unroll
-      for (int h = 0; h < GROUP; ++h)
-        held[h][grp] = as_f32(__builtin_amdgcn_ds_bpermute(src_lane4, as_i32(mine[h])));
     }
   }
+  __syncthreads();
+  // a head's PW pages x 16 scores leave as one run: a lane stores 16 bytes, a wavefront 1 KiB
+  if (np > 0) {
 #pragma unroll
-  for (int h = 0; h < GROUP; ++h) {
-    float* orow = a.out + (size_t)(row0 + h) * a.out_stride + (size_t)p0 * TWL_PAGE;
+    for (int h = 0; h < GROUP; ++h) {
+      float* orow = a.out + (size_t)(row0 + h) * a.out_stride + (size_t)p0 * TWL_PAGE;
+      const bool wide = (((uintptr_t)orow) & 15u) == 0;
 #pragma unroll
-    for (int grp = 0; grp < G; ++grp)
-      if (grp * U + (lane >> 4) < np) orow[grp * U * TWL_PAGE + lane] = held[h][grp];
+      for (int e = 0; e < (4 * PW + kWave - 1) / kWave; ++e) {
+        const int f4 = e * kWave + lane;               // which group of four scores
+        if (f4 < 4 * PW && (f4 >> 2) < np) {
+          const f32x4 v = *(const f32x4*)&sc_lds[wave][h][4 * f4];
+          if (wide) {
+            *(f32x4*)(orow + 4 * f4) = v;
+          } else {
+            orow[4 * f4] = v.x; orow[4 * f4 + 1] = v.y; orow[4 * f4 + 2] = v.z;
+            orow[4 * f4 + 3] = v.w;
+          }
+        }
+      }
+    }
   }
 }
 
@@ -548,21 +594,22 @@ extern "C" int twl_gemv_int4_group(const void* q, int q_dtype, float* out, uint3
   a.kv_last_page_len = kv_last_page_len; a.num_q_heads = num_q_heads;
   a.num_kv_heads = num_kv_heads; a.max_pages = max_pages_per_row; a.sm_scale = sm_scale;
   hipStream_t st = (hipStream_t)stream;
-  // 16 pages per wavefront (measured at 8 x 8 kv heads x 512 pages: 8 pages 19.4 us, 16 pages
-  // 18.3, 32 pages 20.0): a kv head's list is short (the budget) and, besides batch x kv heads,
-  // the only source of parallelism, while every wavefront first converts the group's queries
-  constexpr int PW = 16;
-  const uint32_t per_block = PW * (twl::kGemvThreads / twl::kWave);
-  const dim3 grid((max_pages_per_row + per_block - 1) / per_block, batch * num_kv_heads);
-  const dim3 blk(twl::kGemvThreads);
-#define TWL_GEMV_GROUP(DT)                                                                        \
+  // 16 pages per wavefront, 4 in flight (measured at 8 x 8 kv heads x 512 pages: 16 / 4 12.1 us,
+  // 8 / 4 12.3, 16 / 8 12.3, 8 / 8 12.0, 4 / 4 13.9: the launch is about as long as its fixed
+  // phases, launch, page-table and query round trips, the write-out, plus 50 MB at HBM speed)
+#define TWL_GEMV_GROUP2(DT, PW_, U_)                                                              \
   do {                                                                                            \
-    if (group == 2) hipLaunchKernelGGL((twl::gemv_int4_group_kernel<DT, 2, PW>), grid, blk, 0, st, a); \
-    else if (group == 4) hipLaunchKernelGGL((twl::gemv_int4_group_kernel<DT, 4, PW>), grid, blk, 0, st, a); \
-    else hipLaunchKernelGGL((twl::gemv_int4_group_kernel<DT, 8, PW>), grid, blk, 0, st, a);        \
+    const uint32_t per_block = PW_ * (twl::kGemvThreads / twl::kWave);                            \
+    const dim3 grid((max_pages_per_row + per_block - 1) / per_block, batch * num_kv_heads);       \
+    const dim3 blk(twl::kGemvThreads);                                                            \
+    if (group == 2) hipLaunchKernelGGL((twl::gemv_int4_group_kernel<DT, 2, PW_, U_>), grid, blk, 0, st, a); \
+    else if (group == 4) hipLaunchKernelGGL((twl::gemv_int4_group_kernel<DT, 4, PW_, U_>), grid, blk, 0, st, a); \
+    else hipLaunchKernelGGL((twl::gemv_int4_group_kernel<DT, 8, PW_, U_>), grid, blk, 0, st, a);   \
   } while (0)
+#define TWL_GEMV_GROUP(DT) TWL_GEMV_GROUP2(DT, 16, 4)
   if (q_dtype == TWL_F16) TWL_GEMV_GROUP(TWL_F16);
   else TWL_GEMV_GROUP(TWL_BF16);
+#undef TWL_GEMV_GROUP2
 #undef TWL_GEMV_GROUP
   return hipGetLastError() == hipSuccess ? TWL_OK : TWL_ELAUNCH;
 }
