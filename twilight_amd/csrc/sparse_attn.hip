@@ -223,8 +223,10 @@ __device__ __forceinline__ void attn_chunk(const AttnArgs& a, AttnSmem<THREADS>&
   // fold the lane groups (4 per wave) through LDS: every thread adds the groups of its residue
   // class, then the first 128 threads add the classes
   constexpr int kParts = kAttnThreads / TWL_HEAD_DIM;
-#pragma unroll
-  for (int d = 0; d < 8; ++d) oacc[wave * 4 + grp][8 * sub + d] = acc[d];
+  // (two 16-byte stores per lane: the 16 lanes of a token cover 512 contiguous bytes; eight
+  // 4-byte stores at a stride of 32 bytes were 16-way bank conflicts)
+  *(f32x4*)&oacc[wave * 4 + grp][8 * sub] = f32x4{acc[0], acc[1], acc[2], acc[3]};
+  *(f32x4*)&oacc[wave * 4 + grp][8 * sub + 4] = f32x4{acc[4], acc[5], acc[6], acc[7]};
   __syncthreads();
   float o = 0.0f;
   {
