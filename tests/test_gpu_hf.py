@@ -323,3 +323,96 @@ def test_decode_refuses_a_mask_that_hides_positions_and_takes_a_single_first_tok
         assert torch.allclose(got.logits.float(), ref.logits.float(), rtol=1e-3, atol=1e-3)
         step = model2(ids[:, 1:2], past_key_values=got.past_key_values, use_cache=True)
         assert torch.isfinite(step.logits).all()
+
+
+def test_full_size_model_keeping_everything_equals_dense_decode(dev):
+    """The whole model at the benchmark's shape (Llama-3-8B: 32 layers, 32 q heads on 8 kv heads,
+    head_dim 128, bf16, random weights) over a 32704-token context: with p = 1 and a budget that
+    holds every page the patched model (paged caches filled from given K / V, layers 0-1 through the
+    dense paged attention, layers 2-31 through select -> estimate -> prune -> attention over all
+    32704 + step tokens, RoPE, append) must reproduce the model's own dense decode. Size-dependent
+    parts are exercised here: 2044-page tables, 32736-candidate rows, split attention rows of 256
+    chunks, appends that cross a page boundary."""
+    from transformers import DynamicCache, LlamaConfig, LlamaForCausalLM
+    B, N, nl, steps = 1, 32704, 32, 3
+    cfg = LlamaConfig(vocab_size=128256, hidden_size=4096, intermediate_size=14336,
+                      num_hidden_layers=nl, num_attention_heads=32, num_key_value_heads=8,
+                      head_dim=128, max_position_embeddings=N + 4096, rope_theta=500000.0,
+                      attn_implementation="sdpa")
+    torch.manual_seed(0)
+    old = torch.get_default_dtype()
+    torch.set_default_dtype(torch.bfloat16)
+    try:
+        with torch.device(dev):
+            model = LlamaForCausalLM(cfg).eval()
+    finally:
+        torch.set_default_dtype(old)
+
+    def kv(layer):
+        g = torch.Generator(device=dev).manual_seed(1000 + layer)
+        k = torch.randn((B, 8, N, 128), generator=g, device=dev, dtype=torch.bfloat16)
+        v = torch.randn((B, 8, N, 128), generator=g, device=dev, dtype=torch.bfloat16)
+        return k, v
+
+    ids = torch.randint(0, cfg.vocab_size, (steps, B, 1), generator=torch.Generator().manual_seed(7)).to(dev)
+
+    def run(cache, m=None):
+        out = []
+        with torch.no_grad():
+            for s in range(steps):
+                o = (m or model)(ids[s], past_key_values=cache, use_cache=True,
+                                 position_ids=torch.full((B, 1), N + s, device=dev))
+                out.append(o.logits[:, -1].float())
+        return torch.stack(out)
+
+    # the yardstick: the same weights and K / V in fp32 (eager attention), against which both
+    # bf16 runs are measured; then the model's own bf16 dense decode
+    import copy
+    model32 = copy.deepcopy(model).float()
+    model32.config._attn_implementation = "eager"
+    cache = DynamicCache(config=cfg)
+    for i in range(nl):
+        k, v = kv(i)
+        cache.update(k.float(), v.float(), i)
+    exact = run(cache, model32)
+    del cache, model32
+    torch.cuda.empty_cache()
+    cache = DynamicCache(config=cfg)
+    for i in range(nl):
+        cache.update(*kv(i), i)
+    ref = run(cache)
+    del cache
+    torch.cuda.empty_cache()
+    sparse_cfg = json.loads(json.dumps(CFG))
+    sparse_cfg["selector"]["token_budget"] = 32768
+    sparse_cfg["weight_pruner"]["threshold"] = 1.0
+    info, _ = hf.enable_sparse_attention(model, sparse_cfg, enable_budget_info=True, reserve_tokens=16,
+                                         keep_hf_cache=False, dense_layers="paged")
+    for i in range(nl):
+        hf.fill_from_prefill(model.model.layers[i].self_attn._twilight_state, *kv(i), cfg.num_attention_heads)
+    got = run(DynamicCache(config=cfg))
+    hf.disable_sparse_attention(model)
+    assert torch.isfinite(got).all()
+    # every token is kept in every pruned layer
+    first = info._budget_num[0]
+    assert sorted(first) == list(range(2, nl))
+    assert all(int(first[l].min()) >= N for l in first)
+    # both bf16 runs against the fp32 one: the patched model may not be further from it than the
+    # model's own bf16 decode is (plus a fifth), and the two agree with each other
+    err_got = (got - exact).abs().max().item()
+    err_ref = (ref - exact).abs().max().item()
+    rms_got = (got - exact).pow(2).mean().sqrt().item()
+    rms_ref = (ref - exact).pow(2).mean().sqrt().item()
+    scale = exact.abs().max().item()
+    cosf = torch.nn.functional.cosine_similarity
+    cos_got = float(cosf(got.flatten(1), exact.flatten(1), dim=1).min())
+    cos_ref = float(cosf(ref.flatten(1), exact.flatten(1), dim=1).min())
+    rms_between = (got - ref).pow(2).mean().sqrt().item()
+    print(f"full-size model vs fp32: patched max {err_got:.4f} rms {rms_got:.5f} cosine {cos_got:.6f}; "
+          f"bf16 dense max {err_ref:.4f} rms {rms_ref:.5f} cosine {cos_ref:.6f}; max |logit| "
+          f"{scale:.3f}; patched vs bf16 dense rms {rms_between:.5f}")
+    # (measured: rms 0.0556 against 0.0543, cosine 0.99899 against 0.99904 at max |logit| 5.7:
+    # the distance to fp32 is the bf16 arithmetic of the model around the attention)
+    assert rms_got <= 1.2 * rms_ref and err_got <= 1.5 * err_ref
+    assert cos_got >= cos_ref - 5e-4 and cos_got > 0.995
+    assert rms_between <= 2.0 * rms_ref
