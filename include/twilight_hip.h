@@ -103,7 +103,11 @@ int twl_device_count(void);
  *   idx   int32 [rows, idx_stride] + count int32 [rows]: the positions where mask is 1, ascending.
  * low_out (nullable) float [rows]: the final lower pivot; iters_out (nullable) int32 [rows]: the
  * number of bisection iterations executed.
- * d must be in [1, TWL_MAX_CANDIDATES]; idx_stride >= d when idx is given.
+ * d must be in [1, TWL_MAX_CANDIDATES]; idx_stride >= d when idx is given. p is not range-checked,
+ * as in the reference (only NaN is refused): p >= 1 lets no sum reach it, the search ends with
+ * low = 0 and every positive probability is kept; p <= 0 is reached by every sum. The entry
+ * points that are not the reference's (twl_softmax_top_p_f32, twl_gemv_top_p,
+ * twl_select_estimate_prune, twl_decode_layer) require 0 < p <= 1.
  * ------------------------------------------------------------------------------------------- */
 int twl_top_p_f32(const float* probs, uint8_t* mask, int32_t* idx, int32_t* count,
                   const float* p_arr, float p, uint32_t rows, uint32_t d, uint32_t idx_stride,

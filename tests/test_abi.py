@@ -62,8 +62,9 @@ def test_c_level_validation_without_gpu(hip_lib):
     assert L.twl_top_p_f32(fake, 0, fake, 0, 0, 0.9, 1, 8, 8, 0, 0, 0, 0) == -1       # idx without count
     assert L.twl_top_p_f32(fake, fake, 0, 0, 0, 0.9, 1, 0, 8, 0, 0, 0, 0) == -2       # d == 0
     assert L.twl_top_p_f32(fake, fake, 0, 0, 0, 0.9, 1, 40000, 8, 0, 0, 0, 0) == -2   # d too large
-    assert L.twl_top_p_f32(fake, fake, 0, 0, 0, 0.0, 1, 8, 8, 0, 0, 0, 0) == -2       # p out of (0,1]
-    assert L.twl_top_p_f32(fake, fake, 0, 0, 0, 1.5, 1, 8, 8, 0, 0, 0, 0) == -2
+    assert L.twl_top_p_f32(fake, fake, 0, 0, 0, float("nan"), 1, 8, 8, 0, 0, 0, 0) == -2   # p NaN
+    assert L.twl_softmax_top_p_f32(fake, 8, 0, 1, 8, 0, 0.0, 1, 0, 0, fake, 8, fake, 0, 0, 0) == -2   # p out of (0,1]
+    assert L.twl_softmax_top_p_f32(fake, 8, 0, 1, 8, 0, 1.5, 1, 0, 0, fake, 8, fake, 0, 0, 0) == -2
     assert L.twl_top_p_f32(fake, fake, 0, 0, 0, 0.9, 1, 8, 8, 7, 0, 0, 0) == -2       # bad high_mode
     assert L.twl_top_p_f32(fake, 0, fake, fake, 0, 0.9, 1, 8, 4, 0, 0, 0, 0) == -2    # idx_stride < d
     assert L.twl_top_p_f32(fake + 2, fake, 0, 0, 0, 0.9, 1, 8, 8, 0, 0, 0, 0) == -4   # misaligned

@@ -333,6 +333,42 @@ def test_errors(dev):
     with pytest.raises(RuntimeError):
         K.top_p_fp32_return_mask(p.half(), 0.9)               # wrong dtype for the fp32 entry
     with pytest.raises(RuntimeError):
-        K.top_p_fp32_return_mask(p, 1.5)
+        K.top_p_fp32_return_mask(p, float("nan"))
+    with pytest.raises(RuntimeError):
+        K.softmax_top_p(p[:, :, 0].contiguous(), 1.5)         # not one of the reference's ops: 0 < p <= 1
     with pytest.raises(RuntimeError):
         K.top_p_fp32_return_mask(p, torch.rand(5, device=dev))
+
+
+@pytest.mark.parametrize("exact", [False, True])
+def test_reference_takes_any_p_and_any_qo_len(dev, exact):
+    """What csrc/src/sampling.cu:22-63 does with arguments it does not check, reproduced by the
+    drop-in ops: a scalar p outside (0, 1] (p >= 1: no sum reaches it, low stays 0, every positive
+    probability is kept; p <= 0: every sum reaches it) and qo_len != 1 (dim 2 is ignored: the
+    first batch * heads rows of the buffer are processed, the rest of the mask stays False)."""
+    g = torch.Generator().manual_seed(12)
+    probs = _softmax(torch.randn((2, 3, 1, 700), generator=g) * 3.0)
+    probs[0, 1, 0, 5:9] = 0.0
+    pn = probs.numpy().reshape(6, 700)
+    for p in (1.5, 1.0, 0.0, -0.25):
+        for high, mode in (("first", native.HIGH_FIRST), ("max", native.HIGH_MAX)):
+            om, ol, oi = native.top_p_mask_f32(pn, p, mode)
+            idx, count, mask, low, iters = K.top_p_select(probs.to(dev), p, high=high, return_mask=True,
+                                                          return_stats=True, exact=exact)
+            assert np.array_equal(mask.cpu().numpy().reshape(6, 700), om.astype(bool)), (p, high)
+            if not exact:
+                assert np.array_equal(low.cpu().numpy(), ol) and np.array_equal(iters.cpu().numpy(), oi)
+            if p > 1:
+                assert np.array_equal(om.astype(bool), pn > 0)
+        for dt, code in ((torch.float16, 0), (torch.bfloat16, 1)):
+            bits = probs.to(dt).view(torch.int16).numpy().view(np.uint16).reshape(6, 700)
+            om16 = native.top_p_mask_cub(bits, code, p, native.HIGH_FIRST)[0]
+            got = K.top_p_fp16_return_mask(probs.to(dt).to(dev), p).cpu().numpy().reshape(6, 700)
+            assert np.array_equal(got, om16.astype(bool)), (p, dt)
+    # qo_len = 3: rows 0..5 of the flattened [18, 700] buffer are the kernel's six rows
+    wide = _softmax(torch.randn((2, 3, 3, 700), generator=g) * 3.0)
+    om = native.top_p_mask_f32(wide.numpy().reshape(18, 700)[:6], 0.9, native.HIGH_FIRST)[0]
+    got = K.top_p_fp32_return_mask(wide.to(dev), 0.9, exact=exact).cpu().numpy().reshape(18, 700)
+    assert np.array_equal(got[:6], om.astype(bool)) and not got[6:].any()
+    with pytest.raises(RuntimeError):
+        K.top_p_select(wide.to(dev), 0.9)                     # the list form is decode-only

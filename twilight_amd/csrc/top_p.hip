@@ -210,16 +210,19 @@ static int launch_top_p(const TopPArgs& a, uint32_t rows, hipStream_t s) {
 
 using twl::TopPArgs;
 
+// `any_p`: the drop-in mask entries take whatever p the reference takes (csrc/src/sampling.cu:22-63
+// checks nothing: p >= 1 makes every comparison S >= p fail, so the search ends with low = 0 and
+// every positive probability kept; p <= 0 makes every one succeed); only NaN is refused.
 static int check_top_p_common(const void* in, uint8_t* mask, int32_t* idx, int32_t* count,
                               float p, const float* p_arr, uint32_t rows, uint32_t d,
-                              uint32_t idx_stride, int high_mode) {
+                              uint32_t idx_stride, int high_mode, bool any_p = false) {
   if (!in) return TWL_ENULL;
   if (!mask && !idx && !count) return TWL_ENULL;
   if (idx && !count) return TWL_ENULL;
   if (rows == 0 || d == 0 || d > TWL_MAX_CANDIDATES) return TWL_EINVAL;
   if (idx && idx_stride < d) return TWL_EINVAL;
   if (high_mode != TWL_HIGH_FIRST && high_mode != TWL_HIGH_MAX) return TWL_EINVAL;
-  if (!p_arr && !(p > 0.0f && p <= 1.0f)) return TWL_EINVAL;
+  if (!p_arr && (any_p ? (p != p) : !(p > 0.0f && p <= 1.0f))) return TWL_EINVAL;
   return TWL_OK;
 }
 
@@ -227,7 +230,8 @@ extern "C" int twl_top_p_f32(const float* probs, uint8_t* mask, int32_t* idx, in
                              const float* p_arr, float p, uint32_t rows, uint32_t d,
                              uint32_t idx_stride, int high_mode, float* low_out,
                              int32_t* iters_out, void* stream) {
-  int rc = check_top_p_common(probs, mask, idx, count, p, p_arr, rows, d, idx_stride, high_mode);
+  int rc = check_top_p_common(probs, mask, idx, count, p, p_arr, rows, d, idx_stride, high_mode,
+                              true);
   if (rc != TWL_OK) return rc;
   if (((uintptr_t)probs) & 3u) return TWL_EALIGN;
   TopPArgs a{};

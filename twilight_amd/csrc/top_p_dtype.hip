@@ -311,7 +311,7 @@ static int check_top_p_dtype(const void* probs, const uint8_t* mask, const int32
   if (rows == 0 || d == 0 || d > TWL_MAX_CANDIDATES) return TWL_EINVAL;
   if (idx && idx_stride < d) return TWL_EINVAL;
   if (high_mode != TWL_HIGH_FIRST && high_mode != TWL_HIGH_MAX) return TWL_EINVAL;
-  if (!p_arr && !(p > 0.0f && p <= 1.0f)) return TWL_EINVAL;
+  if (!p_arr && p != p) return TWL_EINVAL;   // any p the reference takes; see twl_top_p_f32
   return TWL_OK;
 }
 

@@ -31,13 +31,14 @@ def _to_tensor_scalar_tuple(x):
     return (None, float(x))
 
 
-def _check_probs(probs: torch.Tensor) -> Tuple[int, int]:
+def _check_probs(probs: torch.Tensor, lists: bool = False) -> Tuple[int, int]:
     check_input(probs, "probs")          # csrc/src/sampling.cu:25,48
     check_dim(4, probs, "probs")         # csrc/src/sampling.cu:27,50 (batch, heads, qo_len, kv_len)
-    if probs.size(2) != 1:
-        # the reference silently ignores dim 2 (csrc/src/sampling.cu:51-60), which is only
-        # meaningful for decode (qo_len == 1)
+    if lists and probs.size(2) != 1:
         raise RuntimeError("probs must have qo_len == 1 (shape [batch, heads, 1, kv_len])")
+    # The mask ops do what csrc/src/sampling.cu:51-60 does with qo_len != 1: dim 2 is ignored, the
+    # kernel gets batch * heads rows of kv_len, i.e. the FIRST batch * heads rows of the contiguous
+    # buffer, and the rest of the mask stays False. Only decode (qo_len == 1) is meaningful.
     rows, d = probs.size(0) * probs.size(1), probs.size(3)
     if rows == 0 or d == 0:
         raise RuntimeError("probs must not be empty")
@@ -46,7 +47,9 @@ def _check_probs(probs: torch.Tensor) -> Tuple[int, int]:
     return rows, d
 
 
-def _check_p(top_p, rows: int, ref: torch.Tensor):
+def _check_p(top_p, rows: int, ref: torch.Tensor, any_p: bool = False):
+    """``any_p``: the reference's ops do not look at the value of a scalar ``top_p``
+    (kernel/cuda/sampling.py:111-133); the drop-in ops follow (only NaN raises)."""
     p_arr, p_val = _to_tensor_scalar_tuple(top_p)
     if p_arr is not None:
         check_input(p_arr, "top_p")
@@ -54,14 +57,14 @@ def _check_p(top_p, rows: int, ref: torch.Tensor):
         check_same_device(ref, ("top_p", p_arr))
         if p_arr.numel() != rows:
             raise RuntimeError(f"top_p tensor must have batch*heads = {rows} elements")
-    elif not (0.0 < p_val <= 1.0):
+    elif p_val != p_val or (not any_p and not (0.0 < p_val <= 1.0)):
         raise RuntimeError(f"top_p must be in (0, 1], got {p_val}")
     return p_arr, p_val
 
 
 def _run_top_p(probs, top_p, high, want_mask, want_idx, want_stats=False, exact=False):
-    rows, d = _check_probs(probs)
-    p_arr, p_val = _check_p(top_p, rows, probs)
+    rows, d = _check_probs(probs, lists=want_idx)
+    p_arr, p_val = _check_p(top_p, rows, probs, any_p=True)
     mode = _high_mode(high)
     dev = probs.device
     with torch.cuda.device(dev):
