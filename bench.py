@@ -7,16 +7,21 @@ prune -> sparse paged attention) over one batch of synthetic decode queries, enq
 
 Workload (``config.workload``): the Longchat-7B-shaped layer of the reference's headline figure at
 the batch the target is quoted on — 32 MHA heads, head_dim 128, fp16 paged KV (page 16), batch 8,
-context 32768, Quest budget 8192, top-p 0.95.
+context 32768, Quest budget 8192, top-p 0.95. q, K, V ~ N(0,1) with planted heavy-hitter pages whose
+strength is solved per row so that the pruner keeps 100-400 tokens per row (``--planted
+calibrated``, the default; ``--planted peaked`` is one fixed strength, under which most rows keep
+1-2 tokens and a few keep thousands).
 
 Prints ONE JSON line. ``value`` is microseconds per layer (lower is better). ``roofline`` is for
-the kernel with the largest HBM term (the Quest metadata stream); ``kernels`` lists every kernel of
-the layer with its algorithmic bytes, time and fraction of the 8 TB/s peak, and ``gemv_cfg2`` the
-stand-alone INT4 GEMV at 8 x 32 x 32768 candidates. ``cfg4_b16`` (the same layer at batch 16) and
-``cfg5_layer`` (32 q heads on 8 kv heads, bf16, p 0.9, with the dense paged decode beside it) are
-the other two layer shapes of the headline figure, measured the same way with fewer steps, and
-``cfg5_model`` is the whole 32-layer model at that shape (random weights, tokens/s, 8 decode steps
-replayed from one HIP graph, against the model's own dense decode).
+the step's dominant kernel (the one-launch selector + estimator + pruner); ``kernels`` lists every
+kernel of the layer with its algorithmic bytes, time and fraction of the 8 TB/s peak, and
+``gemv_cfg2`` the stand-alone INT4 GEMV at 8 x 32 x 32768 candidates. ``b8_peaked`` is the same
+layer on the other planted workload, ``cfg4_b16`` / ``cfg4_b32`` / ``cfg4_b64`` the same layer at
+the other batch sizes of the reference's latency figure and ``cfg5_layer`` the Llama-3 shape (32 q
+heads on 8 kv heads, bf16, p 0.9, with the dense paged decode and the one-list-per-kv-head option
+beside it), all measured the same way with fewer steps; ``cfg5_model`` is the whole 32-layer model
+at that shape (random weights, tokens/s, 8 decode steps replayed from one HIP graph, against the
+model's own dense decode).
 ``cpu_baseline`` is the CPU oracle (a port of the reference's torch path) timed on this host on
 one of the 8 batch elements and scaled by 8, plus the reference's own CPU case (B=1, context 4096)
 with warm-ups, repeats, median and per-stage times.
@@ -51,7 +56,8 @@ HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 QUEST_SCORE_TRAFFIC_BYTES_DEFAULT = int((131404.9 * 2.000 + 2048.0 * 1.000) * 1024)
 # The same for select_estimate_prune_kernel (FETCH_SIZE KiB x 2.000 + WRITE_SIZE KiB x 1.000).
 ROW_KERNEL_TRAFFIC_BYTES_RECORDS = int((213640.2 * 2.000 + 596.1 * 1.000) * 1024)  # --no-planes
-ROW_KERNEL_TRAFFIC_BYTES_DEFAULT = int((148094.6 * 2.000 + 596.1 * 1.000) * 1024)  # plane layout
+ROW_KERNEL_TRAFFIC_BYTES_DEFAULT = int((148074.2 * 2.000 + 775.4 * 1.000) * 1024)  # plane layout, calibrated
+ROW_KERNEL_TRAFFIC_BYTES_PEAKED = int((148094.6 * 2.000 + 596.1 * 1.000) * 1024)   # plane layout, peaked
 
 
 def _time_calls(fn, iters: int, warmup: int) -> float:
@@ -900,7 +906,8 @@ def main() -> int:
             elif dom_name == "quest_score_planes":
                 traffic = None  # not measured for this kernel
             elif layers[0].cache.meta_planes is not None:
-                traffic = ROW_KERNEL_TRAFFIC_BYTES_DEFAULT
+                traffic = (ROW_KERNEL_TRAFFIC_BYTES_DEFAULT if survivors is not None
+                           else ROW_KERNEL_TRAFFIC_BYTES_PEAKED)
             else:
                 traffic = ROW_KERNEL_TRAFFIC_BYTES_RECORDS
         roofline = {"bound": "hbm",
