@@ -17,17 +17,18 @@
 //     CUB, and lane 0 of a row only ever needs lanes of its own row, so the lanes whose shifted
 //     source falls outside the row may hold anything;
 //   - the 32 warp results go through LDS and are added one after the other, warp 0 first, as
-//     CUB's thread 0 does; every thread here repeats that chain so no second barrier is needed;
+//     CUB's thread 0 does, by one wavefront per chunk;
 //   - the block sums of successive chunks are added to the running sum in chunk order
 //     (sampling.cuh:191-193).
-// Minima, maxima and comparisons are exact in any order. The row is read from HBM once and kept
-// in registers (at most 32 values per thread); an iteration costs one barrier.
+// Minima, maxima and comparisons are exact in any order, so they are made on bit patterns with
+// integer instructions. The row is read from HBM once and kept in registers (at most 32 values
+// per thread); an iteration costs two barriers.
 //
-// A 16-bit addition is computed as an fp32 addition rounded to the 16-bit type: fp32 carries
-// 24 >= 2 * 11 + 2 significand bits, so the double rounding equals the single one. For float the
-// rounding step is the identity and what remains is the order of the additions, which is what
-// makes the float op reproduce the reference's masks row for row (the faster fp32 kernel of
-// top_p.hip adds in another order and can differ where a sum meets p within rounding).
+// A binary16 addition is the hardware's; a bfloat16 addition is an fp32 addition rounded to
+// bfloat16 (fp32 carries 24 >= 2 * 8 + 2 significand bits, so the double rounding equals the
+// single one). For float what remains is the order of the additions, which is what makes the
+// float op reproduce the reference's masks row for row (the faster fp32 kernel of top_p.hip adds
+// in another order and can differ where a sum meets p within rounding).
 #include "twl_common.h"
 
 namespace twl {
@@ -53,17 +54,68 @@ constexpr int kCubMaxVals = TWL_MAX_CANDIDATES / kCubThreads;  // 32 values per 
 
 constexpr int kDppRowShl1 = 0x101, kDppRowShl2 = 0x102, kDppRowShl4 = 0x104, kDppRowShl8 = 0x108;
 
+// The arithmetic of one element type. The kernel carries a probability as its key: the bit
+// pattern of the value in its own type for binary16 (16 bits, zero-extended), the bit pattern of
+// the equal float for bfloat16 and float. Keys of non-negative numbers order like the numbers, so
+// comparisons and the minimum / maximum searches are integer operations; additions are made in
+// T, where `add` rounds to the element type: natively for binary16 and float, as a float
+// addition rounded to bfloat16 otherwise (24 >= 2 * 8 + 2 significand bits: the double rounding
+// equals the single one). `box` / `unbox` carry a T through a 32-bit register or LDS word.
 template <int DT>
-__device__ __forceinline__ float dt_add(float a, float b) {
-  return round_to<DT>(a + b);
+struct DtNum {   // float and bfloat16
+  using T = float;
+  static constexpr uint32_t kInfKey = 0x7F800000u;
+  static __device__ __forceinline__ uint32_t key(float f) { return as_u32(f); }
+  static __device__ __forceinline__ float keyf(uint32_t k) { return as_f32(k); }
+  static __device__ __forceinline__ T unbox(uint32_t k) { return as_f32(k); }
+  static __device__ __forceinline__ uint32_t box(T v) { return as_u32(v); }
+  static __device__ __forceinline__ T add(T a, T b) { return round_to<DT>(a + b); }
+  static __device__ __forceinline__ float f32(T v) { return v; }
+};
+template <>
+struct DtNum<TWL_F16> {
+  using T = _Float16;
+  static constexpr uint32_t kInfKey = 0x7C00u;
+  static __device__ __forceinline__ uint32_t key(float f) { return f32_to_f16_bits(f); }
+  static __device__ __forceinline__ float keyf(uint32_t k) { return f16_bits_to_f32(k); }
+  static __device__ __forceinline__ T unbox(uint32_t k) {
+    return __builtin_bit_cast(_Float16, (uint16_t)k);
+  }
+  static __device__ __forceinline__ uint32_t box(T v) {
+    return (uint32_t)__builtin_bit_cast(uint16_t, v);
+  }
+  static __device__ __forceinline__ T add(T a, T b) { return a + b; }
+  static __device__ __forceinline__ float f32(T v) { return (float)v; }
+};
+
+__device__ __forceinline__ uint32_t wave_min_u32_to_lane63(uint32_t v) {
+  v = min(v, (uint32_t)dpp<kDppXor1>((int)0xFFFFFFFF, (int)v));
+  v = min(v, (uint32_t)dpp<kDppXor2>((int)0xFFFFFFFF, (int)v));
+  v = min(v, (uint32_t)dpp<kDppHalfMirror>((int)0xFFFFFFFF, (int)v));
+  v = min(v, (uint32_t)dpp<kDppMirror>((int)0xFFFFFFFF, (int)v));
+  v = min(v, (uint32_t)dpp<kDppBcast15, 0xA>((int)0xFFFFFFFF, (int)v));
+  v = min(v, (uint32_t)dpp<kDppBcast31, 0xC>((int)0xFFFFFFFF, (int)v));
+  return v;
+}
+// the smallest of the 16 per-wavefront keys in `slots`, in every lane
+__device__ __forceinline__ uint32_t fold16_min_u32(const uint32_t* slots, int lane) {
+  uint32_t t = slots[lane & (kCubWaves - 1)];
+  t = min(t, (uint32_t)dpp<kDppXor1>((int)0xFFFFFFFF, (int)t));
+  t = min(t, (uint32_t)dpp<kDppXor2>((int)0xFFFFFFFF, (int)t));
+  t = min(t, (uint32_t)dpp<kDppHalfMirror>((int)0xFFFFFFFF, (int)t));
+  t = min(t, (uint32_t)dpp<kDppMirror>((int)0xFFFFFFFF, (int)t));
+  return (uint32_t)__builtin_amdgcn_readfirstlane((int)t);
 }
 
 template <int DT, int VEC>
 __global__ __launch_bounds__(kCubThreads) void top_p_dtype_kernel(TopPDtArgs a) {
+  using N = DtNum<DT>;
+  using T = typename N::T;
   constexpr int MAXC = kCubMaxVals / VEC;
-  __shared__ float wagg[2][MAXC][kCubWarps];
-  __shared__ float wmin[2][kCubWaves], wmax[2][kCubWaves];
-  __shared__ float first_val;
+  __shared__ __align__(16) uint32_t wagg[MAXC][kCubWarps];   // warp aggregates of a chunk, boxed
+  __shared__ uint32_t cagg[MAXC];                            // block aggregate of a chunk, boxed
+  __shared__ uint32_t wkey[kCubWaves], wkey0[kCubWaves];
+  __shared__ uint32_t first_key;
   __shared__ int chunk_tot[MAXC][kCubWaves];
 
   const uint32_t row = blockIdx.x;
@@ -77,7 +129,7 @@ __global__ __launch_bounds__(kCubThreads) void top_p_dtype_kernel(TopPDtArgs a) 
   constexpr uint32_t ESZ = (DT == TWL_F32) ? 4u : 2u;
   const uint8_t* src = (const uint8_t*)a.probs + (size_t)row * d * ESZ;
   const bool vec_ok = ((((uintptr_t)src) & (ESZ * VEC - 1u)) == 0);
-  float x[MAXC][VEC];
+  uint32_t xk[MAXC][VEC];
   bool valid[MAXC];
 #pragma unroll
   for (int c = 0; c < MAXC; ++c) {
@@ -121,97 +173,133 @@ __global__ __launch_bounds__(kCubThreads) void top_p_dtype_kernel(TopPDtArgs a) 
     }
 #pragma unroll
     for (int j = 0; j < VEC; ++j)
-      x[c][j] = (raw[j] > 0.0f) ? raw[j] : 0.0f;   // probabilities; negative, -0 and NaN count as 0
+      xk[c][j] = (raw[j] > 0.0f) ? N::key(raw[j]) : 0u;   // negative, -0 and NaN count as 0
   }
 
   // ---- bounds (sampling.cuh:156-162) ----------------------------------------------------------
+  // A = min{x > low} and B = max{x <= high} as keys, without the reference's caps (it starts the
+  // two searches from `high` and `low`, sampling.cuh:174-175; the caps are applied where the
+  // values are used). One search pattern serves both:
+  //   k = x - c   (c = key(low) + 1)   smallest k -> A = c + k
+  //   k = c - x   (c = key(high))      smallest k -> B = c - k
+  // in wrapping unsigned arithmetic, where elements on the wrong side of the bound wrap to
+  // k >= 2^31. A only moves when `low` moves and B only when `high` moves, so an iteration runs
+  // the search for whichever bound the iteration before it changed. Zeros past the end of the
+  // row never enter either result: they are not above `low`, and a B of 0 is capped by `low`.
   const float p = round_to<DT>(a.p_arr ? a.p_arr[row] : a.p);
   const float eps = round_to<DT>(1e-5f);
   float low = 0.0f, high;
+  uint32_t A_key = N::kInfKey, B_key = 0u;
+  auto min_search = [&](uint32_t c, bool below) -> uint32_t {   // `below` is uniform
+    uint32_t kmin = 0xFFFFFFFFu;
+    if (__builtin_amdgcn_readfirstlane((int)below)) {
+#pragma unroll
+      for (int cc = 0; cc < MAXC; ++cc)
+        if (cc < nchunks) {
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) kmin = min(kmin, c - xk[cc][j]);
+        }
+    } else {
+#pragma unroll
+      for (int cc = 0; cc < MAXC; ++cc)
+        if (cc < nchunks) {
+#pragma unroll
+          for (int j = 0; j < VEC; ++j) kmin = min(kmin, xk[cc][j] - c);
+        }
+    }
+    return wave_min_u32_to_lane63(kmin);
+  };
   if (a.high_mode == TWL_HIGH_FIRST) {
-    if (tx == 0) first_val = x[0][0];
+    if (tx == 0) first_key = xk[0][0];
     __syncthreads();
-    high = first_val;
+    const uint32_t c = first_key;
+    high = N::keyf(c);
+    const uint32_t k = min_search(c, true);
+    if (lane == kWave - 1) wkey0[wave] = k;
+    __syncthreads();
+    const uint32_t kk = fold16_min_u32(wkey0, lane);
+    B_key = (kk < 0x80000000u) ? c - kk : 0u;
   } else {
-    float m = 0.0f;
-#pragma unroll
-    for (int c = 0; c < MAXC; ++c)
-#pragma unroll
-      for (int j = 0; j < VEC; ++j) m = fmaxf(m, x[c][j]);
-    m = wave_allreduce<OpMax>(m);
-    if (lane == 0) wmax[1][wave] = m;
+    // the row's maximum: the largest key below infinity's successor
+    const uint32_t c = N::kInfKey;
+    const uint32_t k = min_search(c, true);
+    if (lane == kWave - 1) wkey0[wave] = k;
     __syncthreads();
-    high = 0.0f;
-#pragma unroll
-    for (int w = 0; w < kCubWaves; ++w) high = fmaxf(high, wmax[1][w]);
-    // the loop's first iteration writes buffer 0; buffer 1 is written again only after the
-    // barrier of that iteration, which every wave reaches after these reads
+    const uint32_t kk = fold16_min_u32(wkey0, lane);
+    B_key = (kk < 0x80000000u) ? c - kk : 0u;
+    high = N::keyf(B_key);
   }
 
   // ---- bisection (sampling.cuh:171-217) -------------------------------------------------------
-  int iters = 0, buf = 0;
+  // Two barriers per iteration: warp aggregates and the wavefronts' search keys meet in LDS at the
+  // first; then ONE wavefront per chunk adds the chunk's 32 warp aggregates one after the other,
+  // warp 0 first (CUB's thread 0), while every wavefront folds the keys; the chunk aggregates
+  // meet at the second.
+  int iters = 0;
+  bool sel_a = true;
   bool more;
   do {
     const float mid = round_to<DT>(round_to<DT>(low + high) * 0.5f);   // :173
-    float mn = high, mx = low;                                          // :174-175
+    const uint32_t midk = N::key(mid);
 #pragma unroll
     for (int c = 0; c < MAXC; ++c) {
       if (c < nchunks) {
-        float acc = 0.0f;
+        T acc = N::unbox(0u);
 #pragma unroll
         for (int j = 0; j < VEC; ++j) {
-          const float v = x[c][j];
-          const float g = (v > mid) ? v : 0.0f;                         // :183
-          acc = (j == 0) ? g : dt_add<DT>(acc, g);                      // cub::ThreadReduce
-          if (valid[c]) {
-            if (v > low) mn = fminf(mn, v);                             // :184-186
-            if (v <= high) mx = fmaxf(mx, v);                           // :187-189
-          }
+          const T g = N::unbox((xk[c][j] > midk) ? xk[c][j] : 0u);     // :183
+          acc = (j == 0) ? g : N::add(acc, g);                          // cub::ThreadReduce
         }
         // a CUDA warp's shuffle-down tree, as far as its lane 0 sees it
-        acc = dt_add<DT>(acc, dpp<kDppRowShl1>(0.0f, acc));
-        acc = dt_add<DT>(acc, dpp<kDppRowShl2>(0.0f, acc));
-        acc = dt_add<DT>(acc, dpp<kDppRowShl4>(0.0f, acc));
-        acc = dt_add<DT>(acc, dpp<kDppRowShl8>(0.0f, acc));
-        const float r0 = as_f32(__builtin_amdgcn_readlane(as_i32(acc), 0));
-        const float r1 = as_f32(__builtin_amdgcn_readlane(as_i32(acc), 16));
-        const float r2 = as_f32(__builtin_amdgcn_readlane(as_i32(acc), 32));
-        const float r3 = as_f32(__builtin_amdgcn_readlane(as_i32(acc), 48));
+        acc = N::add(acc, N::unbox((uint32_t)dpp<kDppRowShl1>(0, (int)N::box(acc))));
+        acc = N::add(acc, N::unbox((uint32_t)dpp<kDppRowShl2>(0, (int)N::box(acc))));
+        acc = N::add(acc, N::unbox((uint32_t)dpp<kDppRowShl4>(0, (int)N::box(acc))));
+        acc = N::add(acc, N::unbox((uint32_t)dpp<kDppRowShl8>(0, (int)N::box(acc))));
+        const int ab = (int)N::box(acc);
+        const T r0 = N::unbox((uint32_t)__builtin_amdgcn_readlane(ab, 0));
+        const T r1 = N::unbox((uint32_t)__builtin_amdgcn_readlane(ab, 16));
+        const T r2 = N::unbox((uint32_t)__builtin_amdgcn_readlane(ab, 32));
+        const T r3 = N::unbox((uint32_t)__builtin_amdgcn_readlane(ab, 48));
         if (lane == 0) {
-          wagg[buf][c][2 * wave] = dt_add<DT>(r0, r1);
-          wagg[buf][c][2 * wave + 1] = dt_add<DT>(r2, r3);
+          wagg[c][2 * wave] = N::box(N::add(r0, r1));
+          wagg[c][2 * wave + 1] = N::box(N::add(r2, r3));
         }
       }
     }
-    mn = wave_allreduce<OpMin>(mn);
-    mx = wave_allreduce<OpMax>(mx);
-    if (lane == 0) {
-      wmin[buf][wave] = mn;
-      wmax[buf][wave] = mx;
-    }
+    const uint32_t sc = sel_a ? N::key(low) + 1u : N::key(high);        // :184-189
+    const uint32_t wk = min_search(sc, !sel_a);
+    if (lane == kWave - 1) wkey[wave] = wk;
     __syncthreads();
-    float total = 0.0f;                                                 // threadlocal_sum, :172
-    for (int c = 0; c < nchunks; ++c) {
-      float agg = wagg[buf][c][0];                                      // thread 0 of CUB's block
+    for (int c = wave; c < nchunks; c += kCubWaves) {
+      const u32x4* pv = (const u32x4*)&wagg[c][0];
+      uint32_t wv[kCubWarps];
 #pragma unroll
-      for (int w = 1; w < kCubWarps; ++w) agg = dt_add<DT>(agg, wagg[buf][c][w]);
-      total = dt_add<DT>(total, agg);                                   // :191-193
-    }
-    float min_gt_low = high, max_le_high = low;
+      for (int i = 0; i < kCubWarps / 4; ++i) {
+        const u32x4 v = pv[i];
+        wv[4 * i] = v.x; wv[4 * i + 1] = v.y; wv[4 * i + 2] = v.z; wv[4 * i + 3] = v.w;
+      }
+      T agg = N::unbox(wv[0]);
 #pragma unroll
-    for (int w = 0; w < kCubWaves; ++w) {
-      min_gt_low = fminf(min_gt_low, wmin[buf][w]);
-      max_le_high = fmaxf(max_le_high, wmax[buf][w]);
+      for (int w = 1; w < kCubWarps; ++w) agg = N::add(agg, N::unbox(wv[w]));
+      if (lane == 0) cagg[c] = N::box(agg);
     }
-    if (total >= p) {                                                   // :211-216
-      low = mid;
-    } else {
-      high = fminf(mid, max_le_high);
-    }
+    const uint32_t kmin = fold16_min_u32(wkey, lane);
+    __syncthreads();
+    T total = N::unbox(cagg[0]);                                        // threadlocal_sum, :172
+    for (int c = 1; c < nchunks; ++c) total = N::add(total, N::unbox(cagg[c]));   // :191-193
+    const bool found = kmin < 0x80000000u;
+    if (sel_a) A_key = found ? sc + kmin : N::kInfKey;
+    else B_key = found ? sc - kmin : 0u;
+    const float min_gt_low = fminf(high, N::keyf(A_key));               // :174,184-186
+    const float max_le_high = fmaxf(low, N::keyf(B_key));               // :175,187-189
+    const bool accept = N::f32(total) >= p;                             // :211-216
+    low = accept ? mid : low;
+    high = accept ? high : fminf(mid, max_le_high);
+    sel_a = accept;
     ++iters;
     more = round_to<DT>(max_le_high - min_gt_low) > eps && iters < 4096;  // :217
-    buf ^= 1;
   } while (more);
+  const uint32_t lowk = N::key(low);
 
   if (tx == 0) {
     if (a.low_out) a.low_out[row] = low;
@@ -232,12 +320,12 @@ __global__ __launch_bounds__(kCubThreads) void top_p_dtype_kernel(TopPDtArgs a) 
             uint32_t w = 0;
 #pragma unroll
             for (int j = 0; j < 4; ++j)
-              w |= (x[c][(j0 + j) % VEC] > low ? 1u : 0u) << (8 * j);
+              w |= (xk[c][(j0 + j) % VEC] > lowk ? 1u : 0u) << (8 * j);
             *(uint32_t*)(dst + e0 + j0) = w;
           }
         } else {
 #pragma unroll
-          for (int j = 0; j < VEC; ++j) dst[e0 + j] = (x[c][j] > low) ? 1 : 0;
+          for (int j = 0; j < VEC; ++j) dst[e0 + j] = (xk[c][j] > lowk) ? 1 : 0;
         }
       }
     }
@@ -252,7 +340,7 @@ __global__ __launch_bounds__(kCubThreads) void top_p_dtype_kernel(TopPDtArgs a) 
     for (int c = 0; c < MAXC; ++c) {
       keep[c] = 0;
 #pragma unroll
-      for (int j = 0; j < VEC; ++j) keep[c] |= (valid[c] && x[c][j] > low) ? (1u << j) : 0u;
+      for (int j = 0; j < VEC; ++j) keep[c] |= (valid[c] && xk[c][j] > lowk) ? (1u << j) : 0u;
       const int mine = __builtin_popcount(keep[c]);
       const int scan = wave_inclusive_scan(mine);
       excl[c] = scan - mine;
