@@ -253,6 +253,47 @@ def test_fp32_exact_entry(dev):
                                             .astype(bool)).reshape(1, rows, 1, d).to(dev))
 
 
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16, torch.float32])
+def test_exact_entries_on_ties_zeros_and_degenerate_rows(dev, dt):
+    # rows the random tests do not produce, for the three kernels that follow the reference's
+    # arithmetic: values from a tiny set (ties everywhere, so the min{x > low} / max{x <= high}
+    # searches return repeated values and the bracket closes on them), rows that are mostly zero,
+    # one-hot, flat and all-zero rows, a zero in front (the `first` bound is then 0: the loop runs
+    # once and keeps every positive entry). Masks, pivots and iteration counts equal the oracle's.
+    g = torch.Generator().manual_seed(11)
+    code = {torch.float16: 0, torch.bfloat16: 1, torch.float32: native.DT_F32}[dt]
+    for d in (8192, 4100, 999, 64, 7):
+        rows = []
+        levels = torch.tensor([0.0, 1.0, 2.0, 3.0, 8.0, 64.0])
+        for zeros in (0.0, 0.5, 0.97):
+            r = levels[torch.randint(1, 6, (d,), generator=g)]
+            r[torch.rand(d, generator=g) < zeros] = 0.0
+            rows.append(r)
+        one_hot = torch.zeros(d); one_hot[d // 3] = 1.0
+        first_zero = levels[torch.randint(1, 6, (d,), generator=g)].clone(); first_zero[0] = 0.0
+        rows += [one_hot, torch.ones(d), torch.zeros(d), first_zero]
+        x = torch.stack(rows)
+        probs = (x / x.sum(-1, keepdim=True).clamp(min=1.0)).to(dt)   # rounded to the type once
+        n = probs.shape[0]
+        vals = (probs.numpy() if dt == torch.float32
+                else probs.view(torch.int16).numpy().view(np.uint16)).reshape(n, d)
+        for high, mode in (("max", native.HIGH_MAX), ("first", native.HIGH_FIRST)):
+            for p in (0.5, 0.9, 1.0):
+                om, ol, oi = native.top_p_mask_cub(vals, code, p, mode)
+                idx, count, mask, low, iters = K.top_p_select(
+                    probs.reshape(1, n, 1, d).to(dev), p, high=high, return_mask=True,
+                    return_stats=True, exact=True)
+                gm = mask.cpu().numpy().reshape(n, d)
+                assert np.array_equal(gm, om.astype(bool)), (d, high, p)
+                assert np.array_equal(low.cpu().numpy().reshape(-1), ol), (d, high, p)
+                assert np.array_equal(iters.cpu().numpy().reshape(-1), oi), (d, high, p)
+                cn = count.cpu().numpy().reshape(-1)
+                assert np.array_equal(cn, gm.sum(-1))
+        # the zero in front under the reference's bound: one iteration, every positive entry kept
+        om, _, oi = native.top_p_mask_cub(vals[-1:], code, 0.9, native.HIGH_FIRST)
+        assert int(oi[0]) == 1 and np.array_equal(om[0].astype(bool), vals[-1] != 0)
+
+
 @pytest.mark.parametrize("first_is_max", [True, False])
 def test_fp32_exact_entry_cfg3(dev, first_is_max):
     # the pruner workload (8 x 32 rows of 8192 probabilities, Zipf spikes over a normal
