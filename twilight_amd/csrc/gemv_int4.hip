@@ -38,10 +38,10 @@ struct GemvArgs {
 // launch shape, chosen by sweeps over (threads, pages per wave, unroll) at 8 x 32 x 32768 and
 // 8 x 32 x 8192 candidates
 constexpr int kGemvThreads = 256;       // 4 wavefronts
-// pages per wavefront (<= 64: one lane per page id): 64 when the grid fills the chip anyway (long
-// runs, few large store bursts); 16 or 8 for small batches, where a wavefront's groups of four
-// pages are serial memory round trips and the launch needs more wavefronts, not longer ones
-constexpr int kGemvPagesPerWave = 64;
+// pages per wavefront (the PW template argument, <= 64: one lane per page id): 64 when the grid
+// fills the chip anyway (long runs, few large store bursts); 16 or 8 for small batches, where a
+// wavefront's groups of four pages are serial memory round trips and the launch needs more
+// wavefronts, not longer ones
 constexpr int kGemvUnroll = 4;          // pages in flight per wavefront
 
 // 8 nibbles of one dword against 8 q values held as 4 half2 pairs (n0,n4),(n1,n5),(n2,n6),(n3,n7).

@@ -48,7 +48,6 @@ __global__ __launch_bounds__(THREADS) void top_p_kernel(TopPArgs a) {
   constexpr int NWAVES = THREADS / kWave;
   constexpr int CHUNKS = VPT / 4;
   __shared__ float red[2][2][16];
-  __shared__ int wave_tot[16];
 
   const uint32_t row = blockIdx.x;
   const int tx = threadIdx.x;
