@@ -468,6 +468,23 @@ def bench_llama3_model(args, dev, emit: bool = True):
     torch.cuda.synchronize()
     layer_us = sum(a.elapsed_time(b) for a, b in ev) * 1e3 / max(len(ev), 1)
     hf.disable_sparse_attention(model)
+    del cache, states
+    torch.cuda.empty_cache()
+    # one more run: the graph-replayed step with one Quest candidate list per kv head
+    info, _ = hf.enable_sparse_attention(model, sparse_cfg, enable_budget_info=True,
+                                         reserve_tokens=reserve + 16, keep_hf_cache=False,
+                                         dense_layers="paged", group_select=True)
+    for i in range(nl):
+        hf.fill_from_prefill(model.model.layers[i].self_attn._twilight_state, *kv(i),
+                             cfg.num_attention_heads)
+    tg, lg = run_graphed()
+    grp_run = {"what": "enable_sparse_attention(group_select=True): one Quest candidate list per "
+                       "kv head instead of one per q head (not the reference's selection); the "
+                       "step replayed from a HIP graph",
+               "ms_per_step": round(tg * 1e3, 3), "tokens_per_s": round(B / tg, 1),
+               "kept_tokens_per_head_mean": round(info.get_total_avg_budget(), 1),
+               "finite_logits": bool(torch.isfinite(lg).all())}
+    hf.disable_sparse_attention(model)
     line = {
         "metric": "tokens/s, whole-model decode with Twilight applied", "value": round(B / twi_ms * 1e3, 1),
         "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
@@ -491,8 +508,9 @@ def bench_llama3_model(args, dev, emit: bool = True):
         "kept_tokens_per_head_mean": round(kept, 1),
         "twilight_layer_us": round(layer_us, 1),
         "finite_logits": bool(torch.isfinite(logits).all()),
+        "group_select": grp_run,
     }
-    del model, cache, states
+    del model
     torch.cuda.empty_cache()
     if emit:
         print(json.dumps(line))
@@ -1028,7 +1046,7 @@ def main() -> int:
         extra["cfg5_model"] = {k: m[k] for k in ("config", "value", "unit", "ms_per_step", "steps",
                                                  "dense", "speedup_vs_dense",
                                                  "kept_tokens_per_head_mean", "twilight_layer_us",
-                                                 "finite_logits")}
+                                                 "finite_logits", "group_select")}
 
     cpu = None
     if not args.no_cpu_baseline and not llama:

@@ -63,6 +63,35 @@ def test_decode_with_p_one_equals_dense_decode(dev, kv_heads):
     assert torch.allclose(again, ref_logits, rtol=1e-3, atol=1e-3)
 
 
+@pytest.mark.parametrize("kv_heads", [2, 1])
+def test_group_select_through_the_model_patch(dev, kv_heads):
+    """enable_sparse_attention(group_select=True): one Quest list per kv head. With everything
+    kept it is dense decoding; with a real budget the q heads of a kv head share their page list
+    and the step still prunes."""
+    model = _tiny_llama(layers=4, heads=4, kv_heads=kv_heads, dtype=torch.float16).to(dev)
+    ids = torch.randint(0, 97, (2, 200), generator=torch.Generator().manual_seed(6)).to(dev)
+    ref_logits, toks = _decode(model, ids, 6)
+    cfg = json.loads(json.dumps(CFG))
+    cfg["selector"]["token_budget"] = 4096
+    cfg["weight_pruner"]["threshold"] = 1.0
+    hf.enable_sparse_attention(model, cfg, reserve_tokens=64, group_select=True)
+    got = _forced_decode(model, ids, toks)
+    assert torch.allclose(got, ref_logits, rtol=2e-2, atol=2e-2), (got - ref_logits).abs().max()
+    hf.disable_sparse_attention(model)
+    cfg["selector"]["token_budget"] = 64
+    cfg["weight_pruner"]["threshold"] = 0.9
+    info, _ = hf.enable_sparse_attention(model, cfg, enable_budget_info=True, reserve_tokens=64,
+                                         group_select=True)
+    got = _forced_decode(model, ids, toks)
+    assert torch.isfinite(got).all()
+    lay = model.model.layers[2].self_attn._twilight_state.layer
+    assert lay.group_select
+    sel = lay.sel_pages.reshape(2, kv_heads, 4 // kv_heads, -1)
+    assert bool((sel == sel[:, :, :1]).all()) and int(lay.sel_count.max()) == 4
+    assert 0 < info.get_total_avg_budget() <= 64
+    hf.disable_sparse_attention(model)
+
+
 def test_decode_with_estimated_weights_and_sparsity_rate(dev):
     """use_estimated_weights_in_attn and selector.sparsity_rate through the model patch: with
     everything kept the estimator's weights move the logits only by the 4-bit error, and the

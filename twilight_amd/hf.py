@@ -292,7 +292,8 @@ def _twilight_attention_forward(self, hidden_states, position_embeddings=None, a
 def enable_sparse_attention(model, sparse_config: Dict, enable_budget_info: bool = False,
                             enable_score_info: bool = False, reserve_tokens: int = 4096,
                             high: str = "max", keep_hf_cache: bool = True,
-                            dense_layers: str = "model") -> Tuple[Optional[HistoryBudgetInfo],
+                            dense_layers: str = "model",
+                            group_select: bool = False) -> Tuple[Optional[HistoryBudgetInfo],
                                        Optional[HistoryAccumulatedScoreInfo]]:
     """Patch every Llama / Mistral attention module of ``model`` (twilight/pyimpl/attention.py:
     351-418, 481-493). ``sparse_config`` is the reference's JSON template
@@ -307,13 +308,17 @@ def enable_sparse_attention(model, sparse_config: Dict, enable_budget_info: bool
     (K / V read once per kv head). With "paged" and ``keep_hf_cache=False`` nothing updates the
     model's cache at decode time, so the caller passes ``position_ids`` to the model itself. ``enable_score_info`` adds a dense pass over all of K
     to every patched layer's decode step (:func:`kept_attention_mass`): a diagnostic, not for
-    timing runs."""
+    timing runs. ``group_select``: with q heads that share kv heads (GQA), one Quest candidate list
+    per kv head (a page scores the largest of its group's q-head scores) instead of the
+    reference's list per q head (attention.py:124-126 repeats K per q head); top-p and attention
+    stay per q head. Fewer bytes per layer; not the reference's selection."""
     for part in ("compressor",):
         t = sparse_config.get(part, {}).get("type", "none")
         if str(t).lower() not in ("none", ""):
             raise RuntimeError(f"{part} type {t!r} is not supported")
     cfg = parse_sparse_config(sparse_config)
     cfg["high"] = high
+    cfg["group_select"] = bool(group_select)
     skip = 2 if sparse_config.get("skip_first_two_layers", True) else 0
     if dense_layers not in ("model", "paged"):
         raise RuntimeError(f"dense_layers must be 'model' or 'paged', got {dense_layers!r}")
